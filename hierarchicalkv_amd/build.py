@@ -1,0 +1,54 @@
+"""Build step for the native library (libhkv.so) and the CPU oracle.
+
+The library is compiled in-tree with hipcc for gfx950 only; the oracle is the
+test checker under oracle/ and is built with gcc.  Nothing here runs a GPU.
+"""
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(ROOT, "include")
+LIB_PATH = os.path.join(PKG_DIR, "libhkv.so")
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "libhkv_oracle.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    "-Wall",
+    "-Wno-unused-function",
+    # packed fp32 VALU forms are kept out of every kernel in this build
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def build_library(verbose=True):
+    cmd = [HIPCC, *HIP_FLAGS, "-I", INCLUDE, "-I", CSRC,
+           os.path.join(CSRC, "hkv_table.hip"), "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+def build_oracle(verbose=True):
+    cmd = ["make", "-C", ORACLE_DIR, "-B", "libhkv_oracle.so"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return ORACLE_LIB
+
+
+if __name__ == "__main__":
+    what = sys.argv[1:] or ["lib", "oracle"]
+    if "lib" in what:
+        build_library()
+    if "oracle" in what:
+        build_oracle()

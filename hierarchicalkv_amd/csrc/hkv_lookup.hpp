@@ -1,0 +1,204 @@
+/*
+ * Read-only lookups: find (value copy), find* (row pointer), contains, and
+ * the missed-keys variant of find.  One 64-lane wavefront per workgroup,
+ * 64 keys per wavefront.
+ *
+ * Replaces lookup_kernel_with_io_pipeline_v1 (lookup.cuh:119-378),
+ * lookup_ptr_kernel_with_pipeline / tlp_lookup_ptr_kernel_with_filter
+ * (lookup_ptr.cuh:25-374) and the contains kernels (contains.cuh:46-216).
+ * No slot locks are taken: the API-level group lock keeps writers out, as in
+ * the reference (group_lock.cuh:43-56).
+ *
+ * Phases of a wavefront
+ *   own    lane L loads key L, hashes it and stages (key, bucket, digest) in LDS;
+ *   probe  tile t (8 lanes) probes key r*8+t in round r = 0..7: lane j loads
+ *          16 of the 128 digest bytes, so a tile reads one whole 128-byte line
+ *          per round; the 8 rounds are issued back to back so 8 KB of digests
+ *          are in flight per wavefront;
+ *   verify every digest match is checked against the 8-byte key (two
+ *          candidates per lane and round are fetched in the batched pass, the
+ *          rare third and later ones in a loop); the hit slot goes to LDS;
+ *   copy   the whole wavefront copies the found rows, VEC bytes per lane,
+ *          so the output side is written in fully coalesced 1 KB pieces.
+ */
+#ifndef HKV_LOOKUP_HPP_
+#define HKV_LOOKUP_HPP_
+
+#include "hkv_common.hpp"
+
+namespace hkv {
+
+struct FindArgs {
+  const uint64_t* keys;
+  uint8_t* out_values;     /* find */
+  void** out_ptrs;         /* find* */
+  uint8_t* founds;         /* may be null for the missed-keys variant */
+  uint64_t* out_scores;    /* optional */
+  uint64_t* missed_keys;   /* missed-keys variant */
+  int32_t* missed_indices;
+  int32_t* missed_size;
+  uint64_t n;
+};
+
+/*
+ * Probe the 64 keys staged in s_meta.  On return (after the caller's barrier)
+ * s_slot[k] is the table slot of key k or -1.  WANT_EMPTY selects the writers'
+ * probe: s_emask[r][lane] (when given) receives the lane's mask of EMPTY
+ * digests for round r (bw order), and LOCKED candidates count as hits.
+ */
+template <bool WANT_EMPTY>
+__device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
+                                           int64_t* s_slot,
+                                           uint32_t (*s_emask)[kWave],
+                                           int lane) {
+  const int tile = lane >> 3, j = lane & 7;
+  uint4 dg[kTile];
+  uint32_t bkt[kTile];
+  uint32_t inf[kTile];
+#pragma unroll
+  for (int r = 0; r < kTile; r++) {
+    const KeyMeta m = s_meta[r * kTile + tile];
+    bkt[r] = m.bkt;
+    inf[r] = m.info;
+    dg[r] = make_uint4(0, 0, 0, 0);
+    if (m.info & 0x100u)
+      dg[r] = *reinterpret_cast<const uint4*>(v.digests + (uint64_t)m.bkt * kBucketSize + j * 16);
+  }
+  uint32_t cm[kTile];
+  uint64_t k0[kTile], k1[kTile];
+#pragma unroll
+  for (int r = 0; r < kTile; r++) {
+    const bool valid = inf[r] & 0x100u;
+    const uint32_t d = inf[r] & 0xFFu;
+    cm[r] = valid ? match16(dg[r], d * 0x01010101u) : 0u;
+    if (WANT_EMPTY && s_emask != nullptr)
+      s_emask[r][lane] = valid ? match16(dg[r], v.empty_digest * 0x01010101u) : 0u;
+    const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
+    k0[r] = v.empty_key;
+    k1[r] = v.empty_key;
+    if (cm[r]) {
+      k0[r] = kb[bw_to_pos(__ffs(cm[r]) - 1)];
+      const uint32_t rest = cm[r] & (cm[r] - 1);
+      if (rest) k1[r] = kb[bw_to_pos(__ffs(rest) - 1)];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kTile; r++) {
+    if (!cm[r]) continue;
+    const uint64_t key = s_meta[r * kTile + tile].key;
+    const uint64_t slot0 = (uint64_t)bkt[r] * kBucketSize + j * 16;
+    uint32_t m = cm[r];
+    int hit = -1;
+    const uint32_t p0 = bw_to_pos(__ffs(m) - 1);
+    m &= m - 1;
+    /* WANT_EMPTY marks the writers' probe: a LOCKED candidate may be this key
+     * under another tile's lock that will be given back, so it is kept as the
+     * hit and settled by the writer's own CAS. */
+    if (k0[r] == key || (WANT_EMPTY && k0[r] == v.locked_key)) {
+      hit = (int)p0;
+    } else if (m) {
+      const uint32_t p1 = bw_to_pos(__ffs(m) - 1);
+      m &= m - 1;
+      if (k1[r] == key || (WANT_EMPTY && k1[r] == v.locked_key)) {
+        hit = (int)p1;
+      } else {
+        while (m) {
+          const uint32_t p = bw_to_pos(__ffs(m) - 1);
+          m &= m - 1;
+          const uint64_t kx = v.keys[slot0 + p];
+          if (kx == key || (WANT_EMPTY && kx == v.locked_key)) {
+            hit = (int)p;
+            break;
+          }
+        }
+      }
+    }
+    if (hit >= 0) s_slot[r * kTile + tile] = (int64_t)(slot0 + hit);
+  }
+}
+
+/* Lane-owned part shared by all wave-per-64-keys kernels: load, hash, stage. */
+__device__ __forceinline__ uint64_t stage_keys(const View& v,
+                                               const uint64_t* keys, uint64_t n,
+                                               uint64_t i, KeyMeta* s_meta,
+                                               int64_t* s_slot, int lane) {
+  uint64_t key = v.empty_key;
+  if (i < n) key = keys[i];
+  const bool valid = (i < n) && !is_reserved_key(v, key);
+  uint32_t bkt = 0, start = 0, digest = 0;
+  locate(v, key, bkt, start, digest);
+  KeyMeta m;
+  m.key = key;
+  m.bkt = bkt;
+  m.info = digest | (valid ? 0x100u : 0u) | (start << 16);
+  s_meta[lane] = m;
+  s_slot[lane] = -1;
+  return key;
+}
+
+enum LookupMode { kLookupValues = 0, kLookupPtr = 1, kLookupContains = 2 };
+
+template <int MODE, int VEC>
+__global__ void __launch_bounds__(kWave)
+lookup_kernel(View v, FindArgs a) {
+  __shared__ KeyMeta s_meta[kWave];
+  __shared__ int64_t s_slot[kWave];
+  const int lane = threadIdx.x;
+  const uint64_t base = (uint64_t)blockIdx.x * kWave;
+  const uint64_t i = base + lane;
+  const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
+  __syncthreads();
+  probe_wave<false>(v, s_meta, s_slot, nullptr, lane);
+  __syncthreads();
+
+  const int64_t my_slot = s_slot[lane];
+  if (i < a.n) {
+    if (a.founds) a.founds[i] = my_slot >= 0;
+    if (my_slot >= 0) {
+      if (a.out_scores) a.out_scores[i] = v.scores[my_slot];
+      if (MODE == kLookupPtr) a.out_ptrs[i] = value_row(v, (uint64_t)my_slot);
+    } else {
+      if (MODE == kLookupPtr) a.out_ptrs[i] = nullptr;
+      if (a.missed_size) {
+        /* missed-keys variant (lookup.cuh:36-60): compact list of misses;
+         * reserved keys are not probed and count as missed. */
+        const int at = atomicAdd(a.missed_size, 1);
+        a.missed_keys[at] = key;
+        a.missed_indices[at] = (int32_t)i;
+      }
+    }
+  }
+  if (MODE != kLookupValues) return;
+
+  /* copy stage: 64 rows x units-per-row spread over the 64 lanes */
+  using T = typename VecType<VEC>::type;
+  const uint32_t units = v.value_bytes / VEC;
+  const uint32_t total = units * kWave;
+  const bool pow2 = (units & (units - 1)) == 0;
+  const uint32_t sh = 31 - __clz(units);
+  constexpr int kBatch = 4;
+  for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
+    T buf[kBatch];
+    T* dst[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * kWave;
+      dst[b] = nullptr;
+      if (idx < total) {
+        const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
+        const uint32_t c = idx - kk * units;
+        const int64_t slot = s_slot[kk];
+        if (slot >= 0) {
+          buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)slot))[c];
+          dst[b] = reinterpret_cast<T*>(a.out_values + (base + kk) * v.value_bytes) + c;
+        }
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; b++)
+      if (dst[b]) *dst[b] = buf[b];
+  }
+}
+
+}  // namespace hkv
+#endif

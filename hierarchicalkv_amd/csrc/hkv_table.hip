@@ -1,0 +1,918 @@
+/*
+ * Host side of the table and the C ABI (include/hkv_c_api.h).
+ *
+ * What lives here: argument checks with the reference's messages
+ * (merlin_hashtable.cuh:1016-1048, 3832-3861), table memory (flat arenas; HBM
+ * first, pinned mapped host memory for value rows past max_hbm_for_vectors),
+ * the stream-ordered group lock, and the choice of kernel instance per call.
+ */
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "hkv_c_api.h"
+#include "hkv_misc.hpp"
+#include "hkv_upsert.hpp"
+
+using namespace hkv;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HKV_HIP(expr)                                                        \
+  do {                                                                       \
+    hipError_t e_ = (expr);                                                  \
+    if (e_ != hipSuccess)                                                    \
+      return fail(HKV_ERROR_HIP, "%s:%d %s: %s", __FILE__, __LINE__, #expr,  \
+                  hipGetErrorString(e_));                                    \
+  } while (0)
+
+#define HKV_TRY(expr)              \
+  do {                             \
+    int rc_ = (expr);              \
+    if (rc_ != HKV_SUCCESS) return rc_; \
+  } while (0)
+
+bool ispow2(uint64_t x) { return x && !(x & (x - 1)); }
+
+/*
+ * Group lock with the three roles of group_shared_mutex (group_lock.cuh:43-56):
+ * readers run with readers, updaters with updaters, an inserter runs alone.
+ * The reference blocks the host on a one-thread kernel per call; here the
+ * exclusion is expressed between streams with events, so a call never waits on
+ * the host: begin() makes `stream` wait for the conflicting work already
+ * enqueued on other streams, end() remembers that `stream` now carries work of
+ * this role.  Work on one stream is ordered by the stream itself, so a table
+ * that is only ever used from one stream records and waits on nothing.
+ */
+class StreamGroupLock {
+ public:
+  enum Role { kReader = 0, kUpdater = 1, kInserter = 2 };
+
+  ~StreamGroupLock() {
+    for (auto& r : roles_)
+      for (auto& kv : r) (void)hipEventDestroy(kv.second.ev);
+  }
+
+  hipError_t begin(Role role, hipStream_t s) {
+    mu_.lock();
+    hipError_t e = hipSuccess;
+    for (int other = 0; other < 3 && e == hipSuccess; other++) {
+      if (!conflicts(role, (Role)other)) continue;
+      for (auto& kv : roles_[other]) {
+        if (kv.first == s) continue;
+        Entry& en = kv.second;
+        if (en.dirty) {
+          e = hipEventRecord(en.ev, kv.first);
+          if (e != hipSuccess) break;
+          en.dirty = false;
+        }
+        e = hipStreamWaitEvent(s, en.ev, 0);
+        if (e != hipSuccess) break;
+      }
+    }
+    if (e != hipSuccess) mu_.unlock();
+    return e;
+  }
+
+  hipError_t end(Role role, hipStream_t s) {
+    hipError_t e = hipSuccess;
+    auto it = roles_[role].find(s);
+    if (it == roles_[role].end()) {
+      Entry en;
+      e = hipEventCreateWithFlags(&en.ev, hipEventDisableTiming);
+      if (e == hipSuccess) {
+        en.dirty = true;
+        roles_[role].emplace(s, en);
+      }
+    } else {
+      it->second.dirty = true;
+    }
+    mu_.unlock();
+    return e;
+  }
+
+  /* counts of streams carrying unpublished work per role (tests) */
+  int pending(Role role) {
+    std::lock_guard<std::mutex> g(mu_);
+    int c = 0;
+    for (auto& kv : roles_[role]) c += kv.second.dirty;
+    return c;
+  }
+
+ private:
+  struct Entry {
+    hipEvent_t ev;
+    bool dirty;
+  };
+  static bool conflicts(Role a, Role b) {
+    if (a == kInserter || b == kInserter) return true;
+    return a != b;
+  }
+  std::mutex mu_;
+  std::map<hipStream_t, Entry> roles_[3];
+};
+
+}  // namespace
+
+struct hkv_table {
+  hkv_options opts;
+  View view;
+  int device;
+  bool pure_hbm;
+  bool own_alloc;
+  hkv_allocator alloc;
+  void* d_meta;          /* digests + keys + scores + sizes in one arena */
+  uint64_t meta_bytes;
+  void* h_values;        /* host address of the pinned value rows (hybrid) */
+  unsigned long long* d_counters; /* ring of scratch words for size / size_if /
+                                     the count-returning insert_and_evict */
+  mutable std::atomic<unsigned> counter_next;
+  uint64_t epoch;
+  Clock clock;
+  mutable StreamGroupLock lock;
+};
+
+namespace {
+
+int table_alloc(hkv_table* t, int type, void** p, size_t bytes) {
+  if (!t->own_alloc) {
+    if (t->alloc.alloc(t->alloc.ctx, type, p, bytes) != 0 || !*p)
+      return fail(HKV_ERROR_RUNTIME, "allocator failed for %zu bytes (type %d)", bytes, type);
+    return HKV_SUCCESS;
+  }
+  if (type == 0) {
+    HKV_HIP(hipMalloc(p, bytes));
+  } else {
+    HKV_HIP(hipHostMalloc(p, bytes, hipHostMallocMapped | hipHostMallocPortable));
+  }
+  return HKV_SUCCESS;
+}
+
+void table_free(hkv_table* t, int type, void* p) {
+  if (!p) return;
+  if (!t->own_alloc) {
+    t->alloc.free(t->alloc.ctx, type, p);
+  } else if (type == 0) {
+    (void)hipFree(p);
+  } else {
+    (void)hipHostFree(p);
+  }
+}
+
+struct DeviceGuard {
+  int prev = -1;
+  bool ok = true;
+  explicit DeviceGuard(int dev) {
+    if (hipGetDevice(&prev) != hipSuccess) ok = false;
+    if (ok && prev != dev && hipSetDevice(dev) != hipSuccess) ok = false;
+  }
+  ~DeviceGuard() {
+    if (prev >= 0) (void)hipSetDevice(prev);
+  }
+};
+
+struct LockGuard {
+  const hkv_table* t;
+  StreamGroupLock::Role role;
+  hipStream_t s;
+  bool held = false;
+  LockGuard(const hkv_table* t_, StreamGroupLock::Role r, hipStream_t s_)
+      : t(t_), role(r), s(s_) {}
+  hipError_t acquire() {
+    if (!t->opts.api_lock) return hipSuccess;
+    hipError_t e = t->lock.begin(role, s);
+    held = e == hipSuccess;
+    return e;
+  }
+  ~LockGuard() {
+    if (held) (void)t->lock.end(role, s);
+  }
+};
+
+/* check_evict_strategy, merlin_hashtable.cuh:3832-3861 */
+int check_scores_arg(const hkv_table* t, int strategy, const uint64_t* scores) {
+  if ((strategy == HKV_LRU || strategy == HKV_EPOCH_LRU) && scores)
+    return fail(HKV_ERROR_CHECK,
+                "the scores should not be specified when running on LRU or Epoch LRU mode.");
+  if ((strategy == HKV_LFU || strategy == HKV_EPOCH_LFU) && !scores)
+    return fail(HKV_ERROR_CHECK,
+                "the scores should be specified when running on LFU or Epoch LFU mode.");
+  if (strategy == HKV_CUSTOMIZED && !scores)
+    return fail(HKV_ERROR_CHECK,
+                "the scores should be specified when running on customized mode.");
+  if ((strategy == HKV_EPOCH_LRU || strategy == HKV_EPOCH_LFU) &&
+      t->epoch == kIgnoredEpoch)
+    return fail(HKV_ERROR_CHECK,
+                "the global_epoch is invalid and should be assigned by calling "
+                "`set_global_epoch` when running on Epoch LRU or Epoch LFU mode.");
+  return HKV_SUCCESS;
+}
+
+/* widest unit (16, 4 or 1 bytes) that the row size and every pointer allow */
+int pick_vec(uint32_t value_bytes, std::initializer_list<const void*> ptrs) {
+  uintptr_t mis = value_bytes;
+  for (const void* p : ptrs) mis |= (uintptr_t)p;
+  if ((mis & 15) == 0) return 16;
+  if ((mis & 3) == 0) return 4;
+  return 1;
+}
+
+inline unsigned grid_for(uint64_t n) { return (unsigned)((n + kWave - 1) / kWave); }
+
+template <int OP, bool LOCKED_RULE>
+void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
+  const dim3 grid(grid_for(a.n)), block(kWave);
+  if (vec == 16)
+    hipLaunchKernelGGL((upsert_kernel<OP, 16, LOCKED_RULE>), grid, block, 0, s, v, a);
+  else if (vec == 4)
+    hipLaunchKernelGGL((upsert_kernel<OP, 4, LOCKED_RULE>), grid, block, 0, s, v, a);
+  else
+    hipLaunchKernelGGL((upsert_kernel<OP, 1, LOCKED_RULE>), grid, block, 0, s, v, a);
+}
+
+template <int OP>
+int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
+               hipStream_t s) {
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.value_kind = t->opts.value_kind;
+  {
+    LockGuard g(t, StreamGroupLock::kInserter, s);
+    HKV_HIP(g.acquire());
+    if (locked_rule)
+      launch_upsert<OP, true>(vec, t->view, a, s);
+    else
+      launch_upsert<OP, false>(vec, t->view, a, s);
+    HKV_HIP(hipGetLastError());
+  }
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
+}
+
+template <int MODE>
+void launch_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
+  const dim3 grid(grid_for(a.n)), block(kWave);
+  if (vec == 16)
+    hipLaunchKernelGGL((lookup_kernel<MODE, 16>), grid, block, 0, s, v, a);
+  else if (vec == 4)
+    hipLaunchKernelGGL((lookup_kernel<MODE, 4>), grid, block, 0, s, v, a);
+  else
+    hipLaunchKernelGGL((lookup_kernel<MODE, 1>), grid, block, 0, s, v, a);
+}
+
+template <class Pred>
+void launch_export(const hkv_table* t, uint64_t pattern, uint64_t threshold,
+                   uint64_t n, uint64_t offset, uint64_t* d_counter,
+                   uint64_t* keys, void* values, uint64_t* scores, hipStream_t s) {
+  const uint64_t waves = (n + kWave - 1) / kWave;
+  const unsigned blocks = (unsigned)std::min<uint64_t>((waves + 3) / 4, 16384);
+  hipLaunchKernelGGL((export_if_kernel<Pred>), dim3(blocks), dim3(256), 0, s,
+                     t->view, Pred(), pattern, threshold, offset, n,
+                     (unsigned long long*)d_counter, keys, (uint8_t*)values, scores);
+}
+
+template <class Pred>
+void launch_size_if(const hkv_table* t, uint64_t pattern, uint64_t threshold,
+                    unsigned long long* d_out, hipStream_t s) {
+  const unsigned blocks =
+      (unsigned)std::min<uint64_t>((t->view.capacity + 255) / 256, 8192);
+  hipLaunchKernelGGL((size_if_kernel<Pred>), dim3(blocks), dim3(256), 0, s,
+                     t->view, Pred(), pattern, threshold, d_out);
+}
+
+constexpr unsigned kCounterRing = 32;
+
+/* Calls that return a count synchronise before they return, so at most one
+ * word per concurrently calling host thread is in use. */
+unsigned long long* take_counter(const hkv_table* t) {
+  return t->d_counters + (t->counter_next.fetch_add(1) % kCounterRing);
+}
+
+int read_counter(unsigned long long* d, hipStream_t s, uint64_t* out) {
+  unsigned long long h = 0;
+  HKV_HIP(hipMemcpyAsync(&h, d, sizeof h, hipMemcpyDeviceToHost, s));
+  HKV_HIP(hipStreamSynchronize(s));
+  *out = h;
+  return HKV_SUCCESS;
+}
+
+int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) {
+  if (!o || !out) return fail(HKV_ERROR_ARGUMENT, "null argument");
+  /* HashTable::init, merlin_hashtable.cuh:1016-1048 */
+  if (o->table_mode != 0)
+    return fail(HKV_ERROR_UNSUPPORTED, "TableMode::kMemory (dual bucket) is not supported");
+  if (o->reserved_key_start_bit < 0 || o->reserved_key_start_bit > 62)
+    return fail(HKV_ERROR_CHECK, "options.reserved_key_start_bit should >= 0 and <= 62.");
+  if (!ispow2(o->max_bucket_size))
+    return fail(HKV_ERROR_CHECK, "Bucket size should be the pow of 2");
+  if (!ispow2(o->num_of_buckets_per_alloc))
+    return fail(HKV_ERROR_CHECK, "Then `num_of_buckets_per_alloc` should be the pow of 2");
+  if (o->init_capacity < o->num_of_buckets_per_alloc * o->max_bucket_size)
+    return fail(HKV_ERROR_CHECK,
+                "Then `num_of_buckets_per_alloc` must be equal or less than "
+                "initial required buckets number");
+  if (o->max_bucket_size != kBucketSize)
+    return fail(HKV_ERROR_UNSUPPORTED, "only max_bucket_size == 128 is supported");
+  if (o->io_by_cpu && o->max_hbm_for_vectors != 0)
+    return fail(HKV_ERROR_CHECK,
+                "[HierarchicalKV] `io_by_cpu` should not be true when "
+                "`max_hbm_for_vectors` is not 0!");
+  if (o->io_by_cpu)
+    return fail(HKV_ERROR_UNSUPPORTED, "io_by_cpu is not supported");
+  if (o->evict_strategy < 0 || o->evict_strategy > 4)
+    return fail(HKV_ERROR_ARGUMENT, "bad evict_strategy %d", o->evict_strategy);
+  if (o->score_size != 8)
+    return fail(HKV_ERROR_UNSUPPORTED, "only 64-bit scores are supported");
+  if (o->dim == 0 || o->value_size == 0)
+    return fail(HKV_ERROR_ARGUMENT, "dim and value_size must be positive");
+  if (o->dim * (uint64_t)o->value_size > (1u << 20))
+    return fail(HKV_ERROR_UNSUPPORTED, "value rows above 1 MiB are not supported");
+  const uint32_t ksz[] = {0, 4, 8, 4, 8};
+  if (o->value_kind < 0 || o->value_kind > 4 ||
+      (o->value_kind != 0 && ksz[o->value_kind] != o->value_size))
+    return fail(HKV_ERROR_ARGUMENT, "value_kind does not match value_size");
+
+  hkv_table* t = new (std::nothrow) hkv_table();
+  if (!t) return fail(HKV_ERROR_RUNTIME, "out of memory");
+  t->opts = *o;
+  t->own_alloc = al == nullptr;
+  if (al) t->alloc = *al;
+  t->d_meta = nullptr;
+  t->d_counters = nullptr;
+  t->h_values = nullptr;
+  t->counter_next = 0;
+  memset(&t->view, 0, sizeof t->view);
+  t->epoch = kIgnoredEpoch;
+  t->clock.base = 0;
+  t->clock.mode = 0;
+  t->clock.ns_per_tick = 10;
+
+  auto bail = [&](int rc) {
+    std::string keep = g_err;
+    hkv_table_destroy(t);
+    g_err = keep;
+    return rc;
+  };
+
+  if (o->device_id >= 0) {
+    hipError_t e = hipSetDevice(o->device_id);
+    if (e != hipSuccess) return bail(fail(HKV_ERROR_HIP, "hipSetDevice: %s", hipGetErrorString(e)));
+    t->device = o->device_id;
+  } else {
+    hipError_t e = hipGetDevice(&t->device);
+    if (e != hipSuccess) return bail(fail(HKV_ERROR_HIP, "hipGetDevice: %s", hipGetErrorString(e)));
+    t->opts.device_id = t->device;
+  }
+  int khz = 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, t->device) == hipSuccess &&
+      khz > 0)
+    t->clock.ns_per_tick = (uint32_t)std::max(1, 1000000 / khz);
+
+  View& v = t->view;
+  /* create_table, core_kernels.cuh:343-357 */
+  const uint64_t max_size = std::max(o->init_capacity, o->max_capacity);
+  if (o->init_capacity * 2 > max_size) {
+    v.buckets_num = 1 + (max_size - 1) / kBucketSize;
+  } else {
+    v.buckets_num = 1;
+    while (v.buckets_num * kBucketSize < o->init_capacity) v.buckets_num *= 2;
+  }
+  if (v.buckets_num >= (UINT64_C(1) << 31))
+    return bail(fail(HKV_ERROR_UNSUPPORTED, "more than 2^31 buckets"));
+  v.capacity = v.buckets_num * kBucketSize;
+  v.pow2_buckets = ispow2(v.buckets_num);
+  v.dim = (uint32_t)o->dim;
+  v.value_bytes = (uint32_t)(o->dim * o->value_size);
+  /* init_reserved_keys, types.cuh:80-109 */
+  const int b = o->reserved_key_start_bit;
+  if (b == 0) {
+    v.empty_key = UINT64_C(0xFFFFFFFFFFFFFFFF);
+    v.reclaim_key = UINT64_C(0xFFFFFFFFFFFFFFFE);
+    v.locked_key = UINT64_C(0xFFFFFFFFFFFFFFFD);
+    v.reserved_mask1 = v.reserved_mask2 = UINT64_C(0xFFFFFFFFFFFFFFFC);
+  } else {
+    v.reserved_mask1 = ~(UINT64_C(3) << b);
+    v.reserved_mask2 = v.reserved_mask1 & ~UINT64_C(1);
+    v.empty_key = v.reserved_mask2 | (UINT64_C(3) << b);
+    v.reclaim_key = ~(UINT64_C(1) << b) & ~UINT64_C(1);
+    v.locked_key = v.empty_key & ~(UINT64_C(2) << b);
+  }
+  v.empty_digest = (uint8_t)(fmix64(v.empty_key) >> 32);
+  v.reclaim_digest = (uint8_t)(fmix64(v.reclaim_key) >> 32);
+
+  /* metadata arena: digests | keys | scores | sizes, each 256-byte aligned */
+  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
+  const uint64_t off_keys = up(v.capacity);
+  const uint64_t off_scores = off_keys + up(v.capacity * 8);
+  const uint64_t off_sizes = off_scores + up(v.capacity * 8);
+  t->meta_bytes = off_sizes + up(v.buckets_num * 4);
+  int rc = table_alloc(t, 0, &t->d_meta, t->meta_bytes);
+  if (rc) return bail(rc);
+  uint8_t* m = (uint8_t*)t->d_meta;
+  v.digests = m;
+  v.keys = (uint64_t*)(m + off_keys);
+  v.scores = (uint64_t*)(m + off_scores);
+  v.sizes = (int32_t*)(m + off_sizes);
+  void* cnt = nullptr;
+  rc = table_alloc(t, 0, &cnt, kCounterRing * sizeof(unsigned long long));
+  if (rc) return bail(rc);
+  t->d_counters = (unsigned long long*)cnt;
+
+  /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
+   * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
+  const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
+  uint64_t hbm_buckets = std::min<uint64_t>(v.buckets_num, o->max_hbm_for_vectors / bucket_bytes);
+  v.hbm_slots = hbm_buckets * kBucketSize;
+  t->pure_hbm = hbm_buckets == v.buckets_num;
+  if (hbm_buckets) {
+    void* p = nullptr;
+    rc = table_alloc(t, 0, &p, hbm_buckets * bucket_bytes);
+    if (rc) return bail(rc);
+    v.values = (uint8_t*)p;
+  }
+  if (!t->pure_hbm) {
+    void* p = nullptr;
+    rc = table_alloc(t, 1, &p, (v.buckets_num - hbm_buckets) * bucket_bytes);
+    if (rc) return bail(rc);
+    t->h_values = p;
+    void* dp = nullptr;
+    hipError_t e = hipHostGetDevicePointer(&dp, p, 0);
+    if (e != hipSuccess) {
+      return bail(fail(HKV_ERROR_HIP, "hipHostGetDevicePointer: %s", hipGetErrorString(e)));
+    }
+    v.host_values = (uint8_t*)dp;
+  }
+
+  const uint64_t groups = v.capacity / 16;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, 0, v, 1);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e != hipSuccess) return bail(fail(HKV_ERROR_HIP, "table fill: %s", hipGetErrorString(e)));
+  *out = t;
+  return HKV_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" {
+
+void hkv_options_default(hkv_options* o) {
+  memset(o, 0, sizeof *o);
+  o->max_bucket_size = 128;
+  o->dim = 64;
+  o->max_load_factor = 0.5f;
+  o->block_size = 128;
+  o->io_block_size = 1024;
+  o->device_id = -1;
+  o->num_of_buckets_per_alloc = 1;
+  o->api_lock = 1;
+  o->evict_strategy = HKV_LRU;
+  o->value_kind = HKV_VALUE_F32;
+  o->value_size = 4;
+  o->score_size = 8;
+}
+
+const char* hkv_last_error(void) { return g_err.c_str(); }
+const char* hkv_version(void) { return "hkv-amd 0.1 (gfx950)"; }
+
+int hkv_table_create(const hkv_options* opts, hkv_table** out) {
+  return create_impl(opts, nullptr, out);
+}
+
+int hkv_table_create_with_allocator(const hkv_options* opts,
+                                    const hkv_allocator* allocator,
+                                    hkv_table** out) {
+  if (!allocator || !allocator->alloc || !allocator->free)
+    return fail(HKV_ERROR_ARGUMENT, "allocator callbacks must not be null");
+  return create_impl(opts, allocator, out);
+}
+
+int hkv_table_destroy(hkv_table* t) {
+  if (!t) return HKV_SUCCESS;
+  (void)hipSetDevice(t->device);
+  (void)hipDeviceSynchronize();
+  table_free(t, 0, t->d_meta);
+  table_free(t, 0, t->d_counters);
+  table_free(t, 0, t->view.values);
+  table_free(t, 1, t->h_values);
+  delete t;
+  return HKV_SUCCESS;
+}
+
+int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
+                         const void* values, const uint64_t* scores,
+                         hkv_stream_t stream, int unique_key, int ignore) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.values_in = (const uint8_t*)values;
+  a.scores = scores;
+  a.n = n;
+  a.strategy = strategy;
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  return run_upsert<kOpInsertOrAssign>(t, a, vec, !t->pure_hbm, (hipStream_t)stream);
+}
+
+int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
+                         const void* values, const uint64_t* scores,
+                         uint64_t* evicted_keys, void* evicted_values,
+                         uint64_t* evicted_scores, uint64_t* d_evicted_counter,
+                         hkv_stream_t stream, int unique_key, int ignore) {
+  if (n == 0) return HKV_SUCCESS;
+  /* merlin_hashtable.cuh:1384-1386 */
+  if (!t->pure_hbm)
+    return fail(HKV_ERROR_RUNTIME, "Only support pure HBM mode for insert_and_evict.");
+  if (!unique_key)
+    return fail(HKV_ERROR_UNSUPPORTED, "insert_and_evict needs unique keys in a batch");
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.values_in = (const uint8_t*)values;
+  a.scores = scores;
+  a.evicted_keys = evicted_keys;
+  a.evicted_values = (uint8_t*)evicted_values;
+  a.evicted_scores = evicted_scores;
+  a.evicted_counter = (unsigned long long*)d_evicted_counter;
+  a.n = n;
+  a.strategy = strategy;
+  const int vec = pick_vec(t->view.value_bytes, {values, evicted_values});
+  return run_upsert<kOpInsertAndEvict>(t, a, vec, false, (hipStream_t)stream);
+}
+
+int hkv_insert_and_evict_count(hkv_table* t, uint64_t n, const uint64_t* keys,
+                               const void* values, const uint64_t* scores,
+                               uint64_t* evicted_keys, void* evicted_values,
+                               uint64_t* evicted_scores, hkv_stream_t stream,
+                               int unique_key, int ignore, uint64_t* n_evicted) {
+  *n_evicted = 0;
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  unsigned long long* d = take_counter(t);
+  hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
+  HKV_TRY(hkv_insert_and_evict(t, n, keys, values, scores, evicted_keys,
+                               evicted_values, evicted_scores, (uint64_t*)d,
+                               stream, unique_key, ignore));
+  return read_counter(d, s, n_evicted);
+}
+
+int hkv_accum_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
+                        const void* value_or_deltas, const uint8_t* flags,
+                        const uint64_t* scores, hkv_stream_t stream, int ignore) {
+  if (n == 0) return HKV_SUCCESS;
+  if (t->opts.value_kind == HKV_VALUE_BYTES)
+    return fail(HKV_ERROR_ARGUMENT, "accum_or_assign needs an arithmetic value_kind");
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.values_in = (const uint8_t*)value_or_deltas;
+  a.accum_flags = flags;
+  a.scores = scores;
+  a.n = n;
+  a.strategy = strategy;
+  const int vec = pick_vec(t->view.value_bytes, {value_or_deltas});
+  return run_upsert<kOpAccumOrAssign>(t, a, vec, false, (hipStream_t)stream);
+}
+
+int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
+                       void* values, const uint64_t* scores, hkv_stream_t stream,
+                       int unique_key, int ignore) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.values_io = (uint8_t*)values;
+  a.scores = scores;
+  a.n = n;
+  a.strategy = strategy;
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  return run_upsert<kOpFindOrInsert>(t, a, vec, !t->pure_hbm, (hipStream_t)stream);
+}
+
+int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
+                           void** values, uint8_t* founds, const uint64_t* scores,
+                           hkv_stream_t stream, int unique_key, int ignore) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.out_ptrs = values;
+  a.founds = founds;
+  a.scores = scores;
+  a.n = n;
+  a.strategy = strategy;
+  return run_upsert<kOpFindOrInsertPtr>(t, a, 16, true, (hipStream_t)stream);
+}
+
+static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
+                         const void* values, const uint64_t* scores,
+                         int touch_scores, hipStream_t s) {
+  AssignArgs a{};
+  a.keys = keys;
+  a.values = (const uint8_t*)values;
+  a.scores = scores;
+  a.n = n;
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.touch_scores = touch_scores;
+  a.strategy = t->opts.evict_strategy;
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  {
+    LockGuard g(t, StreamGroupLock::kUpdater, s);
+    HKV_HIP(g.acquire());
+    const dim3 grid(grid_for(n)), block(kWave);
+    if (vec == 16)
+      hipLaunchKernelGGL((assign_kernel<16>), grid, block, 0, s, t->view, a);
+    else if (vec == 4)
+      hipLaunchKernelGGL((assign_kernel<4>), grid, block, 0, s, t->view, a);
+    else
+      hipLaunchKernelGGL((assign_kernel<1>), grid, block, 0, s, t->view, a);
+    HKV_HIP(hipGetLastError());
+  }
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
+}
+
+int hkv_assign(hkv_table* t, uint64_t n, const uint64_t* keys, const void* values,
+               const uint64_t* scores, hkv_stream_t stream, int unique_key) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
+  return assign_common(t, n, keys, values, scores, 1, (hipStream_t)stream);
+}
+
+int hkv_assign_scores(hkv_table* t, uint64_t n, const uint64_t* keys,
+                      const uint64_t* scores, hkv_stream_t stream, int unique_key) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
+  return assign_common(t, n, keys, nullptr, scores, 1, (hipStream_t)stream);
+}
+
+int hkv_assign_values(hkv_table* t, uint64_t n, const uint64_t* keys,
+                      const void* values, hkv_stream_t stream, int unique_key) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  return assign_common(t, n, keys, values, nullptr, 0, (hipStream_t)stream);
+}
+
+int hkv_find(const hkv_table* t, uint64_t n, const uint64_t* keys, void* values,
+             uint8_t* founds, uint64_t* scores, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  FindArgs a{};
+  a.keys = keys;
+  a.out_values = (uint8_t*)values;
+  a.founds = founds;
+  a.out_scores = scores;
+  a.n = n;
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  LockGuard g(t, StreamGroupLock::kReader, s);
+  HKV_HIP(g.acquire());
+  launch_lookup<kLookupValues>(vec, t->view, a, s);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_find_missed(const hkv_table* t, uint64_t n, const uint64_t* keys,
+                    void* values, uint64_t* missed_keys, int32_t* missed_indices,
+                    int32_t* missed_size, uint64_t* scores, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  FindArgs a{};
+  a.keys = keys;
+  a.out_values = (uint8_t*)values;
+  a.out_scores = scores;
+  a.missed_keys = missed_keys;
+  a.missed_indices = missed_indices;
+  a.missed_size = missed_size;
+  a.n = n;
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(1), 0, s, missed_size);
+  LockGuard g(t, StreamGroupLock::kReader, s);
+  HKV_HIP(g.acquire());
+  launch_lookup<kLookupValues>(vec, t->view, a, s);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_find_ptr(const hkv_table* t, uint64_t n, const uint64_t* keys,
+                 void** values, uint8_t* founds, uint64_t* scores,
+                 hkv_stream_t stream, int unique_key) {
+  (void)unique_key;
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  FindArgs a{};
+  a.keys = keys;
+  a.out_ptrs = values;
+  a.founds = founds;
+  a.out_scores = scores;
+  a.n = n;
+  LockGuard g(t, StreamGroupLock::kReader, s);
+  HKV_HIP(g.acquire());
+  launch_lookup<kLookupPtr>(16, t->view, a, s);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_contains(const hkv_table* t, uint64_t n, const uint64_t* keys,
+                 uint8_t* founds, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  FindArgs a{};
+  a.keys = keys;
+  a.founds = founds;
+  a.n = n;
+  LockGuard g(t, StreamGroupLock::kReader, s);
+  HKV_HIP(g.acquire());
+  launch_lookup<kLookupContains>(16, t->view, a, s);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  LockGuard g(t, StreamGroupLock::kInserter, s);
+  HKV_HIP(g.acquire());
+  hipLaunchKernelGGL(erase_kernel, dim3(grid_for(n)), dim3(kWave), 0, s, t->view, keys, n);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_clear(hkv_table* t, hkv_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  LockGuard g(t, StreamGroupLock::kInserter, s);
+  HKV_HIP(g.acquire());
+  const uint64_t groups = t->view.capacity / 16;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s,
+                     t->view, 0);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_export_batch_if(const hkv_table* t, int predicate, uint64_t pattern,
+                        uint64_t threshold, uint64_t n, uint64_t offset,
+                        uint64_t* d_counter, uint64_t* keys, void* values,
+                        uint64_t* scores, hkv_stream_t stream) {
+  hipStream_t s = (hipStream_t)stream;
+  if (predicate < HKV_PRED_ALWAYS || predicate > HKV_PRED_KEY_HIGH16_EQ_AND_SCORE_LT)
+    return fail(HKV_ERROR_ARGUMENT, "unknown predicate %d", predicate);
+  LockGuard g(t, StreamGroupLock::kReader, s);
+  HKV_HIP(g.acquire());
+  /* merlin_hashtable.cuh:3205-3213 */
+  hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, (unsigned long long*)d_counter);
+  if (offset >= t->view.capacity) return HKV_SUCCESS;
+  n = std::min(t->view.capacity - offset, n);
+  if (n == 0) return HKV_SUCCESS;
+  switch (predicate) {
+    case HKV_PRED_ALWAYS:
+      launch_export<PredAlways>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+    case HKV_PRED_SCORE_LT:
+      launch_export<PredScoreLt>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+    case HKV_PRED_SCORE_LE:
+      launch_export<PredScoreLe>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+    case HKV_PRED_SCORE_GT:
+      launch_export<PredScoreGt>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+    case HKV_PRED_SCORE_GE:
+      launch_export<PredScoreGe>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+    default:
+      launch_export<PredKeyHigh16AndScoreLt>(t, pattern, threshold, n, offset, d_counter, keys, values, scores, s);
+      break;
+  }
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_export_batch(const hkv_table* t, uint64_t n, uint64_t offset,
+                     uint64_t* d_counter, uint64_t* keys, void* values,
+                     uint64_t* scores, hkv_stream_t stream) {
+  return hkv_export_batch_if(t, HKV_PRED_ALWAYS, 0, 0, n, offset, d_counter, keys,
+                             values, scores, stream);
+}
+
+int hkv_size_if(const hkv_table* t, int predicate, uint64_t pattern,
+                uint64_t threshold, hkv_stream_t stream, uint64_t* out) {
+  hipStream_t s = (hipStream_t)stream;
+  if (predicate < HKV_PRED_ALWAYS || predicate > HKV_PRED_KEY_HIGH16_EQ_AND_SCORE_LT)
+    return fail(HKV_ERROR_ARGUMENT, "unknown predicate %d", predicate);
+  unsigned long long* d = take_counter(t);
+  {
+    LockGuard g(t, StreamGroupLock::kReader, s);
+    HKV_HIP(g.acquire());
+    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
+    switch (predicate) {
+      case HKV_PRED_ALWAYS: launch_size_if<PredAlways>(t, pattern, threshold, d, s); break;
+      case HKV_PRED_SCORE_LT: launch_size_if<PredScoreLt>(t, pattern, threshold, d, s); break;
+      case HKV_PRED_SCORE_LE: launch_size_if<PredScoreLe>(t, pattern, threshold, d, s); break;
+      case HKV_PRED_SCORE_GT: launch_size_if<PredScoreGt>(t, pattern, threshold, d, s); break;
+      case HKV_PRED_SCORE_GE: launch_size_if<PredScoreGe>(t, pattern, threshold, d, s); break;
+      default: launch_size_if<PredKeyHigh16AndScoreLt>(t, pattern, threshold, d, s); break;
+    }
+    HKV_HIP(hipGetLastError());
+  }
+  return read_counter(d, s, out);
+}
+
+int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out) {
+  hipStream_t s = (hipStream_t)stream;
+  unsigned long long* d = take_counter(t);
+  {
+    LockGuard g(t, StreamGroupLock::kReader, s);
+    HKV_HIP(g.acquire());
+    hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
+    const unsigned blocks =
+        (unsigned)std::min<uint64_t>((t->view.buckets_num + 255) / 256, 2048);
+    hipLaunchKernelGGL(size_kernel, dim3(blocks), dim3(256), 0, s, t->view, d);
+    HKV_HIP(hipGetLastError());
+  }
+  return read_counter(d, s, out);
+}
+
+int hkv_empty(const hkv_table* t, hkv_stream_t stream, int* out) {
+  uint64_t n = 0;
+  HKV_TRY(hkv_size(t, stream, &n));
+  *out = n == 0;
+  return HKV_SUCCESS;
+}
+
+uint64_t hkv_capacity(const hkv_table* t) { return t->view.capacity; }
+
+int hkv_load_factor(const hkv_table* t, hkv_stream_t stream, float* out) {
+  uint64_t n = 0;
+  HKV_TRY(hkv_size(t, stream, &n));
+  *out = (float)((double)n / (double)t->view.capacity);
+  return HKV_SUCCESS;
+}
+
+uint64_t hkv_dim(const hkv_table* t) { return t->opts.dim; }
+uint64_t hkv_max_bucket_size(const hkv_table* t) { return t->opts.max_bucket_size; }
+uint64_t hkv_bucket_count(const hkv_table* t) { return t->view.buckets_num; }
+int hkv_is_pure_hbm(const hkv_table* t) { return t->pure_hbm; }
+
+int hkv_set_global_epoch(hkv_table* t, uint64_t epoch) {
+  t->epoch = epoch;
+  return HKV_SUCCESS;
+}
+
+int hkv_table_get_view(const hkv_table* t, hkv_table_view* out) {
+  *out = t->view;
+  return HKV_SUCCESS;
+}
+
+int hkv_lock_begin(const hkv_table* t, int role, hkv_stream_t stream) {
+  if (role < 0 || role > 2) return fail(HKV_ERROR_ARGUMENT, "bad lock role %d", role);
+  if (!t->opts.api_lock) return HKV_SUCCESS;
+  HKV_HIP(t->lock.begin((StreamGroupLock::Role)role, (hipStream_t)stream));
+  return HKV_SUCCESS;
+}
+
+int hkv_lock_end(const hkv_table* t, int role, hkv_stream_t stream) {
+  if (role < 0 || role > 2) return fail(HKV_ERROR_ARGUMENT, "bad lock role %d", role);
+  if (!t->opts.api_lock) return HKV_SUCCESS;
+  HKV_HIP(t->lock.end((StreamGroupLock::Role)role, (hipStream_t)stream));
+  return HKV_SUCCESS;
+}
+
+int hkv_set_clock(hkv_table* t, int mode, uint64_t base) {
+  if (mode != 0 && mode != 1) return fail(HKV_ERROR_ARGUMENT, "bad clock mode %d", mode);
+  t->clock.mode = (uint32_t)mode;
+  t->clock.base = base;
+  return HKV_SUCCESS;
+}
+
+}  // extern "C"

@@ -1,0 +1,546 @@
+"""Pins for the CPU oracle (no GPU needed).
+
+The reference cannot be executed here and its tests hold no golden vectors
+(their inputs are unseeded), so every check below is either a known answer
+that the mathematics fixes, a closed-form scenario taken from one of the
+reference's own tests (cited), or an independent brute-force model written
+differently from the oracle (python dicts and sorting instead of buckets).
+"""
+import numpy as np
+import pytest
+
+import workloads as w
+from hierarchicalkv_amd import EvictStrategy, Predicate, ValueKind, default_options
+
+M64 = (1 << 64) - 1
+
+
+# ---- hash --------------------------------------------------------------------
+
+def test_fmix64_known_answers(oracle):
+    # closed-form evaluations of MurmurHash3's 64-bit finaliser
+    # (reference: utils.cuh:127-135; host twin tests/test_util.cuh:272-280)
+    assert oracle.fmix64(0) == 0
+    assert oracle.fmix64(1) == 0xB456BCFC34C2CB2C
+    assert oracle.fmix64(2) == 0x3ABF2A20650683E7
+    assert oracle.fmix64(0x0123456789ABCDEF) == 0x87CBFBFE89022CEA
+    assert oracle.fmix64(M64) == 0x64B5720B4B825F21
+    assert oracle.fmix64(M64 - 1) == 0x3A8593886C55A02B
+
+
+def test_fmix64_is_inverted_by_the_published_inverse(oracle):
+    # fmix64 is a bijection; its inverse uses the modular inverses of the two
+    # multipliers.  A wrong constant or shift in the oracle breaks the round trip.
+    def unxorshift33(x):
+        return x ^ (x >> 33)  # shift >= 32: one application undoes itself
+
+    def inverse(h):
+        h = unxorshift33(h)
+        h = (h * 0x9CB4B2F8129337DB) & M64
+        h = unxorshift33(h)
+        h = (h * 0x4F74430C22A54005) & M64
+        return unxorshift33(h)
+
+    assert (0xFF51AFD7ED558CCD * 0x4F74430C22A54005) & M64 == 1
+    assert (0xC4CEB9FE1A85EC53 * 0x9CB4B2F8129337DB) & M64 == 1
+    for k in [0, 1, 2, 12345, 0xDEADBEEFCAFEF00D, M64, M64 - 7] + [int(x) for x in w.stream(7, 0, 200)]:
+        assert inverse(oracle.fmix64(k)) == k
+
+
+def test_sentinel_digests(oracle):
+    # digest = hash bits 32..39 (kernel_utils.cuh:72-96)
+    assert (oracle.fmix64(M64) >> 32) & 0xFF == 0x0B       # EMPTY
+    assert (oracle.fmix64(M64 - 1) >> 32) & 0xFF == 0x88   # RECLAIM
+
+
+# ---- addressing ----------------------------------------------------------------
+
+def test_locate_matches_test_util_bucket_formula(oracle):
+    # tests/test_util.cuh:296-331: bkt = (hash & (capacity - 1)) / 128 for a
+    # power-of-two capacity; start = (global % 128) rounded down to 4
+    cap = 1 << 20
+    assert oracle.locate(1, cap // 128) == (1430, 44, 0xFC)
+    for k in [int(x) for x in w.stream(11, 0, 500)]:
+        h = oracle.fmix64(k)
+        g = h & (cap - 1)
+        b, s, d = oracle.locate(k, cap // 128)
+        assert b == g // 128
+        assert s == (g % 128) // 4 * 4
+        assert d == (h >> 32) & 0xFF
+
+
+def test_locate_uses_modulo_for_other_capacities(oracle):
+    nb = 524287
+    for k in [int(x) for x in w.stream(13, 0, 300)]:
+        h = oracle.fmix64(k)
+        g = h % (nb * 128)
+        assert oracle.locate(k, nb)[:2] == (g // 128, (g % 128) // 4 * 4)
+
+
+def test_bucket_count_rule(oracle):
+    # tests/merlin_hashtable_test.cc.cu:180-182, 242: capacity 64M - 129 with
+    # init == max gives 524287 buckets (no rounding to a power of two)
+    o = default_options(init_capacity=64 * 1024 * 1024 - 129, max_capacity=64 * 1024 * 1024 - 129,
+                        dim=1, value_size=1, value_kind=ValueKind.kBytes, reserved_key_start_bit=2,
+                        num_of_buckets_per_alloc=32, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    assert t.bucket_count() == 524287
+    assert t.capacity() == 524287 * 128
+    t.close()
+    # growable table (init * 2 <= max): next power of two of init / 128
+    o = default_options(init_capacity=1000, max_capacity=1 << 20, dim=1, value_size=1,
+                        value_kind=ValueKind.kBytes)
+    t = oracle.OracleTable(o)
+    assert t.bucket_count() == 8
+    t.close()
+
+
+# ---- reserved keys ---------------------------------------------------------------
+
+def test_reserved_key_truth_table(oracle):
+    # tests/reserved_keys_test.cc.cu:84-97
+    for bit in range(0, 63):
+        empty, reclaim, locked, rm1, rm2, vm1, vm2 = oracle.reserved_keys(bit)
+        is_reserved = lambda k: (k & rm1) == rm2
+        assert is_reserved(empty) and is_reserved(reclaim) and is_reserved(locked)
+        assert not is_reserved(0) and not is_reserved(0x10)
+        assert is_reserved(M64) == (bit == 0)
+        assert len({empty, reclaim, locked}) == 3
+        is_vacant = lambda k: (k & vm1) == vm2
+        assert is_vacant(empty) and is_vacant(reclaim) and not is_vacant(locked)
+    assert oracle.reserved_keys(0)[:3] == [M64, M64 - 1, M64 - 2]
+    with pytest.raises(ValueError):
+        oracle.reserved_keys(63)
+
+
+def test_reserved_keys_are_skipped_by_every_op(oracle):
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = np.array([M64, M64 - 1, M64 - 2, M64 - 3, 5], np.uint64)
+    vals = np.arange(10, dtype=np.float32).reshape(5, 2).view(np.uint8).reshape(5, 8)
+    t.insert_or_assign(keys, vals, np.arange(5, dtype=np.uint64) + 1)
+    assert t.size() == 1
+    _, founds, _ = t.find(keys)
+    assert founds.tolist() == [False, False, False, False, True]
+    t.close()
+
+
+# ---- helpers ------------------------------------------------------------------------
+
+def keys_in_bucket(oracle, n, nb, bucket, seed, lo=0, hi=M64 - 3):
+    """Rejection sampling as create_keys_in_one_buckets (test_util.cuh:296-331)."""
+    out = []
+    pos = 0
+    seen = set()
+    while len(out) < n:
+        for k in w.stream(seed, pos, 4096):
+            k = int(k) % (hi - lo) + lo
+            if k in seen:
+                continue
+            if oracle.locate(k, nb)[0] == bucket:
+                seen.add(k)
+                out.append(k)
+                if len(out) == n:
+                    break
+        pos += 4096
+    return np.array(out, np.uint64)
+
+
+def vals_of(keys, dim):
+    """v[i][j] = float(key * 0.00001) (test_util.cuh:160-163)."""
+    v = (keys.astype(np.float64) * 0.00001).astype(np.float32)
+    return np.repeat(v[:, None], dim, axis=1).copy().view(np.uint8).reshape(len(keys), dim * 4)
+
+
+def as_map(keys, values, scores):
+    return {int(k): (values[i].tobytes(), int(scores[i])) for i, k in enumerate(keys)}
+
+
+# ---- eviction scenarios from the reference's tests -----------------------------------------
+
+def test_customized_basic(oracle):
+    # tests/merlin_hashtable_test.cc.cu:2674-2849
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=4, reserved_key_start_bit=15,
+                        num_of_buckets_per_alloc=8, evict_strategy=EvictStrategy.kCustomized)
+    base = keys_in_bucket(oracle, 128, 8, 1, 21, 0, 0x3FFFFFFFFFFFFFFF)
+    test = keys_in_bucket(oracle, 128, 8, 1, 22, 0x3FFFFFFFFFFFFFFF, 0xFFFFFFFFFFFFFFFD)
+    test[64:] = base[64:]
+    bs = np.arange(1000, 1128, dtype=np.uint64)
+    ts = np.arange(1128, 1256, dtype=np.uint64)
+    t = oracle.OracleTable(o)
+    assert t.size() == 0
+    t.insert_or_assign(base, vals_of(base, 4), bs)
+    assert t.size() == 128
+    k, v, s = t.export_all()
+    assert sorted(s.tolist()) == list(range(1000, 1128))
+    assert (v == vals_of(k, 4)).all()
+    t.insert_or_assign(test, vals_of(test, 4), ts)
+    assert t.size() == 128
+    k, v, s = t.export_all()
+    assert len(k) == 128
+    assert sorted(s.tolist()) == list(range(1128, 1256))
+    assert (v == vals_of(k, 4)).all()
+    t.close()
+
+
+def test_customized_advanced(oracle):
+    # tests/merlin_hashtable_test.cc.cu:2851-3053: four low-score keys are
+    # refused, four resident keys are re-scored (one of them downwards)
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=4, reserved_key_start_bit=16,
+                        num_of_buckets_per_alloc=8, evict_strategy=EvictStrategy.kCustomized)
+    base = keys_in_bucket(oracle, 128, 8, 1, 31, 0, 0x3FFFFFFFFFFFFFFF)
+    test = keys_in_bucket(oracle, 8, 8, 1, 32, 0x3FFFFFFFFFFFFFFF, 0xFFFFFFFFFFFFFFFD)
+    test[4:8] = base[72:76]
+    ts = np.array([20, 78, 97, 98, 99, 1010, 1020, 1035], np.uint64)
+    t = oracle.OracleTable(o)
+    assert t.bucket_count() == 8
+    t.insert_or_assign(base, vals_of(base, 4), np.arange(1000, 1128, dtype=np.uint64))
+    t.insert_or_assign(test, vals_of(test, 4), ts)
+    assert t.size() == 128
+    k, v, s = t.export_all()
+    resident = as_map(k, v, s)
+    for i in range(4):
+        assert int(test[i]) not in resident
+    for i in range(4, 8):
+        assert resident[int(test[i])][1] == int(ts[i])
+    assert (v == vals_of(k, 4)).all()
+    t.close()
+
+
+def test_full_bucket_keeps_the_top_128_scores(oracle):
+    """Brute force: with distinct scores that never go down, the residents of a
+    full bucket are the 128 best of (old residents + batch), whatever the order
+    inside the batch.  The model below knows nothing about slots or digests."""
+    nb = 4
+    o = default_options(init_capacity=nb * 128, max_capacity=nb * 128, dim=2,
+                        evict_strategy=EvictStrategy.kCustomized)
+    rng = np.random.Generator(np.random.PCG64(5))
+    for trial in range(6):
+        t = oracle.OracleTable(o)
+        model = {}  # key -> (value bytes, score), per bucket resident sets derived by sorting
+        universe = w.unique_keys(100 + trial, 0, 3000)
+        for batch in range(8):
+            keys = rng.choice(universe, size=400, replace=False)
+            scores = w.monotone_scores(batch + 1, len(keys), seed=trial)
+            vals = rng.integers(0, 255, size=(len(keys), 8), dtype=np.uint8)
+            order = rng.permutation(len(keys))
+            t.insert_or_assign(keys[order].copy(), vals[order].copy(), scores[order].copy())
+            for i in range(len(keys)):
+                model[int(keys[i])] = (vals[i].tobytes(), int(scores[i]))
+            # keep the best 128 per bucket
+            by_bucket = {}
+            for k, (vv, sc) in model.items():
+                by_bucket.setdefault(oracle.locate(k, nb)[0], []).append((sc, k))
+            model = {k: model[k] for b in by_bucket.values() for sc, k in sorted(b, reverse=True)[:128]}
+            k, v, s = t.export_all()
+            assert as_map(k, v, s) == model
+            assert t.size() == len(model)
+        t.close()
+
+
+def test_refusal_rule_strict_vs_hybrid(oracle):
+    # pure HBM refuses on score < min (upsert.cuh:188), hybrid on score <= min (upsert.cuh:1524)
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    base = w.unique_keys(1, 0, 128)
+    vals = np.zeros((128, 4), np.uint8)
+    extra = w.unique_keys(2, 0, 1)
+    for hybrid, expect_in in ((False, True), (True, False)):
+        t = oracle.OracleTable(o, hybrid=hybrid)
+        t.insert_or_assign(base, vals, np.arange(10, 138, dtype=np.uint64))
+        t.insert_or_assign(extra, vals[:1], np.array([10], np.uint64))  # equal to the minimum
+        assert t.contains(extra)[0] == expect_in
+        assert t.size() == 128
+        t.close()
+
+
+# ---- insert_and_evict ------------------------------------------------------------------------
+
+def test_insert_and_evict_conservation(oracle):
+    # tests/insert_and_evict_test.cc.cu:34-48, 94, 115, 287-311:
+    # table_before + batch == table_after + evicted (as key -> value maps) and
+    # n_evicted + size_after == size_before + n_new.  Batches of never-seen keys,
+    # as in the reference's test, so no key is updated and evicted in one batch.
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    for batch in range(10):
+        keys = w.unique_keys(9, batch * 700, 700)
+        vals = vals_of(keys, 2)
+        scores = w.monotone_scores(batch + 1, len(keys), seed=3)
+        bk, bv, bs = t.export_all()
+        before = as_map(bk, bv, bs)
+        size_before = t.size()
+        ek, ev, es = t.insert_and_evict(keys, vals, scores)
+        ak, av, as_ = t.export_all()
+        after = as_map(ak, av, as_)
+        assert len(ek) + t.size() == size_before + len(keys)
+        union_in = {k: v[0] for k, v in before.items()}
+        union_in.update({int(k): vals[i].tobytes() for i, k in enumerate(keys)})
+        union_out = {k: v[0] for k, v in after.items()}
+        assert not (set(union_out) & set(int(k) for k in ek))
+        union_out.update({int(k): ev[i].tobytes() for i, k in enumerate(ek)})
+        assert union_in == union_out
+        # every evicted or refused key scores below everything left in its bucket
+        mins = {}
+        for k, (_, sc) in after.items():
+            b = oracle.locate(k, 8)[0]
+            mins[b] = min(mins.get(b, M64), sc)
+        for i, k in enumerate(ek):
+            assert int(es[i]) < mins[oracle.locate(int(k), 8)[0]]
+        # evicted scores are the scores those keys had (or were offered)
+        offered = {int(k): int(scores[i]) for i, k in enumerate(keys)}
+        for i, k in enumerate(ek):
+            k = int(k)
+            assert int(es[i]) == (before[k][1] if k in before else offered[k])
+    t.close()
+
+
+def test_insert_and_evict_with_updates_is_conservative_after_canonicalisation(oracle):
+    """Keys that are updated by a batch may be evicted earlier in the same batch
+    (with their old row) and come back; such entries are dropped before
+    comparing, everything else is conserved."""
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    universe = w.unique_keys(9, 0, 6000)
+    rng = np.random.Generator(np.random.PCG64(1))
+    for batch in range(10):
+        keys = rng.choice(universe, size=700, replace=False)
+        vals = rng.integers(0, 255, size=(700, 8), dtype=np.uint8)
+        scores = w.monotone_scores(batch + 1, len(keys), seed=3)
+        bk, bv, bs = t.export_all()
+        before = as_map(bk, bv, bs)
+        ek, ev, es = t.insert_and_evict(keys, vals, scores)
+        ak, av, as_ = t.export_all()
+        after = as_map(ak, av, as_)
+        gone = {int(k): ev[i].tobytes() for i, k in enumerate(ek) if int(k) not in after}
+        final_in = {k: v[0] for k, v in before.items()}
+        final_in.update({int(k): vals[i].tobytes() for i, k in enumerate(keys)})
+        final_out = {k: v[0] for k, v in after.items()}
+        final_out.update(gone)
+        assert final_in == final_out
+    t.close()
+
+
+def test_reclaimed_slots_are_reused_without_eviction_output(oracle):
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    base = w.unique_keys(4, 0, 128)
+    vals = np.zeros((128, 4), np.uint8)
+    t.insert_or_assign(base, vals, np.arange(100, 228, dtype=np.uint64))
+    t.erase(base[:10])
+    assert t.size() == 118
+    new = w.unique_keys(5, 0, 12)
+    ek, ev, es = t.insert_and_evict(new, vals[:12], np.arange(300, 312, dtype=np.uint64))
+    # ten tombstones absorb ten keys silently; the other two evict scores 110, 111
+    assert t.size() == 128
+    assert sorted(es.tolist()) == [110, 111]
+    assert sorted(ek.tolist()) == sorted(base[10:12].tolist())
+    t.close()
+
+
+# ---- score strategies ------------------------------------------------------------------------------
+
+def test_lfu_scores_add_up(oracle):
+    # tests/insert_and_evict_test.cc.cu:541-556: score after == increment + score before
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=1, evict_strategy=EvictStrategy.kLfu)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(6, 0, 300)
+    vals = np.zeros((300, 4), np.uint8)
+    t.insert_or_assign(keys, vals, np.full(300, 3, np.uint64))
+    t.insert_or_assign(keys[:100], vals[:100], np.full(100, 5, np.uint64))
+    _, f, s = t.find(keys)
+    assert f.all()
+    assert (s[:100] == 8).all() and (s[100:] == 3).all()
+    with pytest.raises(oracle.OracleError):
+        t.insert_or_assign(keys, vals, None)  # LFU needs scores (merlin_hashtable.cuh:3840-3845)
+    t.close()
+
+
+def test_epoch_lfu_score_format(oracle):
+    # tests/test_util.cuh:371-376: (epoch << 32) | min(freq, 0xFFFFFFFF)
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=1, evict_strategy=EvictStrategy.kEpochLfu)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(7, 0, 4)
+    vals = np.zeros((4, 4), np.uint8)
+    with pytest.raises(oracle.OracleError):
+        t.insert_or_assign(keys, vals, np.ones(4, np.uint64))  # epoch not set (:3853-3860)
+    t.set_global_epoch(7)
+    t.insert_or_assign(keys, vals, np.array([1, 2, 0xFFFFFFF0, 0x1FFFFFFFF], np.uint64))
+    _, _, s = t.find(keys)
+    assert s.tolist() == [(7 << 32) | 1, (7 << 32) | 2, (7 << 32) | 0xFFFFFFF0, (7 << 32) | 0xFFFFFFFF]
+    t.set_global_epoch(9)
+    t.insert_or_assign(keys, vals, np.array([1, 2, 0x20, 5], np.uint64))
+    _, _, s = t.find(keys)
+    # low half adds and saturates, high half takes the new epoch
+    assert s.tolist() == [(9 << 32) | 2, (9 << 32) | 4, (9 << 32) | 0xFFFFFFFF, (9 << 32) | 0xFFFFFFFF]
+    t.close()
+
+
+def test_lru_and_epoch_lru_with_deterministic_clock(oracle):
+    for strat in (EvictStrategy.kLru, EvictStrategy.kEpochLru):
+        o = default_options(init_capacity=1024, max_capacity=1024, dim=1, evict_strategy=strat)
+        t = oracle.OracleTable(o)
+        t.set_clock(1, 5 << 40)
+        if strat == EvictStrategy.kEpochLru:
+            t.set_global_epoch(3)
+        keys = w.unique_keys(8, 0, 8)
+        vals = np.zeros((8, 4), np.uint8)
+        with pytest.raises(oracle.OracleError):
+            t.insert_or_assign(keys, vals, np.ones(8, np.uint64))  # LRU takes no scores
+        t.insert_or_assign(keys, vals)
+        _, _, s = t.find(keys)
+        now = [(5 << 40) + (i << 20) for i in range(8)]
+        if strat == EvictStrategy.kLru:
+            assert s.tolist() == now
+        else:
+            assert s.tolist() == [(3 << 32) | ((x >> 20) & 0xFFFFFFFF) for x in now]
+        t.close()
+
+
+# ---- accum_or_assign -------------------------------------------------------------------------------------
+
+def test_accum_or_assign_truth_table(oracle):
+    # tests/accum_or_assign_test.cc.cu:2818-2845
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=3, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(10, 0, 8)
+    base = np.arange(24, dtype=np.float32).reshape(8, 3)
+    t.insert_or_assign(keys[:4], base[:4].copy().view(np.uint8).reshape(4, 12), np.arange(1, 5, dtype=np.uint64))
+    delta = np.full((8, 3), 0.5, np.float32)
+    flags = np.array([1, 0, 1, 0, 1, 0, 1, 0], np.uint8)  # accum / assign alternating
+    t.accum_or_assign(keys, delta.view(np.uint8).reshape(8, 12), flags, np.arange(11, 19, dtype=np.uint64))
+    v, f, s = t.find(keys)
+    v = v.view(np.float32).reshape(8, 3)
+    # existed & accum -> old + delta ; existed & assign -> unchanged
+    assert f.tolist() == [True, True, True, True, False, True, False, True]
+    assert (v[0] == base[0] + 0.5).all() and s[0] == 11
+    assert (v[1] == base[1]).all() and s[1] == 2
+    assert (v[2] == base[2] + 0.5).all() and s[2] == 13
+    assert (v[3] == base[3]).all() and s[3] == 4
+    # missing & assign -> inserted with the delta as value ; missing & accum -> nothing
+    assert (v[5] == 0.5).all() and s[5] == 16
+    assert (v[7] == 0.5).all() and s[7] == 18
+    assert t.size() == 6
+    t.close()
+
+
+# ---- find_or_insert, assign family -------------------------------------------------------------------------
+
+def test_find_or_insert_reads_hits_and_writes_misses(oracle):
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(12, 0, 6)
+    old = np.arange(6, dtype=np.float32).reshape(3, 2)
+    t.insert_or_assign(keys[:3], old.copy().view(np.uint8).reshape(3, 8), np.array([5, 6, 7], np.uint64))
+    io = np.full((6, 2), 9.0, np.float32).view(np.uint8).reshape(6, 8).copy()
+    t.find_or_insert(keys, io, np.arange(20, 26, dtype=np.uint64))
+    got = io.view(np.float32).reshape(6, 2)
+    assert (got[:3] == old).all() and (got[3:] == 9.0).all()
+    v, f, s = t.find(keys)
+    assert f.all()
+    assert s.tolist() == [20, 21, 22, 23, 24, 25]  # Customized: hit re-scores (kernel_utils.cuh:581-593)
+    assert (v.view(np.float32).reshape(6, 2)[3:] == 9.0).all()
+    t.close()
+
+
+def test_assign_family_never_inserts(oracle):
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(14, 0, 6)
+    z = np.zeros((6, 8), np.uint8)
+    t.insert_or_assign(keys[:3], z[:3], np.array([1, 2, 3], np.uint64))
+    ones = np.ones((6, 2), np.float32).view(np.uint8).reshape(6, 8)
+    t.assign(keys, ones, np.arange(10, 16, dtype=np.uint64))
+    assert t.size() == 3
+    v, f, s = t.find(keys)
+    assert f.tolist() == [True] * 3 + [False] * 3
+    assert (v[:3] == ones[:3]).all() and s[:3].tolist() == [10, 11, 12]
+    t.assign_scores(keys, np.arange(30, 36, dtype=np.uint64))
+    t.assign_values(keys, z)
+    v, f, s = t.find(keys)
+    assert (v[:3] == 0).all() and s[:3].tolist() == [30, 31, 32]
+    t.close()
+
+
+# ---- export / size_if / erase / clear -----------------------------------------------------------------------------
+
+def test_export_batch_if_and_size_if_agree(oracle):
+    # tests/export_batch_if_test.cc.cu:214-222, 268-296
+    o = default_options(init_capacity=4096, max_capacity=4096, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(15, 0, 3000)
+    scores = (w.stream(16, 0, 3000) % np.uint64(1000)).astype(np.uint64)
+    t.insert_or_assign(keys, vals_of(keys, 2), scores)
+    kk, vv, ss = t.export_all()
+    resident = as_map(kk, vv, ss)
+    for pred, fn in ((Predicate.kScoreLt, lambda s: s < 400), (Predicate.kScoreGe, lambda s: s >= 400),
+                     (Predicate.kScoreGt, lambda s: s > 400), (Predicate.kScoreLe, lambda s: s <= 400)):
+        k, v, s = t.export_batch_if(pred, 0, 400)
+        assert len(set(k.tolist())) == len(k)
+        assert t.size_if(pred, 0, 400) == len(k)
+        assert all(fn(int(x)) for x in s)
+        assert as_map(k, v, s) == {a: b for a, b in resident.items() if fn(b[1])}
+    # windows of the slot range partition the table
+    total = 0
+    for off in range(0, 4096, 1000):
+        k, _, _ = t.export_batch_if(Predicate.kAlways, 0, 0, n=1000, offset=off)
+        total += len(k)
+    assert total == t.size()
+    assert len(t.export_batch_if(Predicate.kAlways, 0, 0, n=10, offset=4096)[0]) == 0
+    t.close()
+
+
+def test_erase_and_clear_counts(oracle):
+    # tests/merlin_hashtable_test.cc.cu:336-344
+    o = default_options(init_capacity=4096, max_capacity=4096, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(17, 0, 2000)
+    z = np.zeros((2000, 4), np.uint8)
+    t.insert_or_assign(keys, z, np.arange(1, 2001, dtype=np.uint64))
+    n0 = t.size()
+    present = t.contains(keys)
+    t.erase(keys[:1000])
+    assert t.size() == n0 - int(present[:1000].sum())
+    assert not t.contains(keys[:1000]).any()
+    t.erase(keys[:1000])  # erasing twice changes nothing
+    assert t.size() == n0 - int(present[:1000].sum())
+    t.clear()
+    assert t.size() == 0
+    assert len(t.export_all()[0]) == 0
+    t.insert_or_assign(keys, z, np.arange(1, 2001, dtype=np.uint64))
+    assert t.size() == n0
+    t.close()
+
+
+# ---- argument checks ----------------------------------------------------------------------------------------------------
+
+def test_init_checks(oracle):
+    # merlin_hashtable.cuh:1016-1048
+    with pytest.raises(oracle.OracleError):
+        oracle.OracleTable(default_options(init_capacity=1024, max_capacity=1024, reserved_key_start_bit=63))
+    with pytest.raises(oracle.OracleError):
+        oracle.OracleTable(default_options(init_capacity=1024, max_capacity=1024, max_bucket_size=100))
+    with pytest.raises(oracle.OracleError):
+        oracle.OracleTable(default_options(init_capacity=1024, max_capacity=1024, num_of_buckets_per_alloc=3))
+    with pytest.raises(oracle.OracleError):
+        oracle.OracleTable(default_options(init_capacity=128, max_capacity=128, num_of_buckets_per_alloc=2))
+
+
+def test_multithreaded_baseline_equals_sequential(oracle):
+    o = default_options(init_capacity=1 << 14, max_capacity=1 << 14, dim=4, evict_strategy=EvictStrategy.kCustomized)
+    a = oracle.OracleTable(o)
+    b = oracle.OracleTable(o)
+    for batch in range(4):
+        keys = w.unique_keys(20, batch * 9000, 9000)
+        vals = vals_of(keys, 4)
+        sc = w.monotone_scores(batch + 1, 9000)
+        a.insert_or_assign(keys, vals, sc)
+        b.insert_or_assign_mt(keys, vals, sc, threads=4)
+    ka, va, sa = a.export_all()
+    kb, vb, sb = b.export_all()
+    assert as_map(ka, va, sa) == as_map(kb, vb, sb)
+    q = w.unique_keys(20, 20000, 9000)
+    v1, f1, s1 = a.find(q)
+    v2, f2, s2 = b.find(q, threads=4)
+    assert (f1 == f2).all() and (v1 == v2).all() and (s1 == s2).all()
+    a.close()
+    b.close()
