@@ -122,6 +122,14 @@ def load(path=LIB_PATH):
             f"{path} is missing: the HIP library has not been built. Run "
             "`python -c 'import __graft_entry__ as g; g.build()'` (or "
             "`python hierarchicalkv_amd/build.py lib`) in the repository root.")
+    # A process must hold one HIP runtime only.  PyTorch wheels bundle their own
+    # libamdhip64 (same soname as the system one); when torch is going to be used
+    # for the device buffers it has to be loaded first, so that this library binds
+    # to the runtime torch already brought in instead of loading a second one.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)

@@ -42,15 +42,19 @@ struct FindArgs {
 
 /*
  * Probe the 64 keys staged in s_meta.  On return (after the caller's barrier)
- * s_slot[k] is the table slot of key k or -1.  WANT_EMPTY selects the writers'
- * probe: s_emask[r][lane] (when given) receives the lane's mask of EMPTY
- * digests for round r (bw order), and LOCKED candidates count as hits.
+ * s_slot[k] is the table slot of key k or -1.  WRITER selects the writers'
+ * probe, which runs while other wavefronts change the table:
+ *   - s_emask[r][lane] (when given) receives the lane's mask of EMPTY digests
+ *     for round r (bw order);
+ *   - a candidate slot whose key word reads LOCKED may be this very key under
+ *     another tile's lock, so s_unsure[k] is raised and the writer settles the
+ *     question with a second, coherent probe of its own (tile_reprobe).
  */
-template <bool WANT_EMPTY>
+template <bool WRITER>
 __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
                                            int64_t* s_slot,
                                            uint32_t (*s_emask)[kWave],
-                                           int lane) {
+                                           uint8_t* s_unsure, int lane) {
   const int tile = lane >> 3, j = lane & 7;
   uint4 dg[kTile];
   uint32_t bkt[kTile];
@@ -71,7 +75,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     const bool valid = inf[r] & 0x100u;
     const uint32_t d = inf[r] & 0xFFu;
     cm[r] = valid ? match16(dg[r], d * 0x01010101u) : 0u;
-    if (WANT_EMPTY && s_emask != nullptr)
+    if (WRITER && s_emask != nullptr)
       s_emask[r][lane] = valid ? match16(dg[r], v.empty_digest * 0x01010101u) : 0u;
     const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
     k0[r] = v.empty_key;
@@ -85,36 +89,69 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
 #pragma unroll
   for (int r = 0; r < kTile; r++) {
     if (!cm[r]) continue;
-    const uint64_t key = s_meta[r * kTile + tile].key;
+    const int kk = r * kTile + tile;
+    const uint64_t key = s_meta[kk].key;
     const uint64_t slot0 = (uint64_t)bkt[r] * kBucketSize + j * 16;
     uint32_t m = cm[r];
     int hit = -1;
-    const uint32_t p0 = bw_to_pos(__ffs(m) - 1);
-    m &= m - 1;
-    /* WANT_EMPTY marks the writers' probe: a LOCKED candidate may be this key
-     * under another tile's lock that will be given back, so it is kept as the
-     * hit and settled by the writer's own CAS. */
-    if (k0[r] == key || (WANT_EMPTY && k0[r] == v.locked_key)) {
-      hit = (int)p0;
-    } else if (m) {
-      const uint32_t p1 = bw_to_pos(__ffs(m) - 1);
+    bool unsure = false;
+    int c = 0;
+    while (m) {
+      const uint32_t p = bw_to_pos(__ffs(m) - 1);
       m &= m - 1;
-      if (k1[r] == key || (WANT_EMPTY && k1[r] == v.locked_key)) {
-        hit = (int)p1;
-      } else {
-        while (m) {
-          const uint32_t p = bw_to_pos(__ffs(m) - 1);
-          m &= m - 1;
-          const uint64_t kx = v.keys[slot0 + p];
-          if (kx == key || (WANT_EMPTY && kx == v.locked_key)) {
-            hit = (int)p;
-            break;
-          }
-        }
+      const uint64_t kx = c == 0 ? k0[r] : (c == 1 ? k1[r] : v.keys[slot0 + p]);
+      c++;
+      if (kx == key) {
+        hit = (int)p;
+        break;
       }
+      if (WRITER && kx == v.locked_key) unsure = true;
     }
-    if (hit >= 0) s_slot[r * kTile + tile] = (int64_t)(slot0 + hit);
+    if (hit >= 0)
+      s_slot[kk] = (int64_t)(slot0 + hit);
+    else if (WRITER && unsure)
+      s_unsure[kk] = 1;
   }
+}
+
+/*
+ * Second opinion for a writer, by the 8-lane tile that owns the key, with
+ * coherent loads: returns the slot of the key, -1 when the key is not in the
+ * bucket, or -2 when a digest-matching slot is LOCKED right now (ask again).
+ * `em` receives the lane's fresh mask of EMPTY digests.
+ */
+__device__ __forceinline__ int64_t tile_reprobe(const View& v, uint64_t key,
+                                                uint32_t bkt, uint32_t digest,
+                                                int tile, int j, uint32_t& em) {
+  const uint32_t* dp =
+      reinterpret_cast<const uint32_t*>(v.digests + (uint64_t)bkt * kBucketSize + j * 16);
+  uint4 d;
+  d.x = __hip_atomic_load(dp + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  d.y = __hip_atomic_load(dp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  d.z = __hip_atomic_load(dp + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  d.w = __hip_atomic_load(dp + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  em = match16(d, v.empty_digest * 0x01010101u);
+  uint32_t m = match16(d, digest * 0x01010101u);
+  const uint64_t slot0 = (uint64_t)bkt * kBucketSize + j * 16;
+  int hit = -1;
+  bool locked = false;
+  while (m) {
+    const uint32_t p = bw_to_pos(__ffs(m) - 1);
+    m &= m - 1;
+    const uint64_t kx = ld_u64(v.keys + slot0 + p);
+    if (kx == key) {
+      hit = (int)p;
+      break;
+    }
+    if (kx == v.locked_key) locked = true;
+  }
+  const uint32_t hits = tile_ballot(hit >= 0, tile);
+  const uint32_t locks = tile_ballot(locked, tile);
+  if (hits) {
+    const int jl = __ffs(hits) - 1;
+    return (int64_t)tile_bcast((uint32_t)hit, tile, jl) + (int64_t)bkt * kBucketSize + jl * 16;
+  }
+  return locks ? -2 : -1;
 }
 
 /* Lane-owned part shared by all wave-per-64-keys kernels: load, hash, stage. */
@@ -148,7 +185,7 @@ lookup_kernel(View v, FindArgs a) {
   const uint64_t i = base + lane;
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, lane);
+  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
 
   const int64_t my_slot = s_slot[lane];

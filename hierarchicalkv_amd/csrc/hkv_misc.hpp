@@ -41,7 +41,7 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint64_t key = stage_keys(v, keys, n, i, s_meta, s_slot, lane);
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, lane);
+  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   const int64_t slot = s_slot[lane];
   if (slot >= 0 && cas_acquire(v.keys + slot, key, v.reclaim_key)) {
@@ -114,22 +114,35 @@ __global__ void __launch_bounds__(kWave)
 assign_kernel(View v, AssignArgs a) {
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
+  __shared__ uint8_t s_unsure[kWave];
   const int lane = threadIdx.x;
   const int tile = lane >> 3, j = lane & 7;
   const uint64_t base = (uint64_t)blockIdx.x * kWave;
   stage_keys(v, a.keys, a.n, base + lane, s_meta, s_slot, lane);
+  s_unsure[lane] = 0;
   __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, nullptr, lane);
+  probe_wave<true>(v, s_meta, s_slot, nullptr, s_unsure, lane);
   __syncthreads();
 #pragma unroll 1
   for (int r = 0; r < kTile; r++) {
     const int kk = r * kTile + tile;
     const uint64_t i = base + kk;
-    const uint64_t key = s_meta[kk].key;
+    const KeyMeta m = s_meta[kk];
+    const uint64_t key = m.key;
     int64_t slot = s_slot[kk];
-    bool pending = slot >= 0;
+    bool reprobe = slot < 0 && s_unsure[kk];
+    bool pending = slot >= 0 || reprobe;
     while (true) {
-      if (pending) {
+      if (pending && reprobe) {
+        uint32_t em_unused;
+        slot = tile_reprobe(v, key, m.bkt, m.info & 0xFFu, tile, j, em_unused);
+        if (slot == -2) {
+          __builtin_amdgcn_s_sleep(2);
+        } else {
+          reprobe = false;
+          pending = slot >= 0;
+        }
+      } else if (pending) {
         int ok = 0;
         if (j == 0) {
           uint64_t seen = key;
@@ -149,7 +162,7 @@ assign_kernel(View v, AssignArgs a) {
           if (j == 0) st_release(v.keys + slot, key);
           pending = false;
         } else if (ok < 0) {
-          pending = false;
+          reprobe = true; /* the slot changed hands: look again */
         } else {
           __builtin_amdgcn_s_sleep(2);
         }

@@ -169,6 +169,7 @@ upsert_kernel(View v, UpsertArgs a) {
   __shared__ int64_t s_slot[kWave];
   __shared__ uint64_t s_in_score[kWave];
   __shared__ uint32_t s_emask[kTile][kWave];
+  __shared__ uint8_t s_unsure[kWave];
 
   const int lane = threadIdx.x;
   const int tile = lane >> 3, j = lane & 7;
@@ -177,9 +178,10 @@ upsert_kernel(View v, UpsertArgs a) {
     const uint64_t i = base + lane;
     stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
     s_in_score[lane] = (a.scores && i < a.n) ? a.scores[i] : 0;
+    s_unsure[lane] = 0;
   }
   __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, s_emask, lane);
+  probe_wave<true>(v, s_meta, s_slot, s_emask, s_unsure, lane);
   __syncthreads();
 
 #pragma unroll 1
@@ -195,9 +197,18 @@ upsert_kernel(View v, UpsertArgs a) {
     int64_t hit = s_slot[kk];
     uint32_t em = s_emask[r][lane];
     int status = (m.info & 0x100u) ? kStInitial : kStSkip;
+    bool reprobe = hit < 0 && s_unsure[kk];
 
     while (true) {
-      if (status == kStInitial) {
+      if (status == kStInitial && reprobe) {
+        const int64_t found = tile_reprobe(v, key, m.bkt, digest, tile, j, em);
+        if (found == -2) {
+          __builtin_amdgcn_s_sleep(2);
+        } else {
+          hit = found;
+          reprobe = false;
+        }
+      } else if (status == kStInitial) {
         uint64_t desired = desired_when_missed(a, in_score, i);
         int got = kStInitial;   /* outcome if a lock was taken in this trip */
         uint32_t pos = 0;
@@ -223,7 +234,10 @@ upsert_kernel(View v, UpsertArgs a) {
             pos = (uint32_t)(hit - (int64_t)bslot);
             victim = key;
           } else if (ok < 0) {
+            /* the slot belongs to another key now: ours was evicted in this
+             * batch, or the probe was looking at somebody else's lock */
             hit = -1;
+            reprobe = true;
           } else {
             __builtin_amdgcn_s_sleep(2);
           }
