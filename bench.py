@@ -1,0 +1,236 @@
+#!/usr/bin/env python
+"""Benchmark of the hot path on one MI355X.
+
+Workload (BASELINE.json metric shape): capacity 2^26 keys, uint64 keys, fp32
+values dim 64 (16 GiB of value rows, all in HBM), uint64 scores, LRU, batch
+2^20, table pre-filled to load factor 1.0.  One step = find on 2^20 resident
+keys (100 % hits) followed by insert_or_assign of 2^20 keys, half resident and
+half new (every new key evicts the bucket's minimum).  Inputs and outputs are
+resident in HBM when the timed region starts.
+
+Prints one JSON line: whole-step throughput in 10^9 KV/s, per-op figures, the
+HBM roofline of each kernel from HIP-event timings inside the timed region, and
+a CPU baseline (the multithreaded host oracle on a bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+# algorithmic bytes per key (minimum traffic the mandated layout implies):
+#   find hit   = 8 key + 128 digest line + 8 key verify + VB read + VB write + 1 found
+#   upsert hit = 8 + 128 + 8 lock + VB in + VB out + 8 score + 1 digest + 8 unlock
+#   upsert miss in a full bucket = upsert hit + 1024 (score scan)
+def find_bytes(vb):
+    return 145 + 2 * vb
+
+
+def upsert_bytes(vb, new_fraction):
+    return (1.0 - new_fraction) * (161 + 2 * vb) + new_fraction * (1185 + 2 * vb)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--capacity-log2", type=int, default=26)
+    ap.add_argument("--dim", type=int, default=64)
+    ap.add_argument("--batch-log2", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-capacity-log2", type=int, default=24)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              "(one table per device, as in the reference); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import workloads as w
+    from hierarchicalkv_amd import EvictStrategy, HashTable, default_options
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    cap = 1 << args.capacity_log2
+    dim = args.dim
+    n = 1 << args.batch_log2
+    vb = dim * 4
+    seed = 0x484B5600
+    K, W = args.steps, args.warmup
+
+    opts = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb,
+                           dim=dim, evict_strategy=EvictStrategy.kLru)
+    table = HashTable()
+    table.init(opts)
+    assert table.is_pure_hbm()
+
+    def d64(a):
+        return torch.from_numpy(a.view(np.int64)).to(dev)
+
+    # ---- prefill to load factor 1.0 (untimed) ------------------------------------
+    t0 = time.time()
+    pos = 0
+    vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
+    size0 = 0
+    # uniform hashing fills the last slots slowly: keep inserting (the fullest
+    # buckets evict meanwhile) until 99.9 % of the slots hold a key
+    while size0 < 0.999 * cap and pos < 3 * cap:
+        for _ in range(max(1, (cap // n) // 8)):
+            keys = w.unique_keys(seed, pos, n)
+            vals.uniform_(-1.0, 1.0)
+            table.insert_or_assign(n, d64(keys), vals)
+            pos += n
+        size0 = table.size()
+    prefill_s = time.time() - t0
+
+    # ---- per-step inputs, resident in HBM ------------------------------------------
+    # step s: find the keys inserted by step s-1 (all resident, highest LRU scores);
+    #         insert_or_assign half of those again + as many never-seen keys.
+    steps = K + W
+    prev = w.unique_keys(seed, pos - n, n)  # last prefill batch
+    find_keys, ins_keys = [], []
+    for s in range(steps):
+        find_keys.append(d64(prev))
+        fresh = w.unique_keys(seed, pos, n // 2)
+        pos += n // 2
+        batch = np.concatenate([prev[: n // 2], fresh])
+        ins_keys.append(d64(batch))
+        prev = batch
+    ins_vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
+    out_vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
+    founds = torch.empty(n, dtype=torch.bool, device=dev)
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+
+    def step(s):
+        ev[s][0].record()
+        table.find(n, find_keys[s], out_vals, founds)
+        ev[s][1].record()
+        table.insert_or_assign(n, ins_keys[s], ins_vals)
+        ev[s][2].record()
+
+    for s in range(W):
+        step(s)
+    torch.cuda.synchronize()
+    hit_rate = float(founds.float().mean().item())
+    t_start = time.perf_counter()
+    for s in range(W, steps):
+        step(s)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_start
+
+    find_ms = [ev[s][0].elapsed_time(ev[s][1]) for s in range(W, steps)]
+    ups_ms = [ev[s][1].elapsed_time(ev[s][2]) for s in range(W, steps)]
+    find_avg = sum(find_ms) / K
+    ups_avg = sum(ups_ms) / K
+    size1 = table.size()
+
+    value = 2.0 * n * K / wall / 1e9
+    fb = find_bytes(vb) * n
+    ub = upsert_bytes(vb, 0.5) * n
+    find_gbs = fb / (find_avg * 1e-3) / 1e9
+    ups_gbs = ub / (ups_avg * 1e-3) / 1e9
+
+    result = {
+        "metric": "billion-KV/s for find & insert_or_assign, dim 64, load factor 1.0, 1 GPU",
+        "value": round(value, 4),
+        "unit": "billion-KV/s (10^9 keys/s, find + insert_or_assign per step)",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(wall / K * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u64 keys/scores, fp32 values copied as bytes",
+        "data": "synthetic",
+        "config": {
+            "workload": f"capacity 2^{args.capacity_log2}, dim {dim} fp32, batch 2^{args.batch_log2}, "
+                        "LRU, load factor 1.0; step = find (100% hit) + insert_or_assign (50% new)",
+            "load_factor": round(size0 / cap, 4),
+            "find_hit_rate": round(hit_rate, 4),
+            "size_before": size0,
+            "size_after": size1,
+            "prefill_s": round(prefill_s, 1),
+        },
+        "find": {"ms": round(find_avg, 4), "bkvs": round(n / (find_avg * 1e-3) / 1e9, 4),
+                 "bkvs_2p30": round(n / (find_avg * 1e-3) / 2**30, 4)},
+        "insert_or_assign": {"ms": round(ups_avg, 4), "bkvs": round(n / (ups_avg * 1e-3) / 1e9, 4),
+                             "bkvs_2p30": round(n / (ups_avg * 1e-3) / 2**30, 4)},
+        "roofline": {"kernel": "upsert_kernel<insert_or_assign>", "bound": "hbm",
+                     "achieved": round(ups_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_key": upsert_bytes(vb, 0.5)},
+        "roofline_find": {"kernel": "lookup_kernel<values>", "bound": "hbm",
+                          "achieved": round(find_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": round(find_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                          "bytes_per_key": find_bytes(vb)},
+    }
+    table.close()
+    del find_keys, ins_keys, ins_vals, out_vals
+    torch.cuda.empty_cache()
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args, np, w)
+    print(json.dumps(result))
+
+
+def cpu_baseline(args, np, w):
+    """The host oracle (multithreaded variant, a port of the same semantics) on a
+    bounded sample: same dim / batch / load factor 1.0 at a smaller capacity."""
+    import oracle_binding as ob
+    from hierarchicalkv_amd import EvictStrategy, default_options
+
+    cap = 1 << args.cpu_capacity_log2
+    dim = args.dim
+    n = 1 << args.batch_log2
+    threads = min(ob.online_cores(), 16)
+    seed = 0x484B5600
+    opts = default_options(init_capacity=cap, max_capacity=cap, dim=dim, evict_strategy=EvictStrategy.kLru)
+    t = ob.OracleTable(opts)
+    vals = np.random.default_rng(1).random((n, dim), dtype=np.float32).view(np.uint8).reshape(n, dim * 4)
+    pos = 0
+    while pos < cap:
+        t.insert_or_assign_mt(w.unique_keys(seed, pos, n), vals, threads=threads)
+        pos += n
+    prev = w.unique_keys(seed, pos - n, n)
+    reps = 3
+    tf = ti = 0.0
+    out = np.zeros((n, dim * 4), np.uint8)
+    for r in range(reps):
+        a = time.perf_counter()
+        t.find(prev, out, want_scores=False, threads=threads)
+        b = time.perf_counter()
+        batch = np.concatenate([prev[: n // 2], w.unique_keys(seed, pos, n // 2)])
+        pos += n // 2
+        c = time.perf_counter()
+        t.insert_or_assign_mt(batch, vals, threads=threads)
+        d = time.perf_counter()
+        tf += b - a
+        ti += d - c
+        prev = batch
+    t.close()
+    return {
+        "value": round(2.0 * n * reps / (tf + ti) / 1e9, 5),
+        "unit": "billion-KV/s (10^9 keys/s, find + insert_or_assign per step)",
+        "cores": threads,
+        "kind": "port",
+        "find_bkvs": round(n * reps / tf / 1e9, 5),
+        "insert_or_assign_bkvs": round(n * reps / ti / 1e9, 5),
+        "sample": f"{reps} steps of the same workload at capacity 2^{args.cpu_capacity_log2} "
+                  f"(dim {dim}, batch 2^{args.batch_log2}, load factor 1.0), host oracle with "
+                  f"{threads} threads; table pre-filled by the same code",
+    }
+
+
+if __name__ == "__main__":
+    main()

@@ -89,29 +89,56 @@ __device__ __forceinline__ uint32_t tile_ballot(bool pred, int tile) {
   return (uint32_t)(__ballot(pred) >> (tile * kTile)) & 0xFFu;
 }
 
-/* ---- coherent access to words other wavefronts may be changing ----------- */
+/* ---- coherent access to words other wavefronts may be changing -----------
+ *
+ * An MI355X has one L2 per XCD (8 of them); ordinary cached loads and stores
+ * are only coherent inside one XCD until a kernel ends.  Acquire / release at
+ * agent scope would make the compiler write back and invalidate the whole L2
+ * around every slot lock, which costs far more than the lock protects.  So the
+ * protocol is built from agent-scope *relaxed* accesses instead: such loads
+ * and stores carry the sc1 bit, i.e. stores write through to memory and loads
+ * do not trust a line another XCD may have changed.  Everything a second
+ * wavefront may read or overwrite while this kernel runs (key words, digests,
+ * scores, and value rows of the table) goes through these helpers; the unlock
+ * waits for the wavefront's outstanding stores first (wait_stores). */
 
 __device__ __forceinline__ uint64_t ld_u64(const uint64_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t ld_u32(const uint32_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint8_t ld_u8(const uint8_t* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_u64(uint64_t* p, uint64_t x) {
   __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void st_u32(uint32_t* p, uint32_t x) {
+  __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void st_u8(uint8_t* p, uint8_t x) {
   __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-/* Slot lock: CAS(expected -> LOCKED) with acquire, as the reference's
- * compare_exchange_strong(…, acquire, relaxed) on the key word
- * (upsert.cuh:104-110). */
-__device__ __forceinline__ bool cas_acquire(uint64_t* p, uint64_t expected,
-                                            uint64_t desired) {
-  return __hip_atomic_compare_exchange_strong(
-      p, &expected, desired, __ATOMIC_ACQUIRE, __ATOMIC_RELAXED,
-      __HIP_MEMORY_SCOPE_AGENT);
+/* Slot lock: CAS(expected -> LOCKED) on the key word (the reference's
+ * compare_exchange_strong, upsert.cuh:104-110).  On failure `expected` holds
+ * the word that was found. */
+__device__ __forceinline__ bool cas_lock(uint64_t* p, uint64_t& expected,
+                                         uint64_t desired) {
+  return __hip_atomic_compare_exchange_strong(p, &expected, desired,
+                                              __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
 }
-/* Slot unlock: release store of the key word (upsert.cuh:228-232). */
-__device__ __forceinline__ void st_release(uint64_t* p, uint64_t x) {
-  __hip_atomic_store(p, x, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+/* Every store this wavefront has issued is complete (written through) and the
+ * compiler moves no memory access across this point. */
+__device__ __forceinline__ void wait_stores() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+/* Slot unlock: the key word becomes visible after everything written under
+ * the lock (the reference's release store, upsert.cuh:228-232).  The caller
+ * has executed wait_stores() with all lanes of the tile active. */
+__device__ __forceinline__ void st_unlock(uint64_t* p, uint64_t x) {
+  __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* ---- clock ------------------------------------------------------------------ */
@@ -153,23 +180,73 @@ struct VecType<1> {
   using type = uint8_t;
 };
 
-template <int VEC>
+/* Row copy by the 8 lanes of a tile, VEC bytes per lane and trip (16, 4 or 1).
+ * DST_TABLE / SRC_TABLE say which side is a value row of the table and must be
+ * accessed coherently (8-, 4- or 1-byte agent-scope accesses); the caller's
+ * buffers are accessed with plain VEC-wide loads and stores. */
+template <int VEC, bool DST_TABLE, bool SRC_TABLE>
 __device__ __forceinline__ void tile_copy(uint8_t* __restrict__ dst,
                                           const uint8_t* __restrict__ src,
                                           uint32_t bytes, int j) {
-  using T = typename VecType<VEC>::type;
   const uint32_t units = bytes / VEC;
-  T* d = reinterpret_cast<T*>(dst);
-  const T* s = reinterpret_cast<const T*>(src);
-  uint32_t u = j;
-  /* two units in flight per lane */
-  for (; u + kTile < units; u += 2 * kTile) {
-    T a = s[u];
-    T b = s[u + kTile];
-    d[u] = a;
-    d[u + kTile] = b;
+  if (VEC == 16) {
+    for (uint32_t u = j; u < units; u += 2 * kTile) {
+      const uint32_t u2 = u + kTile;
+      const bool two = u2 < units;
+      uint64_t a0, a1, b0 = 0, b1 = 0;
+      if (SRC_TABLE) {
+        const uint64_t* s = reinterpret_cast<const uint64_t*>(src);
+        a0 = ld_u64(s + 2 * u);
+        a1 = ld_u64(s + 2 * u + 1);
+        if (two) {
+          b0 = ld_u64(s + 2 * u2);
+          b1 = ld_u64(s + 2 * u2 + 1);
+        }
+      } else {
+        const uint4* s = reinterpret_cast<const uint4*>(src);
+        const uint4 a = s[u];
+        a0 = a.x | ((uint64_t)a.y << 32);
+        a1 = a.z | ((uint64_t)a.w << 32);
+        if (two) {
+          const uint4 b = s[u2];
+          b0 = b.x | ((uint64_t)b.y << 32);
+          b1 = b.z | ((uint64_t)b.w << 32);
+        }
+      }
+      if (DST_TABLE) {
+        uint64_t* d = reinterpret_cast<uint64_t*>(dst);
+        st_u64(d + 2 * u, a0);
+        st_u64(d + 2 * u + 1, a1);
+        if (two) {
+          st_u64(d + 2 * u2, b0);
+          st_u64(d + 2 * u2 + 1, b1);
+        }
+      } else {
+        uint4* d = reinterpret_cast<uint4*>(dst);
+        d[u] = make_uint4((uint32_t)a0, (uint32_t)(a0 >> 32), (uint32_t)a1, (uint32_t)(a1 >> 32));
+        if (two)
+          d[u2] = make_uint4((uint32_t)b0, (uint32_t)(b0 >> 32), (uint32_t)b1, (uint32_t)(b1 >> 32));
+      }
+    }
+  } else if (VEC == 4) {
+    const uint32_t* s = reinterpret_cast<const uint32_t*>(src);
+    uint32_t* d = reinterpret_cast<uint32_t*>(dst);
+    for (uint32_t u = j; u < units; u += kTile) {
+      const uint32_t x = SRC_TABLE ? ld_u32(s + u) : s[u];
+      if (DST_TABLE)
+        st_u32(d + u, x);
+      else
+        d[u] = x;
+    }
+  } else {
+    for (uint32_t u = j; u < units; u += kTile) {
+      const uint8_t x = SRC_TABLE ? ld_u8(src + u) : src[u];
+      if (DST_TABLE)
+        st_u8(dst + u, x);
+      else
+        dst[u] = x;
+    }
   }
-  if (u < units) d[u] = s[u];
 }
 
 }  // namespace hkv

@@ -44,7 +44,8 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   const int64_t slot = s_slot[lane];
-  if (slot >= 0 && cas_acquire(v.keys + slot, key, v.reclaim_key)) {
+  uint64_t seen = key;
+  if (slot >= 0 && cas_lock(v.keys + slot, seen, v.reclaim_key)) {
     v.digests[slot] = v.reclaim_digest;
     v.scores[slot] = 0;
     atomicSub(v.sizes + (slot >> 7), 1);
@@ -146,9 +147,7 @@ assign_kernel(View v, AssignArgs a) {
         int ok = 0;
         if (j == 0) {
           uint64_t seen = key;
-          if (__hip_atomic_compare_exchange_strong(
-                  v.keys + slot, &seen, v.locked_key, __ATOMIC_ACQUIRE,
-                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+          if (cas_lock(v.keys + slot, seen, v.locked_key))
             ok = 1;
           else if (seen != v.locked_key)
             ok = -1;
@@ -157,9 +156,10 @@ assign_kernel(View v, AssignArgs a) {
         if (ok > 0) {
           if (a.touch_scores && j == 0) assign_score(v, a, (uint64_t)slot, i);
           if (a.values)
-            tile_copy<VEC>(value_row(v, (uint64_t)slot),
-                           a.values + i * v.value_bytes, v.value_bytes, j);
-          if (j == 0) st_release(v.keys + slot, key);
+            tile_copy<VEC, true, false>(value_row(v, (uint64_t)slot),
+                                        a.values + i * v.value_bytes, v.value_bytes, j);
+          wait_stores();
+          if (j == 0) st_unlock(v.keys + slot, key);
           pending = false;
         } else if (ok < 0) {
           reprobe = true; /* the slot changed hands: look again */

@@ -107,42 +107,49 @@ __device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
   st_u64(v.scores + slot, s);
 }
 
-template <int VEC, int KIND>
+/* dst[e] += delta[e] on a table row, element type by KIND
+ * (accum_or_assign_vector, accum_or_assign.cuh:24-35).  The row is read and
+ * written coherently: another key of the batch may have written it. */
+template <int KIND>
 __device__ __forceinline__ void tile_accum(uint8_t* row, const uint8_t* delta,
                                            uint32_t bytes, int j) {
   if (KIND == HKV_VALUE_F32) {
-    float* d = reinterpret_cast<float*>(row);
+    uint32_t* d = reinterpret_cast<uint32_t*>(row);
     const float* s = reinterpret_cast<const float*>(delta);
-    for (uint32_t e = j; e < bytes / 4; e += kTile) d[e] += s[e];
+    for (uint32_t e = j; e < bytes / 4; e += kTile)
+      st_u32(d + e, __float_as_uint(__uint_as_float(ld_u32(d + e)) + s[e]));
   } else if (KIND == HKV_VALUE_F64) {
-    double* d = reinterpret_cast<double*>(row);
+    uint64_t* d = reinterpret_cast<uint64_t*>(row);
     const double* s = reinterpret_cast<const double*>(delta);
-    for (uint32_t e = j; e < bytes / 8; e += kTile) d[e] += s[e];
+    for (uint32_t e = j; e < bytes / 8; e += kTile)
+      st_u64(d + e, (uint64_t)__double_as_longlong(__longlong_as_double((long long)ld_u64(d + e)) + s[e]));
   } else if (KIND == HKV_VALUE_I32) {
     uint32_t* d = reinterpret_cast<uint32_t*>(row);
     const uint32_t* s = reinterpret_cast<const uint32_t*>(delta);
-    for (uint32_t e = j; e < bytes / 4; e += kTile) d[e] += s[e];
+    for (uint32_t e = j; e < bytes / 4; e += kTile) st_u32(d + e, ld_u32(d + e) + s[e]);
   } else {
     uint64_t* d = reinterpret_cast<uint64_t*>(row);
     const uint64_t* s = reinterpret_cast<const uint64_t*>(delta);
-    for (uint32_t e = j; e < bytes / 8; e += kTile) d[e] += s[e];
+    for (uint32_t e = j; e < bytes / 8; e += kTile) st_u64(d + e, ld_u64(d + e) + s[e]);
   }
 }
 
-/* float rows that allow 16-byte access: 4 adds per 16-byte unit */
+/* float rows that allow 16-byte access on the caller's side: 8 table bytes
+ * (two floats) per coherent access */
 __device__ __forceinline__ void tile_accum_f32x4(uint8_t* row,
                                                  const uint8_t* delta,
                                                  uint32_t bytes, int j) {
-  float4* d = reinterpret_cast<float4*>(row);
+  uint64_t* d = reinterpret_cast<uint64_t*>(row);
   const float4* s = reinterpret_cast<const float4*>(delta);
   for (uint32_t u = j; u < bytes / 16; u += kTile) {
-    float4 x = d[u];
+    const uint64_t lo = ld_u64(d + 2 * u), hi = ld_u64(d + 2 * u + 1);
     const float4 y = s[u];
-    x.x += y.x;
-    x.y += y.y;
-    x.z += y.z;
-    x.w += y.w;
-    d[u] = x;
+    const float x0 = __uint_as_float((uint32_t)lo) + y.x;
+    const float x1 = __uint_as_float((uint32_t)(lo >> 32)) + y.y;
+    const float x2 = __uint_as_float((uint32_t)hi) + y.z;
+    const float x3 = __uint_as_float((uint32_t)(hi >> 32)) + y.w;
+    st_u64(d + 2 * u, __float_as_uint(x0) | ((uint64_t)__float_as_uint(x1) << 32));
+    st_u64(d + 2 * u + 1, __float_as_uint(x2) | ((uint64_t)__float_as_uint(x3) << 32));
   }
 }
 
@@ -221,9 +228,7 @@ upsert_kernel(View v, UpsertArgs a) {
           int ok = 0;
           if (j == 0) {
             uint64_t seen = key;
-            if (__hip_atomic_compare_exchange_strong(
-                    v.keys + hit, &seen, v.locked_key, __ATOMIC_ACQUIRE,
-                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            if (cas_lock(v.keys + hit, seen, v.locked_key))
               ok = 1;
             else if (seen != v.locked_key)
               ok = -1;
@@ -252,7 +257,10 @@ upsert_kernel(View v, UpsertArgs a) {
             const uint32_t eml = tile_bcast(em, tile, jl);
             const uint32_t p = (uint32_t)jl * 16 + bw_to_pos(__ffs(eml) - 1);
             bool ok = false;
-            if (j == 0) ok = cas_acquire(v.keys + bslot + p, v.empty_key, v.locked_key);
+            if (j == 0) {
+              uint64_t seen = v.empty_key;
+              ok = cas_lock(v.keys + bslot + p, seen, v.locked_key);
+            }
             ok = tile_bcast(ok, tile, 0);
             if (j == jl) em &= em - 1;
             if (ok) {
@@ -314,8 +322,9 @@ upsert_kernel(View v, UpsertArgs a) {
                   a.evicted_keys[idx] = key;
                   if (a.evicted_scores) a.evicted_scores[idx] = desired;
                 }
-                tile_copy<VEC>(a.evicted_values + idx * v.value_bytes,
-                               a.values_in + i * v.value_bytes, v.value_bytes, j);
+                tile_copy<VEC, false, false>(a.evicted_values + idx * v.value_bytes,
+                                             a.values_in + i * v.value_bytes,
+                                             v.value_bytes, j);
               }
               if (OP == kOpFindOrInsertPtr && j == 0) {
                 a.out_ptrs[i] = nullptr;
@@ -327,13 +336,14 @@ upsert_kernel(View v, UpsertArgs a) {
               if (j == 0) {
                 uint64_t* kp = v.keys + bslot + bpos;
                 vk = ld_u64(kp);
+                uint64_t seen = vk;
                 if (vk != v.locked_key && vk != v.empty_key &&
-                    cas_acquire(kp, vk, v.locked_key)) {
+                    cas_lock(kp, seen, v.locked_key)) {
                   /* somebody may have raised the score since the scan */
                   if (ld_u64(v.scores + bslot + bpos) <= best)
                     ok = 1;
                   else
-                    st_release(kp, vk);
+                    st_unlock(kp, vk); /* nothing was written under this lock */
                 }
               }
               ok = tile_bcast(ok, tile, 0);
@@ -369,8 +379,8 @@ upsert_kernel(View v, UpsertArgs a) {
                 a.evicted_keys[idx] = victim;
                 if (a.evicted_scores) a.evicted_scores[idx] = min_score;
               }
-              tile_copy<VEC>(a.evicted_values + idx * v.value_bytes, row,
-                             v.value_bytes, j);
+              tile_copy<VEC, false, true>(a.evicted_values + idx * v.value_bytes, row,
+                                          v.value_bytes, j);
             }
             if (j == 0) {
               write_meta(v, a, slot, digest, desired, in_score, i,
@@ -379,13 +389,14 @@ upsert_kernel(View v, UpsertArgs a) {
                 atomicAdd(v.sizes + m.bkt, 1);
             }
             if (OP == kOpInsertOrAssign || OP == kOpInsertAndEvict) {
-              tile_copy<VEC>(row, a.values_in + i * v.value_bytes, v.value_bytes, j);
+              tile_copy<VEC, true, false>(row, a.values_in + i * v.value_bytes,
+                                          v.value_bytes, j);
             } else if (OP == kOpFindOrInsert) {
               uint8_t* user = a.values_io + i * v.value_bytes;
               if (got == kStDuplicate)
-                tile_copy<VEC>(user, row, v.value_bytes, j);
+                tile_copy<VEC, false, true>(user, row, v.value_bytes, j);
               else
-                tile_copy<VEC>(row, user, v.value_bytes, j);
+                tile_copy<VEC, true, false>(row, user, v.value_bytes, j);
             } else if (OP == kOpAccumOrAssign) {
               const uint8_t* user = a.values_in + i * v.value_bytes;
               if (got == kStDuplicate) {
@@ -393,16 +404,16 @@ upsert_kernel(View v, UpsertArgs a) {
                   if (VEC == 16)
                     tile_accum_f32x4(row, user, v.value_bytes, j);
                   else
-                    tile_accum<VEC, HKV_VALUE_F32>(row, user, v.value_bytes, j);
+                    tile_accum<HKV_VALUE_F32>(row, user, v.value_bytes, j);
                 } else if (a.value_kind == HKV_VALUE_F64) {
-                  tile_accum<VEC, HKV_VALUE_F64>(row, user, v.value_bytes, j);
+                  tile_accum<HKV_VALUE_F64>(row, user, v.value_bytes, j);
                 } else if (a.value_kind == HKV_VALUE_I32) {
-                  tile_accum<VEC, HKV_VALUE_I32>(row, user, v.value_bytes, j);
+                  tile_accum<HKV_VALUE_I32>(row, user, v.value_bytes, j);
                 } else {
-                  tile_accum<VEC, HKV_VALUE_I64>(row, user, v.value_bytes, j);
+                  tile_accum<HKV_VALUE_I64>(row, user, v.value_bytes, j);
                 }
               } else {
-                tile_copy<VEC>(row, user, v.value_bytes, j);
+                tile_copy<VEC, true, false>(row, user, v.value_bytes, j);
               }
             } else if (OP == kOpFindOrInsertPtr) {
               if (j == 0) {
@@ -411,7 +422,8 @@ upsert_kernel(View v, UpsertArgs a) {
               }
             }
           }
-          if (j == 0) st_release(v.keys + slot, commit ? key : victim);
+          wait_stores();
+          if (j == 0) st_unlock(v.keys + slot, commit ? key : victim);
           status = got;
         }
       }
