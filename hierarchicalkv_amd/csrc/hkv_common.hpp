@@ -76,6 +76,15 @@ __device__ __forceinline__ uint32_t match16(const uint4& d, uint32_t pat4) {
 __device__ __forceinline__ uint32_t bw_to_pos(uint32_t bit) {
   return ((bit & 7u) << 2) | (bit >> 3);
 }
+/* The same match with bit p set for byte position p (0..15): the four byte
+ * flags of a word are gathered into a nibble by one multiply. */
+__device__ __forceinline__ uint32_t match16_natural(const uint4& d, uint32_t pat4) {
+  const uint32_t n0 = ((zero_bytes(d.x ^ pat4) >> 7) * 0x01020408u) >> 24;
+  const uint32_t n1 = ((zero_bytes(d.y ^ pat4) >> 7) * 0x01020408u) >> 24;
+  const uint32_t n2 = ((zero_bytes(d.z ^ pat4) >> 7) * 0x01020408u) >> 24;
+  const uint32_t n3 = ((zero_bytes(d.w ^ pat4) >> 7) * 0x01020408u) >> 24;
+  return n0 | (n1 << 4) | (n2 << 8) | (n3 << 12);
+}
 
 /* ---- 8-lane tile collectives -------------------------------------------- */
 

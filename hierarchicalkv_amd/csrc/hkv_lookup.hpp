@@ -11,7 +11,7 @@
  *
  * Phases of a wavefront
  *   own    lane L loads key L, hashes it and stages (key, bucket, digest) in LDS;
- *   probe  tile t (8 lanes) probes key r*8+t in round r = 0..7: lane j loads
+ *   probe  tile t (8 lanes) probes key 8t+r in round r = 0..7: lane j loads
  *          16 of the 128 digest bytes, so a tile reads one whole 128-byte line
  *          per round; the 8 rounds are issued back to back so 8 KB of digests
  *          are in flight per wavefront;
@@ -44,8 +44,9 @@ struct FindArgs {
  * Probe the 64 keys staged in s_meta.  On return (after the caller's barrier)
  * s_slot[k] is the table slot of key k or -1.  WRITER selects the writers'
  * probe, which runs while other wavefronts change the table:
- *   - s_emask[r][lane] (when given) receives the lane's mask of EMPTY digests
- *     for round r (bw order);
+ *   - s_em[k][j] (when given) receives lane j's 16-bit mask of EMPTY digests of
+ *     key k's bucket, bit p for byte 16j+p, so the 8 masks of a key read back
+ *     as one 128-bit mask in slot order;
  *   - a candidate slot whose key word reads LOCKED may be this very key under
  *     another tile's lock, so s_unsure[k] is raised and the writer settles the
  *     question with a second, coherent probe of its own (tile_reprobe).
@@ -53,7 +54,7 @@ struct FindArgs {
 template <bool WRITER>
 __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
                                            int64_t* s_slot,
-                                           uint32_t (*s_emask)[kWave],
+                                           uint16_t (*s_em)[kTile],
                                            uint8_t* s_unsure, int lane) {
   const int tile = lane >> 3, j = lane & 7;
   uint4 dg[kTile];
@@ -61,7 +62,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
   uint32_t inf[kTile];
 #pragma unroll
   for (int r = 0; r < kTile; r++) {
-    const KeyMeta m = s_meta[r * kTile + tile];
+    const KeyMeta m = s_meta[tile * kTile + r];
     bkt[r] = m.bkt;
     inf[r] = m.info;
     dg[r] = make_uint4(0, 0, 0, 0);
@@ -75,8 +76,9 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     const bool valid = inf[r] & 0x100u;
     const uint32_t d = inf[r] & 0xFFu;
     cm[r] = valid ? match16(dg[r], d * 0x01010101u) : 0u;
-    if (WRITER && s_emask != nullptr)
-      s_emask[r][lane] = valid ? match16(dg[r], v.empty_digest * 0x01010101u) : 0u;
+    if (WRITER && s_em != nullptr)
+      s_em[tile * kTile + r][j] =
+          (uint16_t)(valid ? match16_natural(dg[r], v.empty_digest * 0x01010101u) : 0u);
     const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
     k0[r] = v.empty_key;
     k1[r] = v.empty_key;
@@ -89,7 +91,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
 #pragma unroll
   for (int r = 0; r < kTile; r++) {
     if (!cm[r]) continue;
-    const int kk = r * kTile + tile;
+    const int kk = tile * kTile + r;
     const uint64_t key = s_meta[kk].key;
     const uint64_t slot0 = (uint64_t)bkt[r] * kBucketSize + j * 16;
     uint32_t m = cm[r];
@@ -118,7 +120,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
  * Second opinion for a writer, by the 8-lane tile that owns the key, with
  * coherent loads: returns the slot of the key, -1 when the key is not in the
  * bucket, or -2 when a digest-matching slot is LOCKED right now (ask again).
- * `em` receives the lane's fresh mask of EMPTY digests.
+ * `em` receives the lane's fresh mask of EMPTY digests (bit p for byte 16j+p).
  */
 __device__ __forceinline__ int64_t tile_reprobe(const View& v, uint64_t key,
                                                 uint32_t bkt, uint32_t digest,
@@ -130,7 +132,7 @@ __device__ __forceinline__ int64_t tile_reprobe(const View& v, uint64_t key,
   d.y = __hip_atomic_load(dp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   d.z = __hip_atomic_load(dp + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   d.w = __hip_atomic_load(dp + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  em = match16(d, v.empty_digest * 0x01010101u);
+  em = match16_natural(d, v.empty_digest * 0x01010101u);
   uint32_t m = match16(d, digest * 0x01010101u);
   const uint64_t slot0 = (uint64_t)bkt * kBucketSize + j * 16;
   int hit = -1;
@@ -207,33 +209,38 @@ lookup_kernel(View v, FindArgs a) {
   }
   if (MODE != kLookupValues) return;
 
-  /* copy stage: 64 rows x units-per-row spread over the 64 lanes */
+  /* copy stage: 64 rows x units-per-row spread over the 64 lanes.  All loads
+   * of a batch are issued before the first store, so a wavefront keeps up to
+   * kBatch KB of value rows in flight (the whole 16 KB for 256-byte rows). */
   using T = typename VecType<VEC>::type;
   const uint32_t units = v.value_bytes / VEC;
   const uint32_t total = units * kWave;
   const bool pow2 = (units & (units - 1)) == 0;
   const uint32_t sh = 31 - __clz(units);
-  constexpr int kBatch = 4;
+  constexpr int kBatch = VEC == 16 ? 16 : 4;
   for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
     T buf[kBatch];
-    T* dst[kBatch];
 #pragma unroll
     for (int b = 0; b < kBatch; b++) {
       const uint32_t idx = idx0 + b * kWave;
-      dst[b] = nullptr;
+      buf[b] = T{};
       if (idx < total) {
         const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
         const uint32_t c = idx - kk * units;
         const int64_t slot = s_slot[kk];
-        if (slot >= 0) {
-          buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)slot))[c];
-          dst[b] = reinterpret_cast<T*>(a.out_values + (base + kk) * v.value_bytes) + c;
-        }
+        if (slot >= 0) buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)slot))[c];
       }
     }
 #pragma unroll
-    for (int b = 0; b < kBatch; b++)
-      if (dst[b]) *dst[b] = buf[b];
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * kWave;
+      if (idx < total) {
+        const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
+        const uint32_t c = idx - kk * units;
+        if (s_slot[kk] >= 0)
+          reinterpret_cast<T*>(a.out_values + (base + kk) * v.value_bytes)[c] = buf[b];
+      }
+    }
   }
 }
 

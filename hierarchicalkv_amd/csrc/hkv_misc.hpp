@@ -1,6 +1,6 @@
 /*
- * Table maintenance kernels: initial fill, clear, erase, size, the assign
- * family (update existing keys only) and the built-in export predicates.
+ * Table maintenance kernels: initial fill, clear, erase, size, and the
+ * built-in export predicates.
  */
 #ifndef HKV_MISC_HPP_
 #define HKV_MISC_HPP_
@@ -60,117 +60,18 @@ size_kernel(View v, unsigned long long* out) {
   for (uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
        b < v.buckets_num; b += stride)
     local += (uint64_t)v.sizes[b];
+  __shared__ unsigned long long s_part[4];
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
-  if ((threadIdx.x & 63) == 0 && local) atomicAdd(out, (unsigned long long)local);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned long long total = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    if (total) atomicAdd(out, total);
+  }
 }
 
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
 __global__ void zero_i32_kernel(int32_t* p) { *p = 0; }
-
-/* ---- assign family: update keys that are present, never insert -------------
- * update kernels (update.cuh, update_score.cuh, update_values.cuh); the score
- * rule is ScoreFunctor::update_without_missed (kernel_utils.cuh:304-321,
- * 373-392, 436-453, 519-557, 594-612).  Several updaters may run at once (the
- * group lock lets them), so the row is changed under the slot lock. */
-
-struct AssignArgs {
-  const uint64_t* keys;
-  const uint8_t* values; /* null: scores only */
-  const uint64_t* scores;
-  uint64_t n;
-  uint64_t epoch;
-  Clock clock;
-  int32_t touch_scores;
-  int32_t strategy;
-};
-
-__device__ __forceinline__ void assign_score(const View& v, const AssignArgs& a,
-                                             uint64_t slot, uint64_t i) {
-  const int STRATEGY = a.strategy;
-  uint64_t s;
-  if (STRATEGY == HKV_LRU) {
-    s = now_ns(a.clock, i);
-  } else if (STRATEGY == HKV_LFU) {
-    if (!a.scores) return;
-    s = ld_u64(v.scores + slot) + a.scores[i];
-  } else if (STRATEGY == HKV_EPOCH_LRU) {
-    s = (a.epoch << 32) | ((now_ns(a.clock, i) >> 20) & kLow32);
-  } else if (STRATEGY == HKV_EPOCH_LFU) {
-    if (!a.scores) return;
-    const uint64_t in = a.scores[i] & kLow32;
-    s = ld_u64(v.scores + slot) & kLow32;
-    if (kLow32 - s > in)
-      s += (a.epoch << 32) | in;
-    else
-      s = (a.epoch << 32) | kLow32;
-  } else {
-    if (!a.scores) return;
-    s = a.scores[i];
-  }
-  st_u64(v.scores + slot, s);
-}
-
-template <int VEC>
-__global__ void __launch_bounds__(kWave)
-assign_kernel(View v, AssignArgs a) {
-  __shared__ KeyMeta s_meta[kWave];
-  __shared__ int64_t s_slot[kWave];
-  __shared__ uint8_t s_unsure[kWave];
-  const int lane = threadIdx.x;
-  const int tile = lane >> 3, j = lane & 7;
-  const uint64_t base = (uint64_t)blockIdx.x * kWave;
-  stage_keys(v, a.keys, a.n, base + lane, s_meta, s_slot, lane);
-  s_unsure[lane] = 0;
-  __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, nullptr, s_unsure, lane);
-  __syncthreads();
-#pragma unroll 1
-  for (int r = 0; r < kTile; r++) {
-    const int kk = r * kTile + tile;
-    const uint64_t i = base + kk;
-    const KeyMeta m = s_meta[kk];
-    const uint64_t key = m.key;
-    int64_t slot = s_slot[kk];
-    bool reprobe = slot < 0 && s_unsure[kk];
-    bool pending = slot >= 0 || reprobe;
-    while (true) {
-      if (pending && reprobe) {
-        uint32_t em_unused;
-        slot = tile_reprobe(v, key, m.bkt, m.info & 0xFFu, tile, j, em_unused);
-        if (slot == -2) {
-          __builtin_amdgcn_s_sleep(2);
-        } else {
-          reprobe = false;
-          pending = slot >= 0;
-        }
-      } else if (pending) {
-        int ok = 0;
-        if (j == 0) {
-          uint64_t seen = key;
-          if (cas_lock(v.keys + slot, seen, v.locked_key))
-            ok = 1;
-          else if (seen != v.locked_key)
-            ok = -1;
-        }
-        ok = tile_bcast(ok, tile, 0);
-        if (ok > 0) {
-          if (a.touch_scores && j == 0) assign_score(v, a, (uint64_t)slot, i);
-          if (a.values)
-            tile_copy<VEC, true, false>(value_row(v, (uint64_t)slot),
-                                        a.values + i * v.value_bytes, v.value_bytes, j);
-          wait_stores();
-          if (j == 0) st_unlock(v.keys + slot, key);
-          pending = false;
-        } else if (ok < 0) {
-          reprobe = true; /* the slot changed hands: look again */
-        } else {
-          __builtin_amdgcn_s_sleep(2);
-        }
-      }
-      if (__ballot(pending) == 0) break;
-    }
-  }
-}
 
 /* ---- built-in predicates (hkv_predicate) -------------------------------------- */
 

@@ -240,15 +240,36 @@ int pick_vec(uint32_t value_bytes, std::initializer_list<const void*> ptrs) {
 
 inline unsigned grid_for(uint64_t n) { return (unsigned)((n + kWave - 1) / kWave); }
 
+/* units per lane that the bulk copy keeps in registers: rows of up to 8 * UPL
+ * units go through in one pass (16-byte units: 128, 256, 512, 1024 bytes) */
+int pick_upl(uint32_t value_bytes, int vec) {
+  if (vec != 16) return 8;
+  const uint32_t units = value_bytes / 16;
+  if (units <= 8) return 1;
+  if (units <= 16) return 2;
+  if (units <= 32) return 4;
+  return 8;
+}
+
 template <int OP, bool LOCKED_RULE>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
-  if (vec == 16)
-    hipLaunchKernelGGL((upsert_kernel<OP, 16, LOCKED_RULE>), grid, block, 0, s, v, a);
-  else if (vec == 4)
-    hipLaunchKernelGGL((upsert_kernel<OP, 4, LOCKED_RULE>), grid, block, 0, s, v, a);
-  else
-    hipLaunchKernelGGL((upsert_kernel<OP, 1, LOCKED_RULE>), grid, block, 0, s, v, a);
+  if (OP == kOpFindOrInsertPtr) {
+    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE>), grid, block, 0, s, v, a);
+    return;
+  }
+  if (vec == 16) {
+    switch (pick_upl(v.value_bytes, 16)) {
+      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE>), grid, block, 0, s, v, a); break;
+      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE>), grid, block, 0, s, v, a); break;
+      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE>), grid, block, 0, s, v, a); break;
+      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE>), grid, block, 0, s, v, a); break;
+    }
+  } else if (vec == 4) {
+    hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+  } else {
+    hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+  }
 }
 
 template <int OP>
@@ -260,10 +281,16 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
-    if (locked_rule)
+    if constexpr (OP == kOpFindOrInsertPtr) {
       launch_upsert<OP, true>(vec, t->view, a, s);
-    else
+    } else if constexpr (OP == kOpInsertOrAssign || OP == kOpFindOrInsert) {
+      if (locked_rule)
+        launch_upsert<OP, true>(vec, t->view, a, s);
+      else
+        launch_upsert<OP, false>(vec, t->view, a, s);
+    } else {
       launch_upsert<OP, false>(vec, t->view, a, s);
+    }
     HKV_HIP(hipGetLastError());
   }
   if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
@@ -650,12 +677,18 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
     LockGuard g(t, StreamGroupLock::kUpdater, s);
     HKV_HIP(g.acquire());
     const dim3 grid(grid_for(n)), block(kWave);
-    if (vec == 16)
-      hipLaunchKernelGGL((assign_kernel<16>), grid, block, 0, s, t->view, a);
-    else if (vec == 4)
-      hipLaunchKernelGGL((assign_kernel<4>), grid, block, 0, s, t->view, a);
-    else
-      hipLaunchKernelGGL((assign_kernel<1>), grid, block, 0, s, t->view, a);
+    if (vec == 16) {
+      switch (pick_upl(t->view.value_bytes, 16)) {
+        case 1: hipLaunchKernelGGL((assign_kernel<16, 1>), grid, block, 0, s, t->view, a); break;
+        case 2: hipLaunchKernelGGL((assign_kernel<16, 2>), grid, block, 0, s, t->view, a); break;
+        case 4: hipLaunchKernelGGL((assign_kernel<16, 4>), grid, block, 0, s, t->view, a); break;
+        default: hipLaunchKernelGGL((assign_kernel<16, 8>), grid, block, 0, s, t->view, a); break;
+      }
+    } else if (vec == 4) {
+      hipLaunchKernelGGL((assign_kernel<4, 8>), grid, block, 0, s, t->view, a);
+    } else {
+      hipLaunchKernelGGL((assign_kernel<1, 8>), grid, block, 0, s, t->view, a);
+    }
     HKV_HIP(hipGetLastError());
   }
   if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;

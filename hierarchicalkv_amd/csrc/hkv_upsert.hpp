@@ -1,31 +1,33 @@
 /*
  * The upsert family: insert_or_assign, insert_and_evict, find_or_insert
- * (values and pointers), accum_or_assign.  One kernel template for every
- * load factor; one 64-lane wavefront per workgroup, 64 keys per wavefront.
+ * (values and pointers), accum_or_assign, and the assign family.  One kernel
+ * template for every load factor; one 64-lane wavefront per workgroup,
+ * 64 keys per wavefront.
  *
  * Replaces tlp_v1/tlp_v2/pipeline_upsert_kernel_with_io (upsert.cuh:27-986),
  * the *_upsert_and_evict_kernel_unique kernels (upsert_and_evict.cuh:27-1099),
  * the find_or_insert kernels (find_or_insert.cuh:27-1050), the pointer kernel
- * (find_ptr_or_insert.cuh:27-246) and accum_or_assign_kernel_with_io
- * (accum_or_assign.cuh:83-174).  Per-key semantics follow upsert.cuh:52-233.
+ * (find_ptr_or_insert.cuh:27-246), accum_or_assign_kernel_with_io
+ * (accum_or_assign.cuh:83-174) and the update kernels (update.cuh,
+ * update_score.cuh, update_values.cuh).  Per-key semantics follow
+ * upsert.cuh:52-233.
  *
- * Phase 1 (batched over the 64 keys): the probe of hkv_lookup.hpp, which also
- *   records where each bucket has EMPTY-looking digests.
- * Phase 2 (8 rounds, one key per 8-lane tile): take the slot lock with a
- *   64-bit CAS on the key word (key -> LOCKED for a hit, EMPTY -> LOCKED for a
- *   free slot, victim -> LOCKED after the min-score scan), write digest and
- *   score, move the value row with the tile, release the key word.
+ * Division of labour inside a wavefront
+ *   control  lane L owns key L: it decides what to lock, issues the 64-bit CAS
+ *            on the key word, writes digest / score, and unlocks.  All 64 keys
+ *            take each of these steps in one instruction, so a wavefront pays
+ *            one memory round trip per step, not one per key.
+ *   bulk     tile t (lanes 8t..8t+7) serves the keys 8t..8t+7 of its own
+ *            lanes: the digest probe (hkv_lookup.hpp), the min-score scan of a
+ *            full bucket (16 scores per lane, 8 coalesced 128-byte lines per
+ *            tile, reduce inside the lane and then over the tile) and the
+ *            value-row copies, each issued for several keys before the first
+ *            result is awaited.
  *
- * The min-score scan reads the bucket's 128 scores as 8 coalesced 128-byte
- * lines per tile (16 scores per lane), reduces inside the lane and then over
- * the 8 lanes; ties go to the lowest slot, as in the reference's sequential
- * scan with a strict '<' (upsert.cuh:166-183).
- *
- * Lock discipline on a SIMD machine: a tile that has taken a lock finishes its
- * critical section in the same trip of the retry loop, and the loop's exit
- * test is a wavefront-wide ballot.  A tile that spins on a slot another tile
- * of the same wavefront holds therefore always finds it released on its next
- * trip.
+ * Lock discipline on a SIMD machine: every lock taken in a trip of the retry
+ * loop is released at the end of the same trip, and the loop's exit test is a
+ * wavefront-wide ballot.  A lane that found a slot LOCKED by another lane of
+ * its wavefront therefore always finds it released on its next trip.
  */
 #ifndef HKV_UPSERT_HPP_
 #define HKV_UPSERT_HPP_
@@ -107,61 +109,314 @@ __device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
   st_u64(v.scores + slot, s);
 }
 
-/* dst[e] += delta[e] on a table row, element type by KIND
- * (accum_or_assign_vector, accum_or_assign.cuh:24-35).  The row is read and
- * written coherently: another key of the batch may have written it. */
-template <int KIND>
-__device__ __forceinline__ void tile_accum(uint8_t* row, const uint8_t* delta,
-                                           uint32_t bytes, int j) {
-  if (KIND == HKV_VALUE_F32) {
-    uint32_t* d = reinterpret_cast<uint32_t*>(row);
-    const float* s = reinterpret_cast<const float*>(delta);
-    for (uint32_t e = j; e < bytes / 4; e += kTile)
-      st_u32(d + e, __float_as_uint(__uint_as_float(ld_u32(d + e)) + s[e]));
-  } else if (KIND == HKV_VALUE_F64) {
-    uint64_t* d = reinterpret_cast<uint64_t*>(row);
-    const double* s = reinterpret_cast<const double*>(delta);
-    for (uint32_t e = j; e < bytes / 8; e += kTile)
-      st_u64(d + e, (uint64_t)__double_as_longlong(__longlong_as_double((long long)ld_u64(d + e)) + s[e]));
-  } else if (KIND == HKV_VALUE_I32) {
-    uint32_t* d = reinterpret_cast<uint32_t*>(row);
-    const uint32_t* s = reinterpret_cast<const uint32_t*>(delta);
-    for (uint32_t e = j; e < bytes / 4; e += kTile) st_u32(d + e, ld_u32(d + e) + s[e]);
+/* x + y on one unit of a row, element type by `kind` (accum_or_assign_vector,
+ * accum_or_assign.cuh:24-35); one IEEE add per element. */
+__device__ __forceinline__ uint4 add_unit(uint4 x, uint4 y, int kind) {
+  if (kind == HKV_VALUE_F32) {
+    x.x = __float_as_uint(__uint_as_float(x.x) + __uint_as_float(y.x));
+    x.y = __float_as_uint(__uint_as_float(x.y) + __uint_as_float(y.y));
+    x.z = __float_as_uint(__uint_as_float(x.z) + __uint_as_float(y.z));
+    x.w = __float_as_uint(__uint_as_float(x.w) + __uint_as_float(y.w));
+  } else if (kind == HKV_VALUE_I32) {
+    x.x += y.x;
+    x.y += y.y;
+    x.z += y.z;
+    x.w += y.w;
   } else {
-    uint64_t* d = reinterpret_cast<uint64_t*>(row);
-    const uint64_t* s = reinterpret_cast<const uint64_t*>(delta);
-    for (uint32_t e = j; e < bytes / 8; e += kTile) st_u64(d + e, ld_u64(d + e) + s[e]);
+    uint64_t a0 = x.x | ((uint64_t)x.y << 32), a1 = x.z | ((uint64_t)x.w << 32);
+    const uint64_t b0 = y.x | ((uint64_t)y.y << 32), b1 = y.z | ((uint64_t)y.w << 32);
+    if (kind == HKV_VALUE_F64) {
+      a0 = (uint64_t)__double_as_longlong(__longlong_as_double((long long)a0) +
+                                          __longlong_as_double((long long)b0));
+      a1 = (uint64_t)__double_as_longlong(__longlong_as_double((long long)a1) +
+                                          __longlong_as_double((long long)b1));
+    } else {
+      a0 += b0;
+      a1 += b1;
+    }
+    x = make_uint4((uint32_t)a0, (uint32_t)(a0 >> 32), (uint32_t)a1, (uint32_t)(a1 >> 32));
   }
+  return x;
+}
+__device__ __forceinline__ uint32_t add_unit(uint32_t x, uint32_t y, int kind) {
+  if (kind == HKV_VALUE_F32) return __float_as_uint(__uint_as_float(x) + __uint_as_float(y));
+  return x + y; /* i32; 8-byte element kinds never take a 4-byte unit (host check) */
+}
+__device__ __forceinline__ uint8_t add_unit(uint8_t x, uint8_t, int) {
+  return x; /* unreachable: arithmetic kinds have 4- or 8-byte elements */
 }
 
-/* float rows that allow 16-byte access on the caller's side: 8 table bytes
- * (two floats) per coherent access */
-__device__ __forceinline__ void tile_accum_f32x4(uint8_t* row,
-                                                 const uint8_t* delta,
-                                                 uint32_t bytes, int j) {
-  uint64_t* d = reinterpret_cast<uint64_t*>(row);
-  const float4* s = reinterpret_cast<const float4*>(delta);
-  for (uint32_t u = j; u < bytes / 16; u += kTile) {
-    const uint64_t lo = ld_u64(d + 2 * u), hi = ld_u64(d + 2 * u + 1);
-    const float4 y = s[u];
-    const float x0 = __uint_as_float((uint32_t)lo) + y.x;
-    const float x1 = __uint_as_float((uint32_t)(lo >> 32)) + y.y;
-    const float x2 = __uint_as_float((uint32_t)hi) + y.z;
-    const float x3 = __uint_as_float((uint32_t)(hi >> 32)) + y.w;
-    st_u64(d + 2 * u, __float_as_uint(x0) | ((uint64_t)__float_as_uint(x1) << 32));
-    st_u64(d + 2 * u + 1, __float_as_uint(x2) | ((uint64_t)__float_as_uint(x3) << 32));
+/* One VEC-byte unit of a row.  Table rows are read and written coherently
+ * (8-, 4- or 1-byte agent-scope accesses), caller buffers plainly. */
+template <int VEC, bool TABLE>
+__device__ __forceinline__ typename VecType<VEC>::type ld_unit(const uint8_t* row, uint32_t u) {
+  using T = typename VecType<VEC>::type;
+  if constexpr (!TABLE) {
+    return reinterpret_cast<const T*>(row)[u];
+  } else if constexpr (VEC == 16) {
+    const uint64_t* p = reinterpret_cast<const uint64_t*>(row) + 2 * u;
+    const uint64_t lo = ld_u64(p), hi = ld_u64(p + 1);
+    return make_uint4((uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32));
+  } else if constexpr (VEC == 4) {
+    return ld_u32(reinterpret_cast<const uint32_t*>(row) + u);
+  } else {
+    return ld_u8(row + u);
+  }
+}
+template <int VEC, bool TABLE>
+__device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecType<VEC>::type x) {
+  using T = typename VecType<VEC>::type;
+  if constexpr (!TABLE) {
+    reinterpret_cast<T*>(row)[u] = x;
+  } else if constexpr (VEC == 16) {
+    uint64_t* p = reinterpret_cast<uint64_t*>(row) + 2 * u;
+    st_u64(p, x.x | ((uint64_t)x.y << 32));
+    st_u64(p + 1, x.z | ((uint64_t)x.w << 32));
+  } else if constexpr (VEC == 4) {
+    st_u32(reinterpret_cast<uint32_t*>(row) + u, x);
+  } else {
+    st_u8(row + u, x);
   }
 }
 
 enum : int {
-  kStInitial = 0,
+  kStNone = 0, /* no lock taken (yet) */
   kStDuplicate = 1,
   kStEmpty = 2,
   kStReclaimed = 3,
   kStEvict = 4,
   kStRefused = 5,
-  kStSkip = 6
+  kStAbsent = 6, /* assign family: key not in the table */
 };
+
+/* what the bulk phase has to move for a key in this trip */
+enum : int {
+  kMoveNone = 0,
+  kMoveInToTable = 1,  /* caller's row -> table row */
+  kMoveTableToIo = 2,  /* table row -> caller's row (find_or_insert hit) */
+  kMoveAccum = 3,      /* table row += caller's row */
+};
+
+/* first set bit of a 128-bit mask at or after bit `s` (wrapping); the mask is
+ * not zero */
+__device__ __forceinline__ uint32_t first_from(uint64_t lo, uint64_t hi, uint32_t s) {
+  if (s & 64) {
+    const uint64_t t = lo;
+    lo = hi;
+    hi = t;
+  }
+  const uint32_t sh = s & 63;
+  uint64_t rlo = lo, rhi = hi;
+  if (sh) {
+    rlo = (lo >> sh) | (hi << (64 - sh));
+    rhi = (hi >> sh) | (lo << (64 - sh));
+  }
+  const uint32_t idx = rlo ? (uint32_t)__ffsll((unsigned long long)rlo) - 1
+                           : 64 + (uint32_t)__ffsll((unsigned long long)rhi) - 1;
+  return (idx + s) & 127u;
+}
+
+/*
+ * Min-score scan of a bucket by the 8 lanes of a tile, split in two so that
+ * the loads of two buckets can be in flight before either is reduced.
+ * Lane j holds scores {16 it + 2j, 16 it + 2j + 1 : it = 0..7}: each `it` is
+ * one coalesced 128-byte line per tile.  LOCKED_RULE hides slots whose key is
+ * LOCKED or EMPTY (find_ptr_or_insert.cuh:170-180).
+ */
+template <bool LOCKED_RULE>
+__device__ __forceinline__ void scan_load(const View& v, uint64_t bslot, int j, uint64_t* sc,
+                                          uint64_t* kc) {
+#pragma unroll
+  for (int it = 0; it < kTile; it++) {
+    const uint64_t* sp = v.scores + bslot + it * 16 + j * 2;
+    sc[2 * it] = ld_u64(sp);
+    sc[2 * it + 1] = ld_u64(sp + 1);
+  }
+  if (LOCKED_RULE) {
+#pragma unroll
+    for (int it = 0; it < kTile; it++) {
+      const uint64_t* kp = v.keys + bslot + it * 16 + j * 2;
+      kc[2 * it] = ld_u64(kp);
+      kc[2 * it + 1] = ld_u64(kp + 1);
+    }
+  }
+}
+/* ties go to the lowest slot, as the reference's sequential scan with a strict
+ * '<' (upsert.cuh:166-183) */
+template <bool LOCKED_RULE>
+__device__ __forceinline__ void scan_reduce(const View& v, const uint64_t* sc, const uint64_t* kc,
+                                            int j, uint64_t& best, uint32_t& bpos) {
+  best = kMaxScore;
+  bpos = 0;
+#pragma unroll
+  for (int q = 0; q < 2 * kTile; q++) {
+    uint64_t s = sc[q];
+    if (LOCKED_RULE && (kc[q] == v.locked_key || kc[q] == v.empty_key)) s = kMaxScore;
+    const uint32_t p = (q >> 1) * 16 + j * 2 + (q & 1);
+    if (s < best) {
+      best = s;
+      bpos = p;
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < kTile; off <<= 1) {
+    const uint64_t ob = __shfl_xor(best, off);
+    const uint32_t op = __shfl_xor(bpos, off);
+    if (ob < best || (ob == best && op < bpos)) {
+      best = ob;
+      bpos = op;
+    }
+  }
+}
+
+/*
+ * Bulk row traffic of one trip.  Round q of a tile is the key owned by lane q
+ * of the tile: `move` says what to do with it, `tab` is its table row, `usr`
+ * the caller's row.  All loads of a group of rounds are issued before the
+ * first store; a group holds 16 units per lane (64 VGPRs at 16-byte units),
+ * i.e. the whole trip for rows up to 256 bytes.
+ * UPL = units per lane and row held in registers (1, 2, 4 or 8).
+ * Every lane of the wavefront must call this.
+ */
+template <int VEC, int UPL, bool CAN_READ_TABLE, bool CAN_ACCUM>
+__device__ __forceinline__ void bulk_rows(int move, uint8_t* tab, uint8_t* usr,
+                                          uint32_t units, int value_kind, int lane) {
+  using T = typename VecType<VEC>::type;
+  constexpr int kGroup = (16 / UPL) < kTile ? (16 / UPL) : kTile;
+  const int j = lane & (kTile - 1);
+  const int lane_base = lane & ~(kTile - 1);
+  for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
+#pragma unroll
+    for (int g = 0; g < kTile; g += kGroup) {
+      T x[kGroup][UPL];
+      T y[CAN_ACCUM ? kGroup : 1][CAN_ACCUM ? UPL : 1];
+#pragma unroll
+      for (int q = 0; q < kGroup; q++) {
+        const int src = lane_base + g + q;
+        const int mv = __shfl(move, src);
+        const uint8_t* tb = reinterpret_cast<const uint8_t*>(__shfl((unsigned long long)tab, src));
+        const uint8_t* us = reinterpret_cast<const uint8_t*>(__shfl((unsigned long long)usr, src));
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = u0 + j + w * kTile;
+          x[q][w] = T{};
+          if (u < units) {
+            if (mv == kMoveInToTable) x[q][w] = ld_unit<VEC, false>(us, u);
+            if (CAN_READ_TABLE && mv == kMoveTableToIo) x[q][w] = ld_unit<VEC, true>(tb, u);
+            if (CAN_ACCUM && mv == kMoveAccum) {
+              x[q][w] = ld_unit<VEC, true>(tb, u);
+              y[q][w] = ld_unit<VEC, false>(us, u);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kGroup; q++) {
+        const int src = lane_base + g + q;
+        const int mv = __shfl(move, src);
+        uint8_t* tb = reinterpret_cast<uint8_t*>(__shfl((unsigned long long)tab, src));
+        uint8_t* us = reinterpret_cast<uint8_t*>(__shfl((unsigned long long)usr, src));
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = u0 + j + w * kTile;
+          if (u < units) {
+            if (mv == kMoveInToTable) st_unit<VEC, true>(tb, u, x[q][w]);
+            if (CAN_READ_TABLE && mv == kMoveTableToIo) st_unit<VEC, false>(us, u, x[q][w]);
+            if (CAN_ACCUM && mv == kMoveAccum)
+              st_unit<VEC, true>(tb, u, add_unit(x[q][w], y[q][w], value_kind));
+          }
+        }
+      }
+    }
+  }
+}
+
+/* Copies towards the evicted-values output: kind 2 = the victim's table row
+ * (coherent read), kind 1 = the refused key's input row, 0 = nothing. */
+template <int VEC, int UPL>
+__device__ __forceinline__ void bulk_evicted(int kind, const uint8_t* src, uint8_t* dst,
+                                             uint32_t units, int lane) {
+  using T = typename VecType<VEC>::type;
+  constexpr int kGroup = (16 / UPL) < kTile ? (16 / UPL) : kTile;
+  const int j = lane & (kTile - 1);
+  const int lane_base = lane & ~(kTile - 1);
+  for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
+#pragma unroll
+    for (int g = 0; g < kTile; g += kGroup) {
+      T x[kGroup][UPL];
+#pragma unroll
+      for (int q = 0; q < kGroup; q++) {
+        const int sl = lane_base + g + q;
+        const int kd = __shfl(kind, sl);
+        const uint8_t* sp = reinterpret_cast<const uint8_t*>(__shfl((unsigned long long)src, sl));
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = u0 + j + w * kTile;
+          x[q][w] = T{};
+          if (u < units) {
+            if (kd == 2) x[q][w] = ld_unit<VEC, true>(sp, u);
+            if (kd == 1) x[q][w] = ld_unit<VEC, false>(sp, u);
+          }
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kGroup; q++) {
+        const int sl = lane_base + g + q;
+        const int kd = __shfl(kind, sl);
+        uint8_t* dp = reinterpret_cast<uint8_t*>(__shfl((unsigned long long)dst, sl));
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = u0 + j + w * kTile;
+          if (u < units && kd) st_unit<VEC, false>(dp, u, x[q][w]);
+        }
+      }
+    }
+  }
+}
+
+/*
+ * Rare path of the writers: lanes whose first probe met a LOCKED candidate, or
+ * whose hit changed hands, get a coherent second probe by their tile.
+ * On return `reprobe` is cleared for every lane whose bucket held no LOCKED
+ * candidate, `hit` is the key's slot or -1, and (em_lo, em_hi) is the fresh
+ * 128-bit mask of EMPTY digests.  Every lane of the wavefront must call this.
+ */
+__device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uint32_t bkt,
+                                                uint32_t digest, bool pending, bool& reprobe,
+                                                int64_t& hit, uint64_t& em_lo, uint64_t& em_hi,
+                                                int lane) {
+  const int tile = lane >> 3, j = lane & 7;
+  const int lane_base = lane & ~(kTile - 1);
+#pragma unroll 1
+  for (int r = 0; r < kTile; r++) {
+    const int src = lane_base + r;
+    if (!__shfl((int)(pending && reprobe), src)) continue; /* tile-uniform */
+    const uint64_t k2 = __shfl((unsigned long long)key, src);
+    const uint32_t b2 = __shfl(bkt, src);
+    const uint32_t d2 = __shfl(digest, src);
+    uint32_t em16 = 0;
+    const int64_t found = tile_reprobe(v, k2, b2, d2, tile, j, em16);
+    uint64_t lo = 0, hi = 0;
+#pragma unroll
+    for (int q = 0; q < kTile; q++) {
+      const uint64_t m = __shfl(em16, lane_base + q) & 0xFFFFu;
+      if (q < 4)
+        lo |= m << (16 * q);
+      else
+        hi |= m << (16 * (q - 4));
+    }
+    if (j == r) {
+      if (found == -2) {
+        __builtin_amdgcn_s_sleep(2);
+      } else {
+        hit = found;
+        reprobe = false;
+        em_lo = lo;
+        em_hi = hi;
+      }
+    }
+  }
+}
 
 /*
  * LOCKED_RULE: behaviour of the lock-key kernels used by the pointer overload
@@ -169,266 +424,313 @@ enum : int {
  * slots whose key is LOCKED or EMPTY are invisible to the victim scan and a
  * key is refused when score <= min instead of score < min.
  */
-template <int OP, int VEC, bool LOCKED_RULE>
+template <int OP, int VEC, int UPL, bool LOCKED_RULE>
 __global__ void __launch_bounds__(kWave)
 upsert_kernel(View v, UpsertArgs a) {
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
-  __shared__ uint64_t s_in_score[kWave];
-  __shared__ uint32_t s_emask[kTile][kWave];
+  __shared__ __attribute__((aligned(16))) uint16_t s_em[kWave][kTile];
   __shared__ uint8_t s_unsure[kWave];
 
   const int lane = threadIdx.x;
   const int tile = lane >> 3, j = lane & 7;
-  const uint64_t base = (uint64_t)blockIdx.x * kWave;
+  const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
+  const uint32_t units = v.value_bytes / VEC;
+
+  const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
+  const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
+  s_unsure[lane] = 0;
+  __syncthreads();
+  probe_wave<true>(v, s_meta, s_slot, s_em, s_unsure, lane);
+  __syncthreads();
+
+  /* ---- state of the key this lane owns ---------------------------------------------- */
+  const KeyMeta me = s_meta[lane];
+  const uint32_t digest = me.info & 0xFFu;
+  const uint32_t start = me.info >> 16;
+  const uint64_t bslot = (uint64_t)me.bkt * kBucketSize;
+  int64_t hit = s_slot[lane];
+  uint64_t em_lo, em_hi;
   {
-    const uint64_t i = base + lane;
-    stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
-    s_in_score[lane] = (a.scores && i < a.n) ? a.scores[i] : 0;
-    s_unsure[lane] = 0;
+    const uint4 e = *reinterpret_cast<const uint4*>(s_em[lane]);
+    em_lo = e.x | ((uint64_t)e.y << 32);
+    em_hi = e.z | ((uint64_t)e.w << 32);
   }
-  __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, s_emask, s_unsure, lane);
-  __syncthreads();
+  bool pending = (me.info & 0x100u) != 0;
+  bool reprobe = pending && hit < 0 && s_unsure[lane];
 
+  /* The trip loop is controlled by a wavefront-uniform value only: all 64
+   * lanes take part in every trip (the tile-cooperative steps read registers
+   * of lanes whose own key is already done), until no lane is pending. */
+  unsigned long long pend_mask = __ballot(pending);
+  while (pend_mask) {
+    if (__ballot(pending && reprobe))
+      settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, lane);
+
+    const bool active = pending && !reprobe;
+    const uint64_t desired = desired_when_missed(a, in_score, i);
+    int got = kStNone;
+    uint32_t pos = 0;
+    uint64_t victim = 0;
+
+    /* ---- step 1: hits and free slots, one CAS per key ------------------------------------ */
+    bool want_scan = false;
+    if (active) {
+      if (hit >= 0) {
+        uint64_t seen = key;
+        if (cas_lock(v.keys + hit, seen, v.locked_key)) {
+          got = kStDuplicate;
+          pos = (uint32_t)(hit - (int64_t)bslot);
+          victim = key;
+        } else if (seen != v.locked_key) {
+          /* the slot belongs to another key now: ours was evicted in this
+           * batch, or the probe was looking at somebody else's lock */
+          hit = -1;
+          reprobe = true;
+        }
+      } else if (em_lo | em_hi) {
+        /* up to three free slots, the first at or after the key's start position
+         * so that keys of one bucket spread over the free slots */
 #pragma unroll 1
-  for (int r = 0; r < kTile; r++) {
-    const int kk = r * kTile + tile;
-    const uint64_t i = base + kk;
-    const KeyMeta m = s_meta[kk];
-    const uint64_t key = m.key;
-    const uint32_t digest = m.info & 0xFFu;
-    const uint32_t start = m.info >> 16;
-    const uint64_t bslot = (uint64_t)m.bkt * kBucketSize;
-    const uint64_t in_score = s_in_score[kk];
-    int64_t hit = s_slot[kk];
-    uint32_t em = s_emask[r][lane];
-    int status = (m.info & 0x100u) ? kStInitial : kStSkip;
-    bool reprobe = hit < 0 && s_unsure[kk];
-
-    while (true) {
-      if (status == kStInitial && reprobe) {
-        const int64_t found = tile_reprobe(v, key, m.bkt, digest, tile, j, em);
-        if (found == -2) {
-          __builtin_amdgcn_s_sleep(2);
-        } else {
-          hit = found;
-          reprobe = false;
-        }
-      } else if (status == kStInitial) {
-        uint64_t desired = desired_when_missed(a, in_score, i);
-        int got = kStInitial;   /* outcome if a lock was taken in this trip */
-        uint32_t pos = 0;
-        uint64_t victim = 0;
-        uint64_t min_score = 0;
-
-        if (hit >= 0) {
-          /* 1 = locked by us, 0 = held by another tile (try again), -1 = the
-           * slot now belongs to another key: ours was evicted in this batch */
-          int ok = 0;
-          if (j == 0) {
-            uint64_t seen = key;
-            if (cas_lock(v.keys + hit, seen, v.locked_key))
-              ok = 1;
-            else if (seen != v.locked_key)
-              ok = -1;
-          }
-          ok = tile_bcast(ok, tile, 0);
-          if (ok > 0) {
-            got = kStDuplicate;
-            pos = (uint32_t)(hit - (int64_t)bslot);
-            victim = key;
-          } else if (ok < 0) {
-            /* the slot belongs to another key now: ours was evicted in this
-             * batch, or the probe was looking at somebody else's lock */
-            hit = -1;
-            reprobe = true;
-          } else {
-            __builtin_amdgcn_s_sleep(2);
-          }
-        } else {
-          const uint32_t lanes = tile_ballot(em != 0, tile);
-          if (lanes) {
-            /* free slot: start with the lane that covers the key's start
-             * position so keys of one bucket spread over the free slots */
-            const int s4 = (int)(start >> 4);
-            const uint32_t rot = ((lanes >> s4) | (lanes << (kTile - s4))) & 0xFFu;
-            const int jl = ((__ffs(rot) - 1) + s4) & 7;
-            const uint32_t eml = tile_bcast(em, tile, jl);
-            const uint32_t p = (uint32_t)jl * 16 + bw_to_pos(__ffs(eml) - 1);
-            bool ok = false;
-            if (j == 0) {
-              uint64_t seen = v.empty_key;
-              ok = cas_lock(v.keys + bslot + p, seen, v.locked_key);
-            }
-            ok = tile_bcast(ok, tile, 0);
-            if (j == jl) em &= em - 1;
-            if (ok) {
-              got = kStEmpty;
-              pos = p;
-              victim = v.empty_key;
-            }
-          } else {
-            /* full bucket: minimum over the 128 scores */
-            uint64_t best = kMaxScore;
-            uint32_t bpos = 0;
-            uint64_t sc[2 * kTile];
-#pragma unroll
-            for (int it = 0; it < kTile; it++) {
-              const uint64_t* sp = v.scores + bslot + it * 16 + j * 2;
-              sc[2 * it] = ld_u64(sp);
-              sc[2 * it + 1] = ld_u64(sp + 1);
-            }
-            if (LOCKED_RULE) {
-#pragma unroll
-              for (int it = 0; it < kTile; it++) {
-                const uint64_t* kp = v.keys + bslot + it * 16 + j * 2;
-                const uint64_t ka = ld_u64(kp), kb = ld_u64(kp + 1);
-                if (ka == v.locked_key || ka == v.empty_key) sc[2 * it] = kMaxScore;
-                if (kb == v.locked_key || kb == v.empty_key) sc[2 * it + 1] = kMaxScore;
-              }
-            }
-#pragma unroll
-            for (int it = 0; it < kTile; it++) {
-              const uint32_t p0 = it * 16 + j * 2;
-              if (sc[2 * it] < best) {
-                best = sc[2 * it];
-                bpos = p0;
-              }
-              if (sc[2 * it + 1] < best) {
-                best = sc[2 * it + 1];
-                bpos = p0 + 1;
-              }
-            }
-#pragma unroll
-            for (int off = 1; off < kTile; off <<= 1) {
-              const uint64_t ob = __shfl_xor(best, off);
-              const uint32_t op = __shfl_xor(bpos, off);
-              if (ob < best || (ob == best && op < bpos)) {
-                best = ob;
-                bpos = op;
-              }
-            }
-            min_score = best;
-            const bool refuse = LOCKED_RULE ? (desired <= best) : (desired < best);
-            if (refuse) {
-              status = kStRefused;
-              if (OP == kOpInsertAndEvict) {
-                /* upsert_and_evict.cuh:188-194, 243-245 */
-                unsigned long long idx = 0;
-                if (j == 0) idx = atomicAdd(a.evicted_counter, 1ull);
-                idx = tile_bcast(idx, tile, 0);
-                if (j == 0) {
-                  a.evicted_keys[idx] = key;
-                  if (a.evicted_scores) a.evicted_scores[idx] = desired;
-                }
-                tile_copy<VEC, false, false>(a.evicted_values + idx * v.value_bytes,
-                                             a.values_in + i * v.value_bytes,
-                                             v.value_bytes, j);
-              }
-              if (OP == kOpFindOrInsertPtr && j == 0) {
-                a.out_ptrs[i] = nullptr;
-                a.founds[i] = 0;
-              }
-            } else {
-              int ok = 0;
-              uint64_t vk = 0;
-              if (j == 0) {
-                uint64_t* kp = v.keys + bslot + bpos;
-                vk = ld_u64(kp);
-                uint64_t seen = vk;
-                if (vk != v.locked_key && vk != v.empty_key &&
-                    cas_lock(kp, seen, v.locked_key)) {
-                  /* somebody may have raised the score since the scan */
-                  if (ld_u64(v.scores + bslot + bpos) <= best)
-                    ok = 1;
-                  else
-                    st_unlock(kp, vk); /* nothing was written under this lock */
-                }
-              }
-              ok = tile_bcast(ok, tile, 0);
-              if (ok) {
-                victim = tile_bcast(vk, tile, 0);
-                got = (victim == v.reclaim_key) ? kStReclaimed : kStEvict;
-                pos = bpos;
-              } else {
-                __builtin_amdgcn_s_sleep(2);
-              }
-            }
+        for (int attempt = 0; attempt < 3 && got == kStNone && (em_lo | em_hi); attempt++) {
+          const uint32_t p = first_from(em_lo, em_hi, start);
+          if (p < 64)
+            em_lo &= ~(UINT64_C(1) << p);
+          else
+            em_hi &= ~(UINT64_C(1) << (p - 64));
+          uint64_t seen = v.empty_key;
+          if (cas_lock(v.keys + bslot + p, seen, v.locked_key)) {
+            got = kStEmpty;
+            pos = p;
+            victim = v.empty_key;
           }
         }
+      } else {
+        want_scan = true;
+      }
+    }
 
-        if (got != kStInitial) {
-          /* critical section: the slot's key word holds LOCKED */
-          const uint64_t slot = bslot + pos;
-          uint8_t* row = value_row(v, slot);
-          bool commit = true;
-          if (OP == kOpAccumOrAssign) {
-            /* accum_or_assign.cuh:139-156: flag and outcome must agree */
-            const bool is_accum = a.accum_flags[i] != 0;
-            commit = is_accum == (got == kStDuplicate);
+    /* ---- step 2: full buckets: min-score scan by the tile, two buckets in flight ------------ */
+    uint64_t best = kMaxScore;
+    uint32_t bpos = 0;
+    {
+      uint32_t need = tile_ballot(want_scan, tile);
+      const int lane_base = lane & ~(kTile - 1);
+      for (unsigned long long more = __ballot(need != 0); more; more = __ballot(need != 0)) {
+        if (need) {
+          const int r0 = __ffs(need) - 1;
+          need &= need - 1;
+          const int r1 = need ? __ffs(need) - 1 : r0;
+          need &= need - 1; /* no-op when need is already 0 */
+          const uint64_t bs0 = __shfl((unsigned long long)bslot, lane_base + r0);
+          const uint64_t bs1 = __shfl((unsigned long long)bslot, lane_base + r1);
+          uint64_t sc0[2 * kTile], sc1[2 * kTile];
+          uint64_t kc0[LOCKED_RULE ? 2 * kTile : 1], kc1[LOCKED_RULE ? 2 * kTile : 1];
+          scan_load<LOCKED_RULE>(v, bs0, j, sc0, kc0);
+          if (r1 != r0) scan_load<LOCKED_RULE>(v, bs1, j, sc1, kc1);
+          uint64_t b0, b1 = kMaxScore;
+          uint32_t p0, p1 = 0;
+          scan_reduce<LOCKED_RULE>(v, sc0, kc0, j, b0, p0);
+          if (r1 != r0) scan_reduce<LOCKED_RULE>(v, sc1, kc1, j, b1, p1);
+          if (j == r0) {
+            best = b0;
+            bpos = p0;
           }
-          if (commit) {
-            if (OP == kOpInsertAndEvict && got == kStEvict) {
-              /* upsert_and_evict.cuh:218-224, 236-238: the old row leaves
-               * before the new one lands */
-              unsigned long long idx = 0;
-              if (j == 0) idx = atomicAdd(a.evicted_counter, 1ull);
-              idx = tile_bcast(idx, tile, 0);
-              if (j == 0) {
-                a.evicted_keys[idx] = victim;
-                if (a.evicted_scores) a.evicted_scores[idx] = min_score;
-              }
-              tile_copy<VEC, false, true>(a.evicted_values + idx * v.value_bytes, row,
-                                          v.value_bytes, j);
-            }
-            if (j == 0) {
-              write_meta(v, a, slot, digest, desired, in_score, i,
-                                   got != kStDuplicate);
-              if (got == kStEmpty || got == kStReclaimed)
-                atomicAdd(v.sizes + m.bkt, 1);
-            }
-            if (OP == kOpInsertOrAssign || OP == kOpInsertAndEvict) {
-              tile_copy<VEC, true, false>(row, a.values_in + i * v.value_bytes,
-                                          v.value_bytes, j);
-            } else if (OP == kOpFindOrInsert) {
-              uint8_t* user = a.values_io + i * v.value_bytes;
-              if (got == kStDuplicate)
-                tile_copy<VEC, false, true>(user, row, v.value_bytes, j);
-              else
-                tile_copy<VEC, true, false>(row, user, v.value_bytes, j);
-            } else if (OP == kOpAccumOrAssign) {
-              const uint8_t* user = a.values_in + i * v.value_bytes;
-              if (got == kStDuplicate) {
-                if (a.value_kind == HKV_VALUE_F32) {
-                  if (VEC == 16)
-                    tile_accum_f32x4(row, user, v.value_bytes, j);
-                  else
-                    tile_accum<HKV_VALUE_F32>(row, user, v.value_bytes, j);
-                } else if (a.value_kind == HKV_VALUE_F64) {
-                  tile_accum<HKV_VALUE_F64>(row, user, v.value_bytes, j);
-                } else if (a.value_kind == HKV_VALUE_I32) {
-                  tile_accum<HKV_VALUE_I32>(row, user, v.value_bytes, j);
-                } else {
-                  tile_accum<HKV_VALUE_I64>(row, user, v.value_bytes, j);
-                }
-              } else {
-                tile_copy<VEC, true, false>(row, user, v.value_bytes, j);
-              }
-            } else if (OP == kOpFindOrInsertPtr) {
-              if (j == 0) {
-                a.out_ptrs[i] = row;
-                a.founds[i] = got == kStDuplicate;
-              }
-            }
+          if (r1 != r0 && j == r1) {
+            best = b1;
+            bpos = p1;
           }
-          wait_stores();
-          if (j == 0) st_unlock(v.keys + slot, commit ? key : victim);
-          status = got;
         }
       }
-      if (__ballot(status == kStInitial) == 0) break;
     }
+
+    /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
+    bool refused_now = false;
+    if (want_scan) {
+      const bool refuse = LOCKED_RULE ? (desired <= best) : (desired < best);
+      if (refuse) {
+        refused_now = true;
+        got = kStRefused;
+      } else {
+        uint64_t* kp = v.keys + bslot + bpos;
+        const uint64_t vk = ld_u64(kp);
+        uint64_t seen = vk;
+        if (vk != v.locked_key && vk != v.empty_key && cas_lock(kp, seen, v.locked_key)) {
+          /* somebody may have raised the score since the scan */
+          if (ld_u64(v.scores + bslot + bpos) <= best) {
+            victim = vk;
+            got = (vk == v.reclaim_key) ? kStReclaimed : kStEvict;
+            pos = bpos;
+          } else {
+            st_unlock(kp, vk); /* nothing was written under this lock */
+          }
+        }
+      }
+    }
+
+    /* ---- step 4: critical sections of every lock taken in this trip ------------------------------ */
+    const bool locked = got != kStNone && got != kStRefused;
+    const uint64_t slot = bslot + pos;
+    uint8_t* row = value_row(v, slot);
+    bool commit = locked;
+    if (OP == kOpAccumOrAssign && locked) {
+      /* accum_or_assign.cuh:139-156: flag and outcome must agree */
+      const bool is_accum = a.accum_flags[i] != 0;
+      commit = is_accum == (got == kStDuplicate);
+    }
+
+    if (OP == kOpInsertAndEvict) {
+      /* upsert_and_evict.cuh:188-194, 218-224, 236-245: an evicted key leaves with
+       * its old row and the scanned minimum, a refused key with its input; one
+       * counter update per wavefront */
+      const bool emit = refused_now || (commit && got == kStEvict);
+      const unsigned long long votes = __ballot(emit);
+      if (votes) {
+        const int leader = (int)__ffsll(votes) - 1;
+        unsigned long long base_idx = 0;
+        if (lane == leader)
+          base_idx = atomicAdd(a.evicted_counter, (unsigned long long)__popcll(votes));
+        base_idx = __shfl(base_idx, leader);
+        const unsigned long long idx = base_idx + __popcll(votes & ((1ull << lane) - 1));
+        if (emit) {
+          a.evicted_keys[idx] = refused_now ? key : victim;
+          if (a.evicted_scores) a.evicted_scores[idx] = refused_now ? desired : best;
+        }
+        bulk_evicted<VEC, UPL>(emit ? (refused_now ? 1 : 2) : 0,
+                               refused_now ? a.values_in + i * v.value_bytes : row,
+                               a.evicted_values + idx * v.value_bytes, units, lane);
+      }
+    }
+    if (OP == kOpFindOrInsertPtr && (locked || refused_now)) {
+      a.out_ptrs[i] = locked ? row : nullptr;
+      a.founds[i] = got == kStDuplicate;
+    }
+    if (commit) {
+      write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
+      if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
+    }
+    if (OP != kOpFindOrInsertPtr) {
+      int move = kMoveNone;
+      uint8_t* usr = nullptr;
+      if (commit) {
+        if (OP == kOpInsertOrAssign || OP == kOpInsertAndEvict) {
+          move = kMoveInToTable;
+          usr = const_cast<uint8_t*>(a.values_in) + i * v.value_bytes;
+        } else if (OP == kOpFindOrInsert) {
+          move = got == kStDuplicate ? kMoveTableToIo : kMoveInToTable;
+          usr = a.values_io + i * v.value_bytes;
+        } else if (OP == kOpAccumOrAssign) {
+          move = got == kStDuplicate ? kMoveAccum : kMoveInToTable;
+          usr = const_cast<uint8_t*>(a.values_in) + i * v.value_bytes;
+        }
+      }
+      if (__ballot(move != kMoveNone))
+        bulk_rows<VEC, UPL, OP == kOpFindOrInsert, OP == kOpAccumOrAssign>(
+            move, row, usr, units, a.value_kind, lane);
+    }
+
+    /* ---- step 5: everything written under the locks is out; release them --------------------------- */
+    wait_stores();
+    if (locked) st_unlock(v.keys + slot, commit ? key : victim);
+    if (got != kStNone) pending = false;
+    pend_mask = __ballot(pending);
+    if (pend_mask) __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+/* ---- assign family: update keys that are present, never insert -----------------
+ * The score rule is ScoreFunctor::update_without_missed (kernel_utils.cuh:
+ * 304-321, 373-392, 436-453, 519-557, 594-612).  Several updaters may run at
+ * once (the group lock lets them), so the row changes under the slot lock. */
+
+struct AssignArgs {
+  const uint64_t* keys;
+  const uint8_t* values; /* null: scores only */
+  const uint64_t* scores;
+  uint64_t n;
+  uint64_t epoch;
+  Clock clock;
+  int32_t touch_scores;
+  int32_t strategy;
+};
+
+__device__ __forceinline__ void assign_score(const View& v, const AssignArgs& a,
+                                             uint64_t slot, uint64_t i) {
+  const int STRATEGY = a.strategy;
+  uint64_t s;
+  if (STRATEGY == HKV_LRU) {
+    s = now_ns(a.clock, i);
+  } else if (STRATEGY == HKV_LFU) {
+    if (!a.scores) return;
+    s = ld_u64(v.scores + slot) + a.scores[i];
+  } else if (STRATEGY == HKV_EPOCH_LRU) {
+    s = (a.epoch << 32) | ((now_ns(a.clock, i) >> 20) & kLow32);
+  } else if (STRATEGY == HKV_EPOCH_LFU) {
+    if (!a.scores) return;
+    const uint64_t in = a.scores[i] & kLow32;
+    s = ld_u64(v.scores + slot) & kLow32;
+    if (kLow32 - s > in)
+      s += (a.epoch << 32) | in;
+    else
+      s = (a.epoch << 32) | kLow32;
+  } else {
+    if (!a.scores) return;
+    s = a.scores[i];
+  }
+  st_u64(v.scores + slot, s);
+}
+
+template <int VEC, int UPL>
+__global__ void __launch_bounds__(kWave)
+assign_kernel(View v, AssignArgs a) {
+  __shared__ KeyMeta s_meta[kWave];
+  __shared__ int64_t s_slot[kWave];
+  __shared__ uint8_t s_unsure[kWave];
+  const int lane = threadIdx.x;
+  const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
+  const uint32_t units = v.value_bytes / VEC;
+  const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
+  s_unsure[lane] = 0;
+  __syncthreads();
+  probe_wave<true>(v, s_meta, s_slot, nullptr, s_unsure, lane);
+  __syncthreads();
+  const KeyMeta me = s_meta[lane];
+  int64_t hit = s_slot[lane];
+  bool reprobe = hit < 0 && s_unsure[lane];
+  bool pending = (me.info & 0x100u) && (hit >= 0 || reprobe);
+  uint64_t em_lo = 0, em_hi = 0;
+  unsigned long long pend_mask = __ballot(pending);
+  while (pend_mask) {
+    if (__ballot(pending && reprobe))
+      settle_reprobes(v, key, me.bkt, me.info & 0xFFu, pending, reprobe, hit, em_lo, em_hi, lane);
+    int got = kStNone;
+    if (pending && !reprobe) {
+      if (hit < 0) {
+        got = kStAbsent;
+      } else {
+        uint64_t seen = key;
+        if (cas_lock(v.keys + hit, seen, v.locked_key)) {
+          got = kStDuplicate;
+        } else if (seen != v.locked_key) {
+          hit = -1;
+          reprobe = true; /* the slot changed hands: look again */
+        }
+      }
+    }
+    const bool locked = got == kStDuplicate;
+    uint8_t* row = value_row(v, (uint64_t)(hit < 0 ? 0 : hit));
+    if (locked && a.touch_scores) assign_score(v, a, (uint64_t)hit, i);
+    if (a.values) {
+      const int move = locked ? kMoveInToTable : kMoveNone;
+      uint8_t* usr = const_cast<uint8_t*>(a.values) + i * v.value_bytes;
+      if (__ballot(move != kMoveNone))
+        bulk_rows<VEC, UPL, false, false>(move, row, usr, units, 0, lane);
+    }
+    wait_stores();
+    if (locked) st_unlock(v.keys + hit, key);
+    if (got != kStNone) pending = false;
+    pend_mask = __ballot(pending);
+    if (pend_mask) __builtin_amdgcn_s_sleep(1);
   }
 }
 
