@@ -8,6 +8,11 @@ keys (100 % hits) followed by insert_or_assign of 2^20 keys, half resident and
 half new (every new key evicts the bucket's minimum).  Inputs and outputs are
 resident in HBM when the timed region starts.
 
+The resident keys of a step come from old pre-fill batches, a different batch
+per step, so their rows are neither in the L2s nor in the 256 MB Infinity Cache
+when the step touches them (--warm-keys takes them from the previous step's
+insert instead, as the reference's benchmark does).
+
 Prints one JSON line: whole-step throughput in 10^9 KV/s, per-op figures, the
 HBM roofline of each kernel from HIP-event timings inside the timed region, and
 a CPU baseline (the multithreaded host oracle on a bounded sample).
@@ -44,6 +49,11 @@ def main():
     ap.add_argument("--dim", type=int, default=64)
     ap.add_argument("--batch-log2", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--warm-keys", action="store_true",
+                    help="resident keys of a step = keys written by the previous step")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference point for "
+                         "FETCH_SIZE / WRITE_SIZE when profiling)")
     ap.add_argument("--cpu-capacity-log2", type=int, default=24)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -81,6 +91,7 @@ def main():
     pos = 0
     vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
     size0 = 0
+    prefill_starts = []
     # uniform hashing fills the last slots slowly: keep inserting (the fullest
     # buckets evict meanwhile) until 99.9 % of the slots hold a key
     while size0 < 0.999 * cap and pos < 3 * cap:
@@ -88,6 +99,7 @@ def main():
             keys = w.unique_keys(seed, pos, n)
             vals.uniform_(-1.0, 1.0)
             table.insert_or_assign(n, d64(keys), vals)
+            prefill_starts.append(pos)
             pos += n
         size0 = table.size()
     prefill_s = time.time() - t0
@@ -96,15 +108,31 @@ def main():
     # step s: find the keys inserted by step s-1 (all resident, highest LRU scores);
     #         insert_or_assign half of those again + as many never-seen keys.
     steps = K + W
-    prev = w.unique_keys(seed, pos - n, n)  # last prefill batch
+    nb = len(prefill_starts)
     find_keys, ins_keys = [], []
-    for s in range(steps):
-        find_keys.append(d64(prev))
-        fresh = w.unique_keys(seed, pos, n // 2)
-        pos += n // 2
-        batch = np.concatenate([prev[: n // 2], fresh])
-        ins_keys.append(d64(batch))
-        prev = batch
+    if args.warm_keys:
+        # step s: find the keys inserted by step s-1; insert half of them again
+        prev = w.unique_keys(seed, pos - n, n)
+        for s in range(steps):
+            find_keys.append(d64(prev))
+            fresh = w.unique_keys(seed, pos, n // 2)
+            pos += n // 2
+            batch = np.concatenate([prev[: n // 2], fresh])
+            ins_keys.append(d64(batch))
+            prev = batch
+    else:
+        # A bucket holds the newest 128 of the ~2 keys per batch it received, i.e.
+        # the last ~64 pre-fill batches, and loses about one key per step.  Batches
+        # 9..(9+steps) from the end serve find, half batches further back serve the
+        # resident half of insert_or_assign; all stay resident for the whole run.
+        assert steps <= 26 and nb >= 9 + steps + (steps + 1) // 2 + 2, "too many steps for cold keys"
+        for s in range(steps):
+            find_keys.append(d64(w.unique_keys(seed, prefill_starts[nb - 9 - s], n)))
+            old = w.unique_keys(seed, prefill_starts[nb - 10 - steps - s // 2], n)
+            half = old[: n // 2] if s % 2 == 0 else old[n // 2:]
+            fresh = w.unique_keys(seed, pos, n // 2)
+            pos += n // 2
+            ins_keys.append(d64(np.concatenate([half, fresh])))
     ins_vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
     out_vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
     founds = torch.empty(n, dtype=torch.bool, device=dev)
@@ -118,6 +146,13 @@ def main():
         table.insert_or_assign(n, ins_keys[s], ins_vals)
         ev[s][2].record()
 
+    if args.calibrate:
+        cal = torch.empty(2, 1 << 28, dtype=torch.float32, device=dev)
+        cal[0].fill_(1.0)
+        torch.cuda.synchronize()
+        cal[1].copy_(cal[0])  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del cal
     for s in range(W):
         step(s)
     torch.cuda.synchronize()
@@ -161,6 +196,7 @@ def main():
             "size_before": size0,
             "size_after": size1,
             "prefill_s": round(prefill_s, 1),
+            "resident_keys": "warm (previous step)" if args.warm_keys else "cold (old pre-fill batches)",
         },
         "find": {"ms": round(find_avg, 4), "bkvs": round(n / (find_avg * 1e-3) / 1e9, 4),
                  "bkvs_2p30": round(n / (find_avg * 1e-3) / 2**30, 4)},

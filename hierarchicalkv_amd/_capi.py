@@ -8,7 +8,7 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libhkv.so")
+LIB_PATH = os.environ.get("HKV_LIB_PATH") or os.path.join(_PKG, "libhkv.so")
 
 HKV_SUCCESS = 0
 HKV_ERROR_CHECK = 1

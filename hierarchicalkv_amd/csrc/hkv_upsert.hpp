@@ -147,7 +147,8 @@ __device__ __forceinline__ uint8_t add_unit(uint8_t x, uint8_t, int) {
 }
 
 /* One VEC-byte unit of a row.  Table rows are read and written coherently
- * (8-, 4- or 1-byte agent-scope accesses), caller buffers plainly. */
+ * (agent-scope accesses: 2 x 8 bytes per 16-byte unit on the load side, one
+ * 16-byte write-through store on the store side), caller buffers plainly. */
 template <int VEC, bool TABLE>
 __device__ __forceinline__ typename VecType<VEC>::type ld_unit(const uint8_t* row, uint32_t u) {
   using T = typename VecType<VEC>::type;
@@ -169,15 +170,21 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
   if constexpr (!TABLE) {
     reinterpret_cast<T*>(row)[u] = x;
   } else if constexpr (VEC == 16) {
-    uint64_t* p = reinterpret_cast<uint64_t*>(row) + 2 * u;
-    st_u64(p, x.x | ((uint64_t)x.y << 32));
-    st_u64(p + 1, x.z | ((uint64_t)x.w << 32));
+    st_u128(row + 16 * (size_t)u, x);
   } else if constexpr (VEC == 4) {
     st_u32(reinterpret_cast<uint32_t*>(row) + u, x);
   } else {
     st_u8(row + u, x);
   }
 }
+
+#ifndef HKV_SCAN_PAIR
+#define HKV_SCAN_PAIR 1
+#endif
+#ifndef HKV_UPSERT_MIN_WAVES
+#define HKV_UPSERT_MIN_WAVES 1
+#endif
+constexpr bool kScanPair = HKV_SCAN_PAIR;
 
 enum : int {
   kStNone = 0, /* no lock taken (yet) */
@@ -425,7 +432,7 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * key is refused when score <= min instead of score < min.
  */
 template <int OP, int VEC, int UPL, bool LOCKED_RULE>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kWave, HKV_UPSERT_MIN_WAVES)
 upsert_kernel(View v, UpsertArgs a) {
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
@@ -520,8 +527,8 @@ upsert_kernel(View v, UpsertArgs a) {
         if (need) {
           const int r0 = __ffs(need) - 1;
           need &= need - 1;
-          const int r1 = need ? __ffs(need) - 1 : r0;
-          need &= need - 1; /* no-op when need is already 0 */
+          const int r1 = (kScanPair && need) ? __ffs(need) - 1 : r0;
+          if (kScanPair) need &= need - 1; /* no-op when need is already 0 */
           const uint64_t bs0 = __shfl((unsigned long long)bslot, lane_base + r0);
           const uint64_t bs1 = __shfl((unsigned long long)bslot, lane_base + r1);
           uint64_t sc0[2 * kTile], sc1[2 * kTile];
