@@ -941,6 +941,17 @@ int hkv_lock_end(const hkv_table* t, int role, hkv_stream_t stream) {
   return HKV_SUCCESS;
 }
 
+#ifdef HKV_STATS
+/* tuning builds only: read and clear the event counters */
+int hkv_debug_stats(uint64_t* out16) {
+  HKV_HIP(hipDeviceSynchronize());
+  HKV_HIP(hipMemcpyFromSymbol(out16, HIP_SYMBOL(g_hkv_stats), 16 * sizeof(uint64_t)));
+  uint64_t z[16] = {0};
+  HKV_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_hkv_stats), z, sizeof z));
+  return HKV_SUCCESS;
+}
+#endif
+
 int hkv_set_clock(hkv_table* t, int mode, uint64_t base) {
   if (mode != 0 && mode != 1) return fail(HKV_ERROR_ARGUMENT, "bad clock mode %d", mode);
   t->clock.mode = (uint32_t)mode;

@@ -178,6 +178,15 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
   }
 }
 
+/* Optional event counters for tuning builds (-DHKV_STATS): trips of the retry
+ * loop, scans, failed lock attempts.  Not compiled into the shipped library. */
+#ifdef HKV_STATS
+__device__ unsigned long long g_hkv_stats[16];
+#define HKV_COUNT(slot, n) atomicAdd(&g_hkv_stats[slot], (unsigned long long)(n))
+#else
+#define HKV_COUNT(slot, n) ((void)0)
+#endif
+
 #ifndef HKV_SCAN_PAIR
 #define HKV_SCAN_PAIR 1
 #endif
@@ -477,6 +486,11 @@ upsert_kernel(View v, UpsertArgs a) {
     const bool active = pending && !reprobe;
     const uint64_t desired = desired_when_missed(a, in_score, i);
     int got = kStNone;
+    if (lane == 0) {
+      HKV_COUNT(0, 1);                                   /* trips */
+      HKV_COUNT(1, __popcll(pend_mask));                 /* pending keys over trips */
+      HKV_COUNT(2, __popcll(__ballot(pending && reprobe))); /* unsettled reprobes */
+    }
     uint32_t pos = 0;
     uint64_t victim = 0;
 
@@ -494,6 +508,9 @@ upsert_kernel(View v, UpsertArgs a) {
            * batch, or the probe was looking at somebody else's lock */
           hit = -1;
           reprobe = true;
+          HKV_COUNT(3, 1);
+        } else {
+          HKV_COUNT(4, 1); /* hit slot locked by somebody else */
         }
       } else if (em_lo | em_hi) {
         /* up to three free slots, the first at or after the key's start position
@@ -510,10 +527,13 @@ upsert_kernel(View v, UpsertArgs a) {
             got = kStEmpty;
             pos = p;
             victim = v.empty_key;
+          } else {
+            HKV_COUNT(5, 1); /* lost a free slot */
           }
         }
       } else {
         want_scan = true;
+        HKV_COUNT(6, 1); /* scans */
       }
     }
 
@@ -570,7 +590,10 @@ upsert_kernel(View v, UpsertArgs a) {
             pos = bpos;
           } else {
             st_unlock(kp, vk); /* nothing was written under this lock */
+            HKV_COUNT(7, 1); /* score was raised between scan and lock */
           }
+        } else {
+          HKV_COUNT(8, 1); /* victim locked or taken by somebody else */
         }
       }
     }
