@@ -38,6 +38,21 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+def build_cpp_tests(verbose=True):
+    """The C++ test of the drop-in header (tests/cpp/api_test.cpp), linked
+    against the in-tree library; a GPU test runs the binary."""
+    src = os.path.join(ROOT, "tests", "cpp", "api_test.cpp")
+    out = os.path.join(ROOT, "tests", "cpp", "api_test")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", INCLUDE, src, "-L", PKG_DIR, "-lhkv",
+           "-Wl,-rpath,$ORIGIN/../../hierarchicalkv_amd", "-o", out]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
+
+
 def build_oracle(verbose=True):
     cmd = ["make", "-C", ORACLE_DIR, "-B", "libhkv_oracle.so"]
     if verbose:
@@ -47,8 +62,10 @@ def build_oracle(verbose=True):
 
 
 if __name__ == "__main__":
-    what = sys.argv[1:] or ["lib", "oracle"]
+    what = sys.argv[1:] or ["lib", "oracle", "cpp"]
     if "lib" in what:
         build_library()
+    if "cpp" in what:
+        build_cpp_tests()
     if "oracle" in what:
         build_oracle()

@@ -361,6 +361,12 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
                 "initial required buckets number");
   if (o->max_bucket_size != kBucketSize)
     return fail(HKV_ERROR_UNSUPPORTED, "only max_bucket_size == 128 is supported");
+  /* a table with init_capacity * 2 <= max_capacity grows by rehashing in the
+   * reference (merlin_hashtable.cuh:1151-1154); refuse rather than never grow */
+  if (o->init_capacity * 2 <= std::max(o->init_capacity, o->max_capacity))
+    return fail(HKV_ERROR_UNSUPPORTED,
+                "growable tables (init_capacity * 2 <= max_capacity) need rehash, "
+                "which is not supported: set init_capacity == max_capacity");
   if (o->io_by_cpu && o->max_hbm_for_vectors != 0)
     return fail(HKV_ERROR_CHECK,
                 "[HierarchicalKV] `io_by_cpu` should not be true when "

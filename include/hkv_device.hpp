@@ -149,5 +149,38 @@ size_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern,
   if (lane == 0 && local) atomicAdd(counter, (unsigned long long)local);
 }
 
+/* erase_if: tombstone every entry the predicate selects (the predicate form of
+ * remove_kernel, core_kernels.cuh:744-843).  Runs under the inserter role, so
+ * no other kernel touches the table meanwhile. */
+template <class Pred>
+__global__ void __launch_bounds__(256)
+erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshold,
+                unsigned long long* counter) {
+  const int lane = lane_id();
+  uint64_t local = 0;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t s = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+       s < v.capacity; s += stride) {
+    uint64_t key = v.keys[s];
+    uint64_t score = v.scores[s];
+    if (!is_reserved_key(v, key) && pred(key, score, pattern, threshold)) {
+      v.keys[s] = v.reclaim_key;
+      v.digests[s] = v.reclaim_digest;
+      v.scores[s] = 0;
+      atomicSub(v.sizes + (s >> 7), 1);
+      local++;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
+  if (lane == 0 && local) atomicAdd(counter, (unsigned long long)local);
+}
+
+/* One-word clear as a kernel: callers may be capturing a graph, where memset
+ * nodes are best avoided. */
+template <class T>
+__global__ void zero_word_kernel(T* p) {
+  *p = T(0);
+}
+
 }  // namespace hkv
 #endif

@@ -1,0 +1,817 @@
+/*
+ * Source-level drop-in for the reference's public header
+ * (include/merlin_hashtable.cuh): the same namespace, class names, method
+ * names, parameter order and defaults, with hipStream_t where the reference
+ * has cudaStream_t.  Every method forwards to one entry point of the C ABI
+ * (include/hkv_c_api.h) of libhkv.so; only the predicate templates
+ * (export_batch_if, size_if, erase_if) instantiate a kernel in the caller's
+ * translation unit, against the table layout of hkv_table_get_view().
+ *
+ * Compile with hipcc for gfx950 and link with -lhkv.
+ *
+ * Reference lines mirrored here:
+ *   EvictStrategy ........ merlin_hashtable.cuh:79-87
+ *   TableMode ............ merlin_hashtable.cuh:95-98
+ *   HashTableOptions ..... merlin_hashtable.cuh:103-136
+ *   HashTableBase ........ merlin_hashtable.cuh:187-885
+ *   HashTable ............ merlin_hashtable.cuh:910-3892
+ *   MemoryType, BaseAllocator, DefaultAllocator .. merlin/allocator.cuh:27-125
+ *   BaseKVFile ........... merlin/types.cuh:242-281
+ *   exceptions, checks ... merlin/debug.hpp:27-72
+ *   GB / MB / KB ......... merlin/utils.cuh:338-342
+ *
+ * Not provided (outside this build's scope, the call throws
+ * std::runtime_error): reserve() to a larger capacity and automatic growth,
+ * lock_keys / unlock_keys, find_and_update, the *_v2 predicate forms and
+ * for_each, TableMode::kMemory, S = uint32_t.
+ */
+#ifndef MERLIN_HASHTABLE_HPP_
+#define MERLIN_HASHTABLE_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdint>
+#include <cstdlib>
+#include <limits>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "hkv_c_api.h"
+#include "hkv_device.hpp"
+
+namespace nv {
+namespace merlin {
+
+/* ---- merlin/debug.hpp ------------------------------------------------------- */
+
+class CudaException : public std::runtime_error {
+ public:
+  CudaException(const std::string& what) : runtime_error(what) {}
+};
+
+class MerlinException : public std::runtime_error {
+ public:
+  MerlinException(const std::string& what) : runtime_error(what) {}
+};
+
+inline void hip_check_(hipError_t val, const char* file, int line) {
+  if (val != hipSuccess) {
+    std::ostringstream os;
+    os << file << ':' << line << ": HIP error " << hipGetErrorName(val) << " (#" << val
+       << "): " << hipGetErrorString(val);
+    throw CudaException(os.str());
+  }
+}
+#define HKV_HIP_CHECK(val) ::nv::merlin::hip_check_((val), __FILE__, __LINE__)
+
+template <class Msg>
+inline void merlin_check_(bool cond, const Msg& msg, const char* file, int line) {
+  if (!cond) {
+    std::ostringstream os;
+    os << file << ':' << line << ": HierarchicalKV error " << msg;
+    throw MerlinException(os.str());
+  }
+}
+#ifndef MERLIN_CHECK
+#define MERLIN_CHECK(cond, msg) ::nv::merlin::merlin_check_((cond), (msg), __FILE__, __LINE__)
+#endif
+
+/* status of a C ABI call -> the exception the reference would have thrown */
+inline void throw_on_error_(int rc) {
+  if (rc == HKV_SUCCESS) return;
+  const std::string msg = hkv_last_error();
+  switch (rc) {
+    case HKV_ERROR_CHECK:
+      throw MerlinException(msg);
+    case HKV_ERROR_HIP:
+      throw CudaException(msg);
+    case HKV_ERROR_ARGUMENT:
+      throw std::invalid_argument(msg);
+    default:
+      throw std::runtime_error(msg);
+  }
+}
+
+/* ---- merlin/utils.cuh --------------------------------------------------------- */
+
+static inline size_t GB(size_t n) { return n << 30; }
+static inline size_t MB(size_t n) { return n << 20; }
+static inline size_t KB(size_t n) { return n << 10; }
+
+/* ---- merlin/allocator.cuh ------------------------------------------------------ */
+
+enum MemoryType {
+  Device,   // HBM
+  Pinned,   // Pinned Host Memory
+  Host,     // Host Memory
+  Managed,  // Pageable Host Memory(Not required)
+};
+
+class BaseAllocator {
+ public:
+  BaseAllocator(const BaseAllocator&) = delete;
+  BaseAllocator(BaseAllocator&&) = delete;
+  BaseAllocator& operator=(const BaseAllocator&) = delete;
+  BaseAllocator& operator=(BaseAllocator&&) = delete;
+  BaseAllocator() = default;
+  virtual ~BaseAllocator() = default;
+
+  virtual void alloc(const MemoryType type, void** ptr, size_t size,
+                     unsigned int pinned_flags = hipHostMallocDefault) = 0;
+  virtual void alloc_async(const MemoryType type, void** ptr, size_t size,
+                           hipStream_t stream) = 0;
+  virtual void free(const MemoryType type, void* ptr) = 0;
+  virtual void free_async(const MemoryType type, void* ptr, hipStream_t stream) = 0;
+};
+
+class DefaultAllocator : public virtual BaseAllocator {
+ public:
+  DefaultAllocator() {}
+  ~DefaultAllocator() override {}
+
+  void alloc(const MemoryType type, void** ptr, size_t size,
+             unsigned int pinned_flags = hipHostMallocDefault) override {
+    switch (type) {
+      case MemoryType::Device:
+        HKV_HIP_CHECK(hipMalloc(ptr, size));
+        break;
+      case MemoryType::Pinned:
+        HKV_HIP_CHECK(hipHostMalloc(ptr, size, pinned_flags));
+        break;
+      case MemoryType::Host:
+        *ptr = std::malloc(size);
+        break;
+      default:
+        throw std::runtime_error("Unsupported memory type.");
+    }
+  }
+  void alloc_async(const MemoryType type, void** ptr, size_t size, hipStream_t stream) override {
+    if (type == MemoryType::Device) {
+      HKV_HIP_CHECK(hipMallocAsync(ptr, size, stream));
+    } else {
+      throw std::runtime_error("Only support async allocation on HBM.");
+    }
+  }
+  void free(const MemoryType type, void* ptr) override {
+    if (ptr == nullptr) return;
+    switch (type) {
+      case MemoryType::Pinned:
+        HKV_HIP_CHECK(hipHostFree(ptr));
+        break;
+      case MemoryType::Device:
+        HKV_HIP_CHECK(hipFree(ptr));
+        break;
+      case MemoryType::Host:
+        std::free(ptr);
+        break;
+      default:
+        throw std::runtime_error("Unsupported memory type.");
+    }
+  }
+  void free_async(const MemoryType type, void* ptr, hipStream_t stream) override {
+    if (ptr == nullptr) return;
+    if (type == MemoryType::Device) {
+      HKV_HIP_CHECK(hipFreeAsync(ptr, stream));
+    } else {
+      throw std::runtime_error("Only support async free on HBM.");
+    }
+  }
+};
+
+/* ---- merlin/types.cuh ------------------------------------------------------------ */
+
+template <class K, class V, class S>
+class BaseKVFile {
+ public:
+  virtual ~BaseKVFile() {}
+  virtual size_t read(const size_t n, const size_t dim, K* keys, V* vectors, S* scores) = 0;
+  virtual size_t write(const size_t n, const size_t dim, const K* keys, const V* vectors,
+                       const S* scores) = 0;
+};
+
+/* ---- merlin_hashtable.cuh ---------------------------------------------------------- */
+
+struct EvictStrategy {
+  enum EvictStrategyEnum {
+    kLru = 0,         ///< LRU mode.
+    kLfu = 1,         ///< LFU mode.
+    kEpochLru = 2,    ///< Epoch Lru mode.
+    kEpochLfu = 3,    ///< Epoch Lfu mode.
+    kCustomized = 4,  ///< Customized mode.
+  };
+};
+
+enum class TableMode {
+  kThroughput = 0,  ///< Default: single-bucket, max throughput.
+  kMemory = 1,      ///< Dual-bucket, higher load factor (not supported here).
+};
+
+/* memory_pool.cuh:139-143; kept so option structs copy over unchanged.  The
+ * library takes its few scratch words from the table allocation instead. */
+struct MemoryPoolOptions {
+  size_t max_stock = 4;
+  size_t max_pending = 16;
+};
+
+struct HashTableOptions {
+  size_t init_capacity = 0;        ///< The initial capacity of the hash table.
+  size_t max_capacity = 0;         ///< The maximum capacity of the hash table.
+  size_t max_hbm_for_vectors = 0;  ///< The maximum HBM for vectors, in bytes.
+  size_t max_bucket_size = 128;    ///< The length of each bucket.
+  size_t dim = 64;                 ///< The dimension of the vectors.
+  float max_load_factor = 0.5f;    ///< The max load factor before rehashing.
+  int block_size = 128;            ///< Kept for source compatibility; unused.
+  int io_block_size = 1024;        ///< Kept for source compatibility; unused.
+  int device_id = -1;              ///< The ID of device.
+  bool io_by_cpu = false;          ///< Not supported (must stay false).
+  bool use_constant_memory = false;  ///< reserved
+  int reserved_key_start_bit = 0;       ///< The binary index of reserved key.
+  size_t num_of_buckets_per_alloc = 1;  ///< Checked as in the reference; the
+                                        ///< table is one arena whatever it says.
+  bool api_lock = true;  ///< Order calls on different streams by role.
+  TableMode table_mode = TableMode::kThroughput;
+  MemoryPoolOptions device_memory_pool;
+  MemoryPoolOptions host_memory_pool;
+};
+
+template <class K, class S>
+using EraseIfPredict = bool (*)(const K& key, S& score, const K& pattern, const S& threshold);
+
+template <typename K, typename V, typename S = uint64_t>
+class HashTableBase {
+ public:
+  using size_type = size_t;
+  using key_type = K;
+  using value_type = V;
+  using score_type = S;
+  using allocator_type = BaseAllocator;
+
+  virtual ~HashTableBase() {}
+  virtual void init(const HashTableOptions& options, allocator_type* allocator = nullptr) = 0;
+  virtual void insert_or_assign(const size_type n, const key_type* keys, const value_type* values,
+                                const score_type* scores = nullptr, hipStream_t stream = 0,
+                                bool unique_key = true, bool ignore_evict_strategy = false) = 0;
+  virtual void insert_and_evict(const size_type n, const key_type* keys, const value_type* values,
+                                const score_type* scores, key_type* evicted_keys,
+                                value_type* evicted_values, score_type* evicted_scores,
+                                size_type* d_evicted_counter, hipStream_t stream = 0,
+                                bool unique_key = true, bool ignore_evict_strategy = false) = 0;
+  virtual size_type insert_and_evict(const size_type n, const key_type* keys,
+                                     const value_type* values, const score_type* scores,
+                                     key_type* evicted_keys, value_type* evicted_values,
+                                     score_type* evicted_scores, hipStream_t stream = 0,
+                                     bool unique_key = true,
+                                     bool ignore_evict_strategy = false) = 0;
+  virtual void accum_or_assign(const size_type n, const key_type* keys,
+                               const value_type* value_or_deltas, const bool* accum_or_assigns,
+                               const score_type* scores = nullptr, hipStream_t stream = 0,
+                               bool ignore_evict_strategy = false) = 0;
+  virtual void find_or_insert(const size_type n, const key_type* keys, value_type* values,
+                              score_type* scores = nullptr, hipStream_t stream = 0,
+                              bool unique_key = true, bool ignore_evict_strategy = false) = 0;
+  virtual void find_or_insert(const size_type n, const key_type* keys, value_type** values,
+                              bool* founds, score_type* scores = nullptr, hipStream_t stream = 0,
+                              bool unique_key = true, bool ignore_evict_strategy = false,
+                              key_type** locked_key_ptrs = nullptr) = 0;
+  virtual void lock_keys(const size_type n, key_type const* keys, key_type** locked_key_ptrs,
+                         bool* succeededs = nullptr, hipStream_t stream = 0,
+                         score_type const* scores = nullptr) = 0;
+  virtual void unlock_keys(const size_type n, key_type** locked_key_ptrs, const key_type* keys,
+                           bool* succeededs = nullptr, hipStream_t stream = 0) = 0;
+  virtual void assign(const size_type n, const key_type* keys, const value_type* values,
+                      const score_type* scores = nullptr, hipStream_t stream = 0,
+                      bool unique_key = true) = 0;
+  virtual void assign_scores(const size_type n, const key_type* keys,
+                             const score_type* scores = nullptr, hipStream_t stream = 0,
+                             bool unique_key = true) = 0;
+  virtual void assign(const size_type n, const key_type* keys, const score_type* scores = nullptr,
+                      hipStream_t stream = 0, bool unique_key = true) = 0;
+  virtual void assign_values(const size_type n, const key_type* keys, const value_type* values,
+                             hipStream_t stream = 0, bool unique_key = true) = 0;
+  virtual void find(const size_type n, const key_type* keys, value_type* values, bool* founds,
+                    score_type* scores = nullptr, hipStream_t stream = 0) const = 0;
+  virtual void find(const size_type n, const key_type* keys, value_type* values,
+                    key_type* missed_keys, int* missed_indices, int* missed_size,
+                    score_type* scores = nullptr, hipStream_t stream = 0) const = 0;
+  virtual void find(const size_type n, const key_type* keys, value_type** values, bool* founds,
+                    score_type* scores = nullptr, hipStream_t stream = 0,
+                    bool unique_key = true) const = 0;
+  virtual void find_and_update(const size_type n, const key_type* keys, value_type** values,
+                               bool* founds, score_type* scores = nullptr, hipStream_t stream = 0,
+                               bool unique_key = true) = 0;
+  virtual void contains(const size_type n, const key_type* keys, bool* founds,
+                        hipStream_t stream = 0) const = 0;
+  virtual void erase(const size_type n, const key_type* keys, hipStream_t stream = 0) = 0;
+  virtual void clear(hipStream_t stream = 0) = 0;
+  virtual void export_batch(size_type n, const size_type offset, size_type* d_counter,
+                            key_type* keys, value_type* values, score_type* scores = nullptr,
+                            hipStream_t stream = 0) const = 0;
+  virtual size_type export_batch(const size_type n, const size_type offset, key_type* keys,
+                                 value_type* values, score_type* scores = nullptr,
+                                 hipStream_t stream = 0) const = 0;
+  virtual bool empty(hipStream_t stream = 0) const = 0;
+  virtual size_type size(hipStream_t stream = 0) const = 0;
+  virtual size_type capacity() const = 0;
+  virtual void reserve(const size_type new_capacity, hipStream_t stream = 0) = 0;
+  virtual float load_factor(hipStream_t stream = 0) const = 0;
+  virtual void set_max_capacity(size_type new_max_capacity) = 0;
+  virtual size_type dim() const noexcept = 0;
+  virtual size_type max_bucket_size() const noexcept = 0;
+  virtual size_type bucket_count() const noexcept = 0;
+  virtual size_type save(BaseKVFile<K, V, S>* file,
+                         const size_t max_workspace_size = 1L * 1024 * 1024,
+                         hipStream_t stream = 0) const = 0;
+  virtual size_type load(BaseKVFile<K, V, S>* file,
+                         const size_t max_workspace_size = 1L * 1024 * 1024,
+                         hipStream_t stream = 0) = 0;
+  virtual void set_global_epoch(const uint64_t epoch) = 0;
+};
+
+namespace detail {
+
+template <class V>
+constexpr int value_kind_of() {
+  if (std::is_same<V, float>::value) return HKV_VALUE_F32;
+  if (std::is_same<V, double>::value) return HKV_VALUE_F64;
+  if (std::is_same<V, int32_t>::value || std::is_same<V, uint32_t>::value) return HKV_VALUE_I32;
+  if (std::is_same<V, int64_t>::value || std::is_same<V, uint64_t>::value) return HKV_VALUE_I64;
+  return HKV_VALUE_BYTES;
+}
+
+/* the caller's functor sees K and S; the kernel works on the 64-bit patterns */
+template <class K, class S, template <typename, typename> class PredFunctor>
+struct PredAdapter {
+  __device__ __forceinline__ bool operator()(const uint64_t& key, uint64_t& score,
+                                             const uint64_t& pattern,
+                                             const uint64_t& threshold) const {
+    PredFunctor<K, S> pred;
+    const K k = static_cast<K>(key);
+    S s = static_cast<S>(score);
+    const K p = static_cast<K>(pattern);
+    const S t = static_cast<S>(threshold);
+    return pred(k, s, p, t);
+  }
+};
+
+inline int alloc_cb(void* ctx, int type, void** ptr, size_t size) {
+  try {
+    static_cast<BaseAllocator*>(ctx)->alloc(static_cast<MemoryType>(type), ptr, size,
+                                            hipHostMallocMapped | hipHostMallocPortable);
+    return 0;
+  } catch (...) {
+    return 1;
+  }
+}
+inline int free_cb(void* ctx, int type, void* ptr) {
+  try {
+    static_cast<BaseAllocator*>(ctx)->free(static_cast<MemoryType>(type), ptr);
+    return 0;
+  } catch (...) {
+    return 1;
+  }
+}
+
+/* RAII bracket of the table's group lock around a caller-compiled kernel */
+struct RoleGuard {
+  const hkv_table* t;
+  int role;
+  hipStream_t s;
+  RoleGuard(const hkv_table* t_, int role_, hipStream_t s_) : t(t_), role(role_), s(s_) {
+    throw_on_error_(hkv_lock_begin(t, role, s));
+  }
+  ~RoleGuard() { (void)hkv_lock_end(t, role, s); }
+};
+
+}  // namespace detail
+
+template <typename K, typename V, typename S = uint64_t, int Strategy = EvictStrategy::kLru,
+          typename ArchTag = void>
+class HashTable : public HashTableBase<K, V, S> {
+ public:
+  using size_type = size_t;
+  using key_type = K;
+  using value_type = V;
+  using score_type = S;
+  static constexpr int evict_strategy = Strategy;
+  using allocator_type = BaseAllocator;
+
+  static_assert(std::is_same<K, int64_t>::value || std::is_same<K, uint64_t>::value,
+                "The key_type must be int64_t or uint64_t.");
+  static_assert(std::is_same<S, uint64_t>::value,
+                "The score_type must be uint64_t (uint32_t scores are not supported).");
+  static_assert(std::is_trivially_copyable<V>::value, "value_type must be trivially copyable");
+  static_assert(sizeof(size_type) == sizeof(uint64_t), "size_type must be 64 bits wide");
+
+ public:
+  HashTable() {}
+  ~HashTable() {
+    if (table_ != nullptr) {
+      (void)hkv_table_destroy(table_);
+      table_ = nullptr;
+    }
+    if (default_allocator_ && allocator_ != nullptr) delete allocator_;
+  }
+
+ private:
+  HashTable(const HashTable&) = delete;
+  HashTable& operator=(const HashTable&) = delete;
+  HashTable(HashTable&&) = delete;
+  HashTable& operator=(HashTable&&) = delete;
+
+ public:
+  void init(const HashTableOptions& options, allocator_type* allocator = nullptr) override {
+    if (initialized_) return;
+    options_ = options;
+    hkv_options o;
+    hkv_options_default(&o);
+    o.init_capacity = options.init_capacity;
+    o.max_capacity = options.max_capacity;
+    o.max_hbm_for_vectors = options.max_hbm_for_vectors;
+    o.max_bucket_size = options.max_bucket_size;
+    o.dim = options.dim;
+    o.max_load_factor = options.max_load_factor;
+    o.block_size = options.block_size;
+    o.io_block_size = options.io_block_size;
+    o.device_id = options.device_id;
+    o.io_by_cpu = options.io_by_cpu;
+    o.use_constant_memory = options.use_constant_memory;
+    o.reserved_key_start_bit = options.reserved_key_start_bit;
+    o.num_of_buckets_per_alloc = options.num_of_buckets_per_alloc;
+    o.api_lock = options.api_lock;
+    o.table_mode = static_cast<int>(options.table_mode);
+    o.evict_strategy = Strategy;
+    o.value_kind = detail::value_kind_of<V>();
+    o.value_size = sizeof(V);
+    o.score_size = sizeof(S);
+    default_allocator_ = (allocator == nullptr);
+    allocator_ = default_allocator_ ? nullptr : allocator;
+    if (allocator_ != nullptr) {
+      hkv_allocator a{allocator_, &detail::alloc_cb, &detail::free_cb};
+      throw_on_error_(hkv_table_create_with_allocator(&o, &a, &table_));
+    } else {
+      throw_on_error_(hkv_table_create(&o, &table_));
+    }
+    if (options_.device_id < 0) HKV_HIP_CHECK(hipGetDevice(&options_.device_id));
+    initialized_ = true;
+  }
+
+  void insert_or_assign(const size_type n, const key_type* keys, const value_type* values,
+                        const score_type* scores = nullptr, hipStream_t stream = 0,
+                        bool unique_key = true, bool ignore_evict_strategy = false) override {
+    throw_on_error_(hkv_insert_or_assign(table_, n, u64(keys), values, scores, stream, unique_key,
+                                         ignore_evict_strategy));
+  }
+
+  void insert_and_evict(const size_type n, const key_type* keys, const value_type* values,
+                        const score_type* scores, key_type* evicted_keys,
+                        value_type* evicted_values, score_type* evicted_scores,
+                        size_type* d_evicted_counter, hipStream_t stream = 0,
+                        bool unique_key = true, bool ignore_evict_strategy = false) override {
+    throw_on_error_(hkv_insert_and_evict(table_, n, u64(keys), values, scores, u64(evicted_keys),
+                                         evicted_values, evicted_scores,
+                                         reinterpret_cast<uint64_t*>(d_evicted_counter), stream,
+                                         unique_key, ignore_evict_strategy));
+  }
+
+  size_type insert_and_evict(const size_type n, const key_type* keys, const value_type* values,
+                             const score_type* scores, key_type* evicted_keys,
+                             value_type* evicted_values, score_type* evicted_scores,
+                             hipStream_t stream = 0, bool unique_key = true,
+                             bool ignore_evict_strategy = false) override {
+    uint64_t cnt = 0;
+    throw_on_error_(hkv_insert_and_evict_count(table_, n, u64(keys), values, scores,
+                                               u64(evicted_keys), evicted_values, evicted_scores,
+                                               stream, unique_key, ignore_evict_strategy, &cnt));
+    return static_cast<size_type>(cnt);
+  }
+
+  void accum_or_assign(const size_type n, const key_type* keys, const value_type* value_or_deltas,
+                       const bool* accum_or_assigns, const score_type* scores = nullptr,
+                       hipStream_t stream = 0, bool ignore_evict_strategy = false) override {
+    throw_on_error_(hkv_accum_or_assign(table_, n, u64(keys), value_or_deltas,
+                                        reinterpret_cast<const uint8_t*>(accum_or_assigns), scores,
+                                        stream, ignore_evict_strategy));
+  }
+
+  void find_or_insert(const size_type n, const key_type* keys, value_type* values,
+                      score_type* scores = nullptr, hipStream_t stream = 0,
+                      bool unique_key = true, bool ignore_evict_strategy = false) override {
+    throw_on_error_(hkv_find_or_insert(table_, n, u64(keys), values, scores, stream, unique_key,
+                                       ignore_evict_strategy));
+  }
+
+  void find_or_insert(const size_type n, const key_type* keys, value_type** values, bool* founds,
+                      score_type* scores = nullptr, hipStream_t stream = 0,
+                      bool unique_key = true, bool ignore_evict_strategy = false,
+                      key_type** locked_key_ptrs = nullptr) override {
+    if (locked_key_ptrs != nullptr)
+      throw std::runtime_error("find_or_insert with locked_key_ptrs is not supported");
+    throw_on_error_(hkv_find_or_insert_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
+                                           reinterpret_cast<uint8_t*>(founds), scores, stream,
+                                           unique_key, ignore_evict_strategy));
+  }
+
+  void lock_keys(const size_type, key_type const*, key_type**, bool* = nullptr, hipStream_t = 0,
+                 score_type const* = nullptr) override {
+    throw std::runtime_error("lock_keys is not supported");
+  }
+  void unlock_keys(const size_type, key_type**, const key_type*, bool* = nullptr,
+                   hipStream_t = 0) override {
+    throw std::runtime_error("unlock_keys is not supported");
+  }
+
+  void assign(const size_type n, const key_type* keys, const value_type* values,
+              const score_type* scores = nullptr, hipStream_t stream = 0,
+              bool unique_key = true) override {
+    throw_on_error_(hkv_assign(table_, n, u64(keys), values, scores, stream, unique_key));
+  }
+  void assign_scores(const size_type n, const key_type* keys, const score_type* scores = nullptr,
+                     hipStream_t stream = 0, bool unique_key = true) override {
+    throw_on_error_(hkv_assign_scores(table_, n, u64(keys), scores, stream, unique_key));
+  }
+  /* alias of assign_scores (merlin_hashtable.cuh:2285-2290) */
+  void assign(const size_type n, const key_type* keys, const score_type* scores = nullptr,
+              hipStream_t stream = 0, bool unique_key = true) override {
+    assign_scores(n, keys, scores, stream, unique_key);
+  }
+  void assign_values(const size_type n, const key_type* keys, const value_type* values,
+                     hipStream_t stream = 0, bool unique_key = true) override {
+    throw_on_error_(hkv_assign_values(table_, n, u64(keys), values, stream, unique_key));
+  }
+
+  void find(const size_type n, const key_type* keys, value_type* values, bool* founds,
+            score_type* scores = nullptr, hipStream_t stream = 0) const override {
+    throw_on_error_(hkv_find(table_, n, u64(keys), values, reinterpret_cast<uint8_t*>(founds),
+                             scores, stream));
+  }
+  void find(const size_type n, const key_type* keys, value_type* values, key_type* missed_keys,
+            int* missed_indices, int* missed_size, score_type* scores = nullptr,
+            hipStream_t stream = 0) const override {
+    throw_on_error_(hkv_find_missed(table_, n, u64(keys), values, u64(missed_keys), missed_indices,
+                                    missed_size, scores, stream));
+  }
+  void find(const size_type n, const key_type* keys, value_type** values, bool* founds,
+            score_type* scores = nullptr, hipStream_t stream = 0,
+            bool unique_key = true) const override {
+    throw_on_error_(hkv_find_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
+                                 reinterpret_cast<uint8_t*>(founds), scores, stream, unique_key));
+  }
+  void find_and_update(const size_type, const key_type*, value_type**, bool*,
+                       score_type* = nullptr, hipStream_t = 0, bool = true) override {
+    throw std::runtime_error("find_and_update is not supported");
+  }
+  void contains(const size_type n, const key_type* keys, bool* founds,
+                hipStream_t stream = 0) const override {
+    throw_on_error_(hkv_contains(table_, n, u64(keys), reinterpret_cast<uint8_t*>(founds), stream));
+  }
+
+  void erase(const size_type n, const key_type* keys, hipStream_t stream = 0) override {
+    throw_on_error_(hkv_erase(table_, n, u64(keys), stream));
+  }
+
+  /* erase every entry for which pred(key, score, pattern, threshold) holds;
+   * returns how many (merlin_hashtable.cuh:2963-2996).  Synchronises `stream`. */
+  template <template <typename, typename> class PredFunctor>
+  size_type erase_if(const key_type& pattern, const score_type& threshold, hipStream_t stream = 0) {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    unsigned long long* d_count = nullptr;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
+    hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
+                       d_count);
+    {
+      detail::RoleGuard g(table_, 2, stream);
+      const unsigned blocks =
+          static_cast<unsigned>(std::min<uint64_t>((v.capacity + 255) / 256, 16384));
+      hipLaunchKernelGGL((hkv::erase_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
+                         dim3(blocks), dim3(256), 0, stream, v,
+                         detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
+                         static_cast<uint64_t>(threshold), d_count);
+      HKV_HIP_CHECK(hipGetLastError());
+    }
+    unsigned long long h = 0;
+    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
+    HKV_HIP_CHECK(hipStreamSynchronize(stream));
+    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
+    return static_cast<size_type>(h);
+  }
+
+  void clear(hipStream_t stream = 0) override { throw_on_error_(hkv_clear(table_, stream)); }
+
+  void export_batch(size_type n, const size_type offset, size_type* d_counter, key_type* keys,
+                    value_type* values, score_type* scores = nullptr,
+                    hipStream_t stream = 0) const override {
+    throw_on_error_(hkv_export_batch(table_, n, offset, reinterpret_cast<uint64_t*>(d_counter),
+                                     u64(keys), values, scores, stream));
+  }
+
+  size_type export_batch(const size_type n, const size_type offset, key_type* keys,
+                         value_type* values, score_type* scores = nullptr,
+                         hipStream_t stream = 0) const override {
+    size_type* d_counter = nullptr;
+    size_type h_counter = 0;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_counter), sizeof(size_type), stream));
+    export_batch(n, offset, d_counter, keys, values, scores, stream);
+    HKV_HIP_CHECK(
+        hipMemcpyAsync(&h_counter, d_counter, sizeof(size_type), hipMemcpyDeviceToHost, stream));
+    HKV_HIP_CHECK(hipStreamSynchronize(stream));
+    HKV_HIP_CHECK(hipFreeAsync(d_counter, stream));
+    return h_counter;
+  }
+
+  /* merlin_hashtable.cuh:3193-3276: the caller's device functor decides. */
+  template <template <typename, typename> class PredFunctor>
+  void export_batch_if(const key_type& pattern, const score_type& threshold, size_type n,
+                       const size_type offset, size_type* d_counter, key_type* keys,
+                       value_type* values, score_type* scores = nullptr,
+                       hipStream_t stream = 0) const {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    detail::RoleGuard g(table_, 0, stream);
+    hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
+    if (offset >= v.capacity) return;
+    n = std::min<size_type>(v.capacity - offset, n);
+    if (n == 0) return;
+    const uint64_t waves = (n + hkv::kWave - 1) / hkv::kWave;
+    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((waves + 3) / 4, 16384));
+    hipLaunchKernelGGL((hkv::export_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
+                       dim3(blocks), dim3(256), 0, stream, v,
+                       detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
+                       static_cast<uint64_t>(threshold), static_cast<uint64_t>(offset),
+                       static_cast<uint64_t>(n), reinterpret_cast<unsigned long long*>(d_counter),
+                       u64(keys), reinterpret_cast<uint8_t*>(values), scores);
+    HKV_HIP_CHECK(hipGetLastError());
+  }
+
+  /* merlin_hashtable.cuh:3460-3476.  Synchronises `stream`. */
+  template <template <typename, typename> class PredFunctor>
+  size_type size_if(const key_type& pattern, const score_type& threshold,
+                    hipStream_t stream = 0) const {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    unsigned long long* d_count = nullptr;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
+    hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
+                       d_count);
+    {
+      detail::RoleGuard g(table_, 0, stream);
+      const unsigned blocks =
+          static_cast<unsigned>(std::min<uint64_t>((v.capacity + 255) / 256, 8192));
+      hipLaunchKernelGGL((hkv::size_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
+                         dim3(blocks), dim3(256), 0, stream, v,
+                         detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
+                         static_cast<uint64_t>(threshold), d_count);
+      HKV_HIP_CHECK(hipGetLastError());
+    }
+    unsigned long long h = 0;
+    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
+    HKV_HIP_CHECK(hipStreamSynchronize(stream));
+    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
+    return static_cast<size_type>(h);
+  }
+
+  bool empty(hipStream_t stream = 0) const override { return size(stream) == 0; }
+
+  size_type size(hipStream_t stream = 0) const override {
+    uint64_t n = 0;
+    throw_on_error_(hkv_size(table_, stream, &n));
+    return static_cast<size_type>(n);
+  }
+
+  size_type capacity() const override { return hkv_capacity(table_); }
+
+  void reserve(const size_type new_capacity, hipStream_t = 0) override {
+    if (new_capacity <= capacity()) return;
+    throw std::runtime_error("reserve() to a larger capacity (rehash) is not supported");
+  }
+
+  float load_factor(hipStream_t stream = 0) const override {
+    float lf = 0.f;
+    throw_on_error_(hkv_load_factor(table_, stream, &lf));
+    return lf;
+  }
+
+  /* merlin_hashtable.cuh:3561-3574 */
+  void set_max_capacity(size_type new_max_capacity) override {
+    if (new_max_capacity == 0 || (new_max_capacity & (new_max_capacity - 1)) != 0)
+      throw std::invalid_argument("None power-of-2 new_max_capacity is not supported.");
+    if (new_max_capacity > capacity())
+      throw std::runtime_error("growing the table (rehash) is not supported");
+    options_.max_capacity = new_max_capacity;
+  }
+
+  size_type dim() const noexcept override { return options_.dim; }
+  size_type max_bucket_size() const noexcept override { return options_.max_bucket_size; }
+  size_type bucket_count() const noexcept override { return hkv_bucket_count(table_); }
+
+  /*
+   * save / load, merlin_hashtable.cuh:3615-3758: the table is exported in
+   * windows of the slot range that fit the workspace, staged through pinned
+   * host memory, and handed to the file; load inserts with the saved scores
+   * (ignore_evict_strategy).
+   */
+  size_type save(BaseKVFile<K, V, S>* file, const size_t max_workspace_size = 1L * 1024 * 1024,
+                 hipStream_t stream = 0) const override {
+    const size_type tuple_size = sizeof(K) + sizeof(S) + sizeof(V) * dim();
+    MERLIN_CHECK(max_workspace_size >= tuple_size,
+                 "[HierarchicalKV] max_workspace_size is smaller than a single `key + score + value` tuple! Please set a larger value!");
+    const size_type total = capacity();
+    const size_type window = std::max<size_type>(max_workspace_size / tuple_size, 1);
+    K* d_keys = nullptr;
+    V* d_vals = nullptr;
+    S* d_scores = nullptr;
+    K* h_keys = nullptr;
+    V* h_vals = nullptr;
+    S* h_scores = nullptr;
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_keys), window * sizeof(K)));
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_vals), window * sizeof(V) * dim()));
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_scores), window * sizeof(S)));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_keys), window * sizeof(K)));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_vals), window * sizeof(V) * dim()));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_scores), window * sizeof(S)));
+    size_type written = 0;
+    for (size_type off = 0; off < total; off += window) {
+      const size_type c = export_batch(window, off, d_keys, d_vals, d_scores, stream);
+      if (c == 0) continue;
+      HKV_HIP_CHECK(hipMemcpyAsync(h_keys, d_keys, c * sizeof(K), hipMemcpyDeviceToHost, stream));
+      HKV_HIP_CHECK(hipMemcpyAsync(h_vals, d_vals, c * sizeof(V) * dim(), hipMemcpyDeviceToHost, stream));
+      HKV_HIP_CHECK(hipMemcpyAsync(h_scores, d_scores, c * sizeof(S), hipMemcpyDeviceToHost, stream));
+      HKV_HIP_CHECK(hipStreamSynchronize(stream));
+      written += file->write(c, dim(), h_keys, h_vals, h_scores);
+    }
+    HKV_HIP_CHECK(hipFree(d_keys));
+    HKV_HIP_CHECK(hipFree(d_vals));
+    HKV_HIP_CHECK(hipFree(d_scores));
+    HKV_HIP_CHECK(hipHostFree(h_keys));
+    HKV_HIP_CHECK(hipHostFree(h_vals));
+    HKV_HIP_CHECK(hipHostFree(h_scores));
+    return written;
+  }
+
+  size_type load(BaseKVFile<K, V, S>* file, const size_t max_workspace_size = 1L * 1024 * 1024,
+                 hipStream_t stream = 0) override {
+    const size_type tuple_size = sizeof(K) + sizeof(S) + sizeof(V) * dim();
+    MERLIN_CHECK(max_workspace_size >= tuple_size,
+                 "[HierarchicalKV] max_workspace_size is smaller than a single `key + score + value` tuple! Please set a larger value!");
+    const size_type window = std::max<size_type>(max_workspace_size / tuple_size, 1);
+    K* d_keys = nullptr;
+    V* d_vals = nullptr;
+    S* d_scores = nullptr;
+    K* h_keys = nullptr;
+    V* h_vals = nullptr;
+    S* h_scores = nullptr;
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_keys), window * sizeof(K)));
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_vals), window * sizeof(V) * dim()));
+    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_scores), window * sizeof(S)));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_keys), window * sizeof(K)));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_vals), window * sizeof(V) * dim()));
+    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_scores), window * sizeof(S)));
+    size_type loaded = 0;
+    while (true) {
+      const size_type c = file->read(window, dim(), h_keys, h_vals, h_scores);
+      if (c == 0) break;
+      HKV_HIP_CHECK(hipMemcpyAsync(d_keys, h_keys, c * sizeof(K), hipMemcpyHostToDevice, stream));
+      HKV_HIP_CHECK(hipMemcpyAsync(d_vals, h_vals, c * sizeof(V) * dim(), hipMemcpyHostToDevice, stream));
+      HKV_HIP_CHECK(hipMemcpyAsync(d_scores, h_scores, c * sizeof(S), hipMemcpyHostToDevice, stream));
+      insert_or_assign(c, d_keys, d_vals, d_scores, stream, true, true);
+      HKV_HIP_CHECK(hipStreamSynchronize(stream));
+      loaded += c;
+    }
+    HKV_HIP_CHECK(hipFree(d_keys));
+    HKV_HIP_CHECK(hipFree(d_vals));
+    HKV_HIP_CHECK(hipFree(d_scores));
+    HKV_HIP_CHECK(hipHostFree(h_keys));
+    HKV_HIP_CHECK(hipHostFree(h_vals));
+    HKV_HIP_CHECK(hipHostFree(h_scores));
+    return loaded;
+  }
+
+  void set_global_epoch(const uint64_t epoch) override {
+    throw_on_error_(hkv_set_global_epoch(table_, epoch));
+  }
+
+  /* this build's additions */
+  bool is_pure_hbm() const { return hkv_is_pure_hbm(table_) != 0; }
+  hkv_table* native_handle() const { return table_; }
+
+ private:
+  static const uint64_t* u64(const K* p) { return reinterpret_cast<const uint64_t*>(p); }
+  static uint64_t* u64(K* p) { return reinterpret_cast<uint64_t*>(p); }
+
+  HashTableOptions options_;
+  hkv_table* table_ = nullptr;
+  bool initialized_ = false;
+  allocator_type* allocator_ = nullptr;
+  bool default_allocator_ = true;
+};
+
+}  // namespace merlin
+}  // namespace nv
+
+#endif  // MERLIN_HASHTABLE_HPP_

@@ -1,0 +1,466 @@
+// Exercises the C++ drop-in header the way the reference's own gtest files
+// use nv::merlin::HashTable (tests/merlin_hashtable_test.cc.cu:178-423,
+// 2674-2849; tests/insert_and_evict_test.cc.cu:34-154;
+// tests/export_batch_if_test.cc.cu:128-301; tests/save_and_load_test.cc.cu),
+// with a small CHECK macro instead of gtest.  Needs a GPU.
+#include <algorithm>
+#include <cstdio>
+#include <map>
+#include <numeric>
+#include <random>
+#include <set>
+#include <unordered_set>
+#include <vector>
+
+#include "merlin_hashtable.cuh"
+#include "merlin_localfile.hpp"
+
+using namespace nv::merlin;
+using K = uint64_t;
+using V = float;
+using S = uint64_t;
+
+static int g_failures = 0;
+#define CHECK(cond)                                                             \
+  do {                                                                          \
+    if (!(cond)) {                                                              \
+      std::printf("CHECK failed %s:%d: %s\n", __FILE__, __LINE__, #cond);       \
+      g_failures++;                                                             \
+    }                                                                           \
+  } while (0)
+#define HIP(x) HKV_HIP_CHECK(x)
+
+template <class T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  explicit DevBuf(size_t n_) : n(n_) { HIP(hipMalloc(reinterpret_cast<void**>(&p), std::max<size_t>(n, 1) * sizeof(T))); }
+  ~DevBuf() { (void)hipFree(p); }
+  void up(const std::vector<T>& h) { HIP(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice)); }
+  using H = typename std::conditional<std::is_same<T, bool>::value, uint8_t, T>::type;
+  std::vector<H> down(size_t c) const {
+    std::vector<H> h(c);
+    HIP(hipMemcpy(h.data(), p, c * sizeof(T), hipMemcpyDeviceToHost));
+    return h;
+  }
+};
+
+template <class Kt, class St>
+struct ExportIfPredFunctor {
+  __forceinline__ __device__ bool operator()(const Kt& key, St& score, const Kt& pattern,
+                                             const St& threshold) {
+    return score > threshold;
+  }
+};
+template <class Kt, class St>
+struct EraseIfPredFunctor {
+  __forceinline__ __device__ bool operator()(const Kt& key, St& score, const Kt& pattern,
+                                             const St& threshold) {
+    return ((key & 0x1u) == 0x1u) && (score > threshold);
+  }
+};
+
+static std::vector<K> random_keys(size_t n, uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  std::unordered_set<K> seen;
+  std::vector<K> out;
+  while (out.size() < n) {
+    K k = rng();
+    if ((k & ~UINT64_C(3)) == ~UINT64_C(3)) continue;
+    if (seen.insert(k).second) out.push_back(k);
+  }
+  return out;
+}
+// v[i][j] = float(key * 0.00001), as tests/test_util.cuh:160-163
+static std::vector<V> values_of(const std::vector<K>& keys, size_t dim) {
+  std::vector<V> v(keys.size() * dim);
+  for (size_t i = 0; i < keys.size(); i++)
+    for (size_t j = 0; j < dim; j++) v[i * dim + j] = static_cast<float>(keys[i] * 0.00001);
+  return v;
+}
+
+static void test_basic() {
+  constexpr size_t DIM = 16, N = 1 << 16;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = 64 * 1024 * 1024UL - (128 + 1);
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(16);
+  o.reserved_key_start_bit = 2;
+  o.num_of_buckets_per_alloc = 32;
+  using Table = HashTable<K, V, S, EvictStrategy::kCustomized>;
+  Table table;
+  table.init(o);
+  CHECK(table.bucket_count() == 524287);
+  hipStream_t stream;
+  HIP(hipStreamCreate(&stream));
+  CHECK(table.size(stream) == 0);
+  CHECK(table.empty(stream));
+  auto keys = random_keys(N, 1);
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  std::iota(scores.begin(), scores.end(), 1);
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM), dout(N * DIM);
+  DevBuf<S> ds(N), dso(N);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p, stream);
+  CHECK(table.size(stream) == N);
+  HIP(hipMemsetAsync(dout.p, 0, N * DIM * sizeof(V), stream));
+  table.find(N, dk.p, dout.p, df.p, dso.p, stream);
+  HIP(hipStreamSynchronize(stream));
+  {
+    auto f = df.down(N);
+    auto out = dout.down(N * DIM);
+    auto so = dso.down(N);
+    size_t found = 0;
+    bool same = true;
+    for (size_t i = 0; i < N; i++) {
+      found += f[i];
+      same &= so[i] == scores[i];
+      for (size_t j = 0; j < DIM; j++) same &= out[i * DIM + j] == vals[i * DIM + j];
+    }
+    CHECK(found == N);
+    CHECK(same);
+  }
+  // accum_or_assign: existing & flagged -> old + delta
+  {
+    std::vector<V> delta(N * DIM, 0.5f);
+    std::vector<char> flags(N, 1);
+    DevBuf<V> dd(N * DIM);
+    dd.up(delta);
+    DevBuf<bool> dflag(N);
+    HIP(hipMemcpy(dflag.p, flags.data(), N, hipMemcpyHostToDevice));
+    table.accum_or_assign(N, dk.p, dd.p, dflag.p, ds.p, stream);
+    table.find(N, dk.p, dout.p, df.p, nullptr, stream);
+    HIP(hipStreamSynchronize(stream));
+    auto out = dout.down(N * DIM);
+    bool same = true;
+    for (size_t i = 0; i < N * DIM; i++) same &= out[i] == vals[i] + 0.5f;
+    CHECK(same);
+  }
+  // contains, erase half, clear
+  table.contains(N, dk.p, df.p, stream);
+  HIP(hipStreamSynchronize(stream));
+  {
+    auto f = df.down(N);
+    CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  }
+  table.erase(N / 2, dk.p, stream);
+  CHECK(table.size(stream) == N / 2);
+  // pointer find on what is left
+  {
+    DevBuf<V*> dp(N);
+    table.find(N, dk.p, dp.p, df.p, nullptr, stream);
+    HIP(hipStreamSynchronize(stream));
+    auto f = df.down(N);
+    auto ptrs = dp.down(N);
+    size_t found = 0, nulls = 0;
+    for (size_t i = 0; i < N; i++) {
+      found += f[i];
+      nulls += ptrs[i] == nullptr;
+      CHECK(f[i] == (i >= N / 2));
+    }
+    CHECK(found == N / 2 && nulls == N / 2);
+    V row[DIM];
+    HIP(hipMemcpy(row, ptrs[N - 1], sizeof row, hipMemcpyDeviceToHost));
+    CHECK(row[3] == vals[(N - 1) * DIM + 3] + 0.5f);
+  }
+  // export == what is resident
+  {
+    DevBuf<K> ek(N);
+    DevBuf<V> ev(N * DIM);
+    DevBuf<S> es(N);
+    size_t total = 0;
+    const size_t cap = table.capacity();
+    std::set<K> exported;
+    for (size_t off = 0; off < cap; off += 8 * 1024 * 1024) {
+      size_t c = table.export_batch(8 * 1024 * 1024, off, ek.p + total, ev.p + total * DIM,
+                                    es.p + total, stream);
+      total += c;
+    }
+    CHECK(total == N / 2);
+    auto hk = ek.down(total);
+    exported.insert(hk.begin(), hk.end());
+    CHECK(exported.size() == N / 2);
+    for (size_t i = N / 2; i < N; i++) CHECK(exported.count(keys[i]) == 1);
+  }
+  table.clear(stream);
+  CHECK(table.size(stream) == 0);
+  CHECK(table.load_factor(stream) == 0.0f);
+  HIP(hipStreamDestroy(stream));
+}
+
+// keys that land in one bucket (test_util.cuh:296-331), host twin of the hash
+static uint64_t fmix64(uint64_t k) {
+  k ^= k >> 33;
+  k *= UINT64_C(0xff51afd7ed558ccd);
+  k ^= k >> 33;
+  k *= UINT64_C(0xc4ceb9fe1a85ec53);
+  k ^= k >> 33;
+  return k;
+}
+static std::vector<K> keys_in_bucket(size_t n, size_t capacity, size_t bucket, K lo, K hi, uint64_t seed) {
+  std::mt19937_64 rng(seed);
+  std::unordered_set<K> s;
+  std::vector<K> out;
+  while (out.size() < n) {
+    K c = rng() % (hi - lo) + lo;
+    if (((fmix64(c) & (capacity - 1)) / 128) == bucket && s.insert(c).second) out.push_back(c);
+  }
+  return out;
+}
+
+static void test_evict_strategy_customized() {
+  constexpr size_t DIM = 4, CAP = 1024;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  o.reserved_key_start_bit = 15;
+  o.num_of_buckets_per_alloc = 8;
+  using Table = HashTable<K, V, S, EvictStrategy::kCustomized>;
+  auto base = keys_in_bucket(128, CAP, 1, 0, 0x3FFFFFFFFFFFFFFF, 3);
+  auto test = keys_in_bucket(128, CAP, 1, 0x3FFFFFFFFFFFFFFF, 0xFFFFFFFFFFFFFFFD, 4);
+  for (int i = 64; i < 128; i++) test[i] = base[i];
+  std::vector<S> bs(128), ts(128);
+  std::iota(bs.begin(), bs.end(), 1000);
+  std::iota(ts.begin(), ts.end(), 1128);
+  DevBuf<K> dk(128), ek(CAP);
+  DevBuf<V> dv(128 * DIM), ev(CAP * DIM);
+  DevBuf<S> ds(128), es(CAP);
+  for (int rep = 0; rep < 16; rep++) {
+    Table table;
+    table.init(o);
+    dk.up(base);
+    dv.up(values_of(base, DIM));
+    ds.up(bs);
+    table.insert_or_assign(128, dk.p, dv.p, ds.p);
+    CHECK(table.size() == 128);
+    dk.up(test);
+    dv.up(values_of(test, DIM));
+    ds.up(ts);
+    table.insert_or_assign(128, dk.p, dv.p, ds.p);
+    CHECK(table.size() == 128);
+    size_t c = table.export_batch(table.capacity(), 0, ek.p, ev.p, es.p);
+    CHECK(c == 128);
+    auto hs = es.down(c);
+    auto hk = ek.down(c);
+    auto hv = ev.down(c * DIM);
+    std::sort(hs.begin(), hs.end());
+    bool ok = true;
+    for (size_t i = 0; i < c; i++) ok &= hs[i] == 1128 + i;
+    CHECK(ok);
+    for (size_t i = 0; i < c; i++) CHECK(hv[i * DIM] == static_cast<float>(hk[i] * 0.00001));
+    // scores are required in customized mode (merlin_hashtable.cuh:3846-3850)
+    bool threw = false;
+    try {
+      table.insert_or_assign(128, dk.p, dv.p, nullptr);
+    } catch (const MerlinException&) {
+      threw = true;
+    }
+    CHECK(threw);
+  }
+}
+
+static void test_insert_and_evict_and_predicates() {
+  constexpr size_t DIM = 8, CAP = 1 << 16, N = 1 << 14;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  using Table = HashTable<int64_t, V, S, EvictStrategy::kCustomized>;
+  Table table;
+  table.init(o);
+  std::map<K, V> model;  // key -> first value element, whatever is resident or evicted
+  DevBuf<int64_t> dk(N), ek(N);
+  DevBuf<V> dv(N * DIM), ev(N * DIM);
+  DevBuf<S> ds(N), es(N);
+  size_t total_evicted = 0;
+  std::map<K, V> resident_or_gone;
+  for (int b = 0; b < 8; b++) {  // 8 * 16384 = 2 * capacity fresh keys
+    auto keys = random_keys(N, 100 + b);
+    auto vals = values_of(keys, DIM);
+    std::vector<S> scores(N);
+    for (size_t i = 0; i < N; i++) scores[i] = (S(b + 1) << 40) | i;
+    std::vector<int64_t> sk(keys.begin(), keys.end());
+    dk.up(sk);
+    dv.up(vals);
+    ds.up(scores);
+    size_t before = table.size();
+    size_t c = table.insert_and_evict(N, dk.p, dv.p, ds.p, ek.p, ev.p, es.p);
+    size_t after = table.size();
+    CHECK(c + after == before + N);  // insert_and_evict_test.cc.cu:94,115
+    total_evicted += c;
+    auto hk = ek.down(c);
+    auto hv = ev.down(c * DIM);
+    for (size_t i = 0; i < c; i++) CHECK(hv[i * DIM] == static_cast<float>(uint64_t(hk[i]) * 0.00001));
+  }
+  CHECK(total_evicted > 0);
+  CHECK(table.size() <= CAP);
+  // size_if == export_batch_if count, every exported tuple satisfies the predicate
+  const S threshold = (S(5) << 40);
+  size_t expect = table.size_if<ExportIfPredFunctor>(0, threshold);
+  DevBuf<int64_t> xk(CAP);
+  DevBuf<V> xv(CAP * DIM);
+  DevBuf<S> xs(CAP);
+  DevBuf<size_t> dc(1);
+  table.export_batch_if<ExportIfPredFunctor>(0, threshold, table.capacity(), 0, dc.p, xk.p, xv.p, xs.p);
+  HIP(hipDeviceSynchronize());
+  size_t got = dc.down(1)[0];
+  CHECK(got == expect && got > 0);
+  auto hs = xs.down(got);
+  CHECK(std::all_of(hs.begin(), hs.end(), [&](S s) { return s > threshold; }));
+  auto hk = xk.down(got);
+  CHECK(std::set<int64_t>(hk.begin(), hk.end()).size() == got);
+  // erase_if removes exactly what size_if counts for the same predicate
+  size_t odd_high = table.size_if<EraseIfPredFunctor>(0, threshold);
+  size_t before = table.size();
+  size_t erased = table.erase_if<EraseIfPredFunctor>(0, threshold);
+  CHECK(erased == odd_high);
+  CHECK(table.size() == before - erased);
+  CHECK(table.size_if<EraseIfPredFunctor>(0, threshold) == 0);
+}
+
+struct CountingAllocator : public DefaultAllocator {
+  int allocs = 0, frees = 0;
+  void alloc(const MemoryType type, void** ptr, size_t size, unsigned int flags = hipHostMallocDefault) override {
+    allocs++;
+    DefaultAllocator::alloc(type, ptr, size, flags);
+  }
+  void free(const MemoryType type, void* ptr) override {
+    frees++;
+    DefaultAllocator::free(type, ptr);
+  }
+};
+
+static void test_allocator_hybrid_and_checkpoint() {
+  constexpr size_t DIM = 32, CAP = 1 << 15, N = 1 << 14;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = CAP * DIM * sizeof(V) / 4;  // a quarter of the rows in HBM
+  CountingAllocator alloc;
+  auto keys = random_keys(N, 7);
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  std::iota(scores.begin(), scores.end(), 10);
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM), dout(N * DIM);
+  DevBuf<S> ds(N);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  {
+    using Table = HashTable<K, V, S, EvictStrategy::kLfu>;
+    Table table;
+    table.init(o, &alloc);
+    CHECK(!table.is_pure_hbm());
+    CHECK(alloc.allocs >= 3);
+    table.insert_or_assign(N, dk.p, dv.p, ds.p);
+    CHECK(table.size() == N);
+    table.find(N, dk.p, dout.p, df.p);
+    HIP(hipDeviceSynchronize());
+    auto out = dout.down(N * DIM);
+    CHECK(out == vals);
+    // insert_and_evict is refused in hybrid mode (merlin_hashtable.cuh:1384-1386)
+    bool threw = false;
+    try {
+      DevBuf<size_t> dc(1);
+      table.insert_and_evict(N, dk.p, dv.p, ds.p, dk.p, dout.p, ds.p, dc.p);
+    } catch (const std::runtime_error&) {
+      threw = true;
+    }
+    CHECK(threw);
+    // save -> load into a second table
+    LocalKVFile<K, V, S> file;
+    CHECK(file.open("/tmp/hkv_k.bin", "/tmp/hkv_v.bin", "/tmp/hkv_s.bin", "wb"));
+    CHECK(table.save(&file) == N);
+    file.close();
+    HashTableOptions o2 = o;
+    o2.max_hbm_for_vectors = GB(1);
+    Table t2;
+    t2.init(o2);
+    CHECK(file.open("/tmp/hkv_k.bin", "/tmp/hkv_v.bin", "/tmp/hkv_s.bin", "rb"));
+    CHECK(t2.load(&file) == N);
+    file.close();
+    CHECK(t2.size() == N);
+    DevBuf<S> dso(N);
+    t2.find(N, dk.p, dout.p, df.p, dso.p);
+    HIP(hipDeviceSynchronize());
+    CHECK(dout.down(N * DIM) == vals);
+    CHECK(dso.down(N) == scores);
+  }
+  CHECK(alloc.allocs == alloc.frees);
+}
+
+static void test_option_checks() {
+  using Table = HashTable<K, V, S, EvictStrategy::kEpochLru>;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = 1024;
+  o.max_hbm_for_vectors = GB(1);
+  auto expect_merlin = [&](HashTableOptions bad) {
+    bool threw = false;
+    try {
+      Table t;
+      t.init(bad);
+    } catch (const MerlinException&) {
+      threw = true;
+    }
+    CHECK(threw);
+  };
+  HashTableOptions b1 = o;
+  b1.reserved_key_start_bit = 63;
+  expect_merlin(b1);
+  HashTableOptions b2 = o;
+  b2.max_bucket_size = 100;
+  expect_merlin(b2);
+  HashTableOptions b3 = o;
+  b3.num_of_buckets_per_alloc = 3;
+  expect_merlin(b3);
+  Table t;
+  t.init(o);
+  DevBuf<K> dk(8);
+  DevBuf<V> dv(8 * 64);
+  bool threw = false;
+  try {  // epoch not set (merlin_hashtable.cuh:3853-3860)
+    t.insert_or_assign(8, dk.p, dv.p);
+  } catch (const MerlinException&) {
+    threw = true;
+  }
+  CHECK(threw);
+  t.set_global_epoch(1);
+  dk.up(random_keys(8, 5));
+  t.insert_or_assign(8, dk.p, dv.p);
+  CHECK(t.size() == 8);
+  threw = false;
+  try {
+    t.set_max_capacity(1000);
+  } catch (const std::invalid_argument&) {
+    threw = true;
+  }
+  CHECK(threw);
+  t.insert_or_assign(0, nullptr, nullptr);  // n == 0 is a no-op
+}
+
+int main() {
+  try {
+    test_basic();
+    test_evict_strategy_customized();
+    test_insert_and_evict_and_predicates();
+    test_allocator_hybrid_and_checkpoint();
+    test_option_checks();
+  } catch (const std::exception& e) {
+    std::printf("unexpected exception: %s\n", e.what());
+    return 2;
+  }
+  if (g_failures) {
+    std::printf("%d checks failed\n", g_failures);
+    return 1;
+  }
+  std::printf("api_test: all checks passed\n");
+  return 0;
+}

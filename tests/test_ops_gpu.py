@@ -1,0 +1,373 @@
+"""GPU parity for the remaining entry points and edge cases: pointer lookups,
+contains, missed-keys find, assign family, find_or_insert pointers, value type
+and dim matrix, ragged and empty batches, reserved keys, non-power-of-two
+capacity, LFU / EpochLFU arithmetic, hybrid mode, error behaviour, streams."""
+import numpy as np
+import pytest
+import torch
+
+import workloads as w
+from gpu_util import (DEV, assert_same_table, dev, export_table, host_bytes, host_u64,
+                      read_device, sort_by_key)
+from hierarchicalkv_amd import (EvictStrategy, HashTable, MerlinException, Predicate, ValueKind,
+                                default_options)
+
+pytestmark = pytest.mark.gpu
+M64 = (1 << 64) - 1
+
+
+def make_pair(oracle, hybrid=False, **kw):
+    kw.setdefault("max_hbm_for_vectors", 1 << 34)
+    o = default_options(**kw)
+    t = HashTable()
+    t.init(o)
+    return t, oracle.OracleTable(o, hybrid=hybrid), o
+
+
+def bytes_of(vals):
+    return np.ascontiguousarray(vals).view(np.uint8).reshape(len(vals), -1)
+
+
+def fill(t, o, seed, nbatch, bs, dim, scores_fn=None, start=0):
+    for b in range(nbatch):
+        keys = w.unique_keys(seed, start + b * bs, bs)
+        vals = w.uniform_values(seed, start + b * bs, bs, dim)
+        sc = scores_fn(b, bs) if scores_fn else None
+        t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+
+
+def test_find_ptr_contains_and_missed(oracle):
+    cap, dim, bs = 1 << 16, 24, 5000  # 96-byte rows, ragged batch size
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    fill(t, o, 41, 10, bs, dim, lambda b, n: w.monotone_scores(b + 1, n))
+    q = np.concatenate([w.unique_keys(41, 2 * bs + 17, 3001), w.unique_keys(42, 0, 2000),
+                        np.array([M64, M64 - 1, M64 - 2, M64 - 3], np.uint64)])
+    n = len(q)
+    # find* : pointers to the rows
+    ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+    scores = torch.zeros(n, dtype=torch.int64, device=DEV)
+    t.find_ptr(n, dev(q), ptrs, founds, scores)
+    torch.cuda.synchronize()
+    ov, of, osc = o.find(q)
+    gf = founds.cpu().numpy()
+    gp = ptrs.cpu().numpy()
+    assert (gf == of).all() and not gf[-4:].any()
+    assert ((gp != 0) == of).all()
+    assert (host_u64(scores)[gf] == osc[of]).all()
+    for i in np.flatnonzero(gf)[:: 97]:
+        assert (read_device(int(gp[i]), dim * 4) == ov[i]).all()
+    # contains
+    c = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.contains(n, dev(q), c)
+    torch.cuda.synchronize()
+    assert (c.cpu().numpy() == of).all()
+    # find with the missed-keys outputs
+    out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+    mk = torch.zeros(n, dtype=torch.int64, device=DEV)
+    mi = torch.zeros(n, dtype=torch.int32, device=DEV)
+    ms = torch.full((1,), 77, dtype=torch.int32, device=DEV)
+    t.find_missed(n, dev(q), out, mk, mi, ms)
+    torch.cuda.synchronize()
+    m = int(ms.item())
+    assert m == int((~of).sum())  # missed + found == n (find_with_missed_keys_test.cc.cu:32-212)
+    idx = np.sort(mi[:m].cpu().numpy())
+    assert (idx == np.flatnonzero(~of)).all()
+    order = np.argsort(mi[:m].cpu().numpy())
+    assert (host_u64(mk[:m])[order] == q[~of]).all()
+    assert (bytes_of(out.cpu().numpy())[of] == ov[of]).all()
+    t.close()
+
+
+@pytest.mark.parametrize("np_dtype,torch_dtype,kind,dim", [
+    (np.int8, torch.int8, ValueKind.kBytes, 3),
+    (np.uint8, torch.uint8, ValueKind.kBytes, 129),
+    (np.int16, torch.int16, ValueKind.kBytes, 66),
+    (np.int32, torch.int32, ValueKind.kI32, 202),
+    (np.float32, torch.float32, ValueKind.kF32, 224),
+    (np.float32, torch.float32, ValueKind.kF32, 3),
+    (np.float64, torch.float64, ValueKind.kF64, 128),
+    (np.int64, torch.int64, ValueKind.kI64, 5),
+])
+def test_value_types_and_dims(oracle, np_dtype, torch_dtype, kind, dim):
+    # the matrix of test_find_using_pipeline (merlin_hashtable_test.cc.cu:675-798, 3816-3830)
+    cap, bs = 1 << 14, 3000
+    esz = np.dtype(np_dtype).itemsize
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, value_size=esz,
+                        value_kind=kind, evict_strategy=EvictStrategy.kCustomized)
+    rng = np.random.Generator(np.random.PCG64(dim))
+    for b in range(7):  # past capacity: evictions with odd row sizes
+        keys = w.unique_keys(50, b * bs, bs)
+        vals = rng.integers(0, 256, size=(bs, dim * esz), dtype=np.uint8)
+        sc = w.monotone_scores(b + 1, bs)
+        t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+        o.insert_or_assign(keys, vals, sc)
+    assert_same_table(t, o, dim * esz)
+    q = w.unique_keys(50, 5 * bs, 2 * bs)
+    out = torch.zeros(len(q), dim * esz, dtype=torch.uint8, device=DEV)
+    founds = torch.zeros(len(q), dtype=torch.bool, device=DEV)
+    t.find(len(q), dev(q), out, founds, None)
+    torch.cuda.synchronize()
+    ov, of, _ = o.find(q)
+    assert (founds.cpu().numpy() == of).all() and of.any()
+    assert (out.cpu().numpy()[of] == ov[of]).all()
+    if kind != ValueKind.kBytes:
+        # accum_or_assign on every arithmetic element type
+        keys = q[: bs]
+        delta = (rng.integers(0, 100, size=(bs, dim)).astype(np_dtype))
+        flags = o.contains(keys)
+        t.accum_or_assign(bs, dev(keys), dev(bytes_of(delta)), dev(flags.astype(np.uint8)),
+                          dev(w.monotone_scores(9, bs)))
+        o.accum_or_assign(keys, bytes_of(delta), flags.astype(np.uint8), w.monotone_scores(9, bs))
+        assert_same_table(t, o, dim * esz)
+    t.close()
+
+
+def test_empty_ragged_and_reserved_batches(oracle):
+    cap, dim = 1 << 12, 8
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    t.insert_or_assign(0, None, None, None)  # n == 0: nothing is dereferenced
+    t.find(0, None, None, None)
+    t.erase(0, None)
+    assert t.size() == 0 and t.empty()
+    for n in (1, 63, 64, 65, 127, 1000):
+        keys = w.unique_keys(60 + n, 0, n)
+        keys[0] = np.uint64(M64 - (n % 4))  # a reserved key in every batch
+        vals = w.uniform_values(60, 0, n, dim)
+        sc = w.monotone_scores(n, n)
+        t.insert_or_assign(n, dev(keys), dev(vals), dev(sc))
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+        out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        founds = torch.ones(n, dtype=torch.bool, device=DEV)
+        t.find(n, dev(keys), out, founds, None)
+        torch.cuda.synchronize()
+        ov, of, _ = o.find(keys)
+        assert (founds.cpu().numpy() == of).all() and not of[0] and of[1:].all()
+        assert (bytes_of(out.cpu().numpy()) == ov).all()
+    assert_same_table(t, o, dim * 4)
+    t.close()
+
+
+def test_non_power_of_two_capacity_and_reserved_bit(oracle):
+    cap, dim, bs = 1000 * 128 - 129 + 128, 4, 1 << 13  # 1000 buckets
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, reserved_key_start_bit=17,
+                        evict_strategy=EvictStrategy.kCustomized)
+    assert t.bucket_count() == o.bucket_count() == 1000
+    assert t.capacity() == 128000
+    fill(t, o, 70, 20, bs, dim, lambda b, n: w.monotone_scores(b + 1, n))
+    # with start bit 17 the default sentinels are ordinary keys, the relocated ones are reserved
+    special = np.array([M64, M64 - 1, M64 - 2] + oracle.reserved_keys(17)[:3], np.uint64)
+    vals = w.uniform_values(71, 0, 6, dim)
+    sc = w.monotone_scores(30, 6)
+    t.insert_or_assign(6, dev(special), dev(vals), dev(sc))
+    o.insert_or_assign(special, bytes_of(vals), sc)
+    c = torch.zeros(6, dtype=torch.bool, device=DEV)
+    t.contains(6, dev(special), c)
+    torch.cuda.synchronize()
+    assert c.cpu().numpy().tolist() == o.contains(special).tolist() == [True] * 3 + [False] * 3
+    assert_same_table(t, o, dim * 4)
+    t.close()
+
+
+def test_assign_family_and_find_or_insert_ptr(oracle):
+    cap, dim, bs = 1 << 15, 16, 1 << 12
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    fill(t, o, 80, 6, bs, dim, lambda b, n: w.monotone_scores(b + 1, n))
+    keys = np.concatenate([w.unique_keys(80, 3 * bs, bs // 2), w.unique_keys(81, 0, bs // 2)])
+    vals = w.uniform_values(82, 0, bs, dim)
+    sc = w.monotone_scores(20, bs)
+    t.assign(bs, dev(keys), dev(vals), dev(sc))
+    o.assign(keys, bytes_of(vals), sc)
+    assert t.size() == o.size()
+    assert_same_table(t, o, dim * 4)
+    sc = w.monotone_scores(21, bs)
+    t.assign_scores(bs, dev(keys), dev(sc))
+    o.assign_scores(keys, sc)
+    vals = w.uniform_values(83, 0, bs, dim)
+    t.assign_values(bs, dev(keys), dev(vals))
+    o.assign_values(keys, bytes_of(vals))
+    assert_same_table(t, o, dim * 4)
+    # pointer overload of find_or_insert: hits report found, misses get a row to fill
+    keys = np.concatenate([w.unique_keys(80, 4 * bs, bs // 2), w.unique_keys(84, 0, bs // 2)])
+    sc = w.monotone_scores(22, bs)
+    ptrs = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.find_or_insert_ptr(bs, dev(keys), ptrs, founds, dev(sc))
+    torch.cuda.synchronize()
+    oslots, ofounds = o.find_or_insert_slot(keys, sc)
+    gf = founds.cpu().numpy()
+    assert (gf == ofounds.astype(bool)).all()
+    gp = ptrs.cpu().numpy()
+    assert ((gp != 0) == (oslots != np.uint64(M64))).all()
+    assert t.size() == o.size()
+    # every returned pointer is the row of its key: write through it, read back with find
+    vals = w.uniform_values(85, 0, bs, dim)
+    view = t.view()
+    slots = (gp - view.values) // (dim * 4)
+    assert (slots[gp != 0] >= 0).all() and (slots[gp != 0] < cap).all()
+    t.assign_values(bs, dev(keys), dev(vals))
+    torch.cuda.synchronize()
+    for i in range(0, bs, 211):
+        if gp[i]:
+            assert (read_device(int(gp[i]), dim * 4) == bytes_of(vals)[i]).all()
+    o.assign_values(keys, bytes_of(vals))
+    # rows of the new keys held whatever was there before; make both sides equal first
+    assert_same_table(t, o, dim * 4)
+    t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLfu, EvictStrategy.kEpochLfu])
+def test_frequency_strategies(oracle, strategy):
+    cap, dim, bs = 1 << 14, 4, 1 << 12
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, evict_strategy=strategy)
+    with pytest.raises(MerlinException):
+        t.insert_or_assign(4, dev(w.unique_keys(1, 0, 4)), dev(np.zeros((4, dim), np.float32)), None)
+    if strategy == EvictStrategy.kEpochLfu:
+        with pytest.raises(MerlinException):  # epoch not set
+            t.insert_or_assign(4, dev(w.unique_keys(1, 0, 4)), dev(np.zeros((4, dim), np.float32)),
+                               dev(np.ones(4, np.uint64)))
+        t.set_global_epoch(3)
+        o.set_global_epoch(3)
+    # distinct frequencies, larger for later batches, so victims are well defined and
+    # the keys re-used below are never the minimum of their bucket
+    freq = lambda b, n: np.uint64(1000 * (b + 1)) + np.arange(n, dtype=np.uint64) * np.uint64(7919) % np.uint64(997)
+    def distinct(b, n):
+        return (np.uint64(b + 1) << np.uint64(20)) + np.random.Generator(np.random.PCG64(b)).permutation(n).astype(np.uint64)
+    fill(t, o, 90, 6, bs, dim, distinct)
+    assert_same_table(t, o, dim * 4)
+    if strategy == EvictStrategy.kEpochLfu:
+        t.set_global_epoch(4)
+        o.set_global_epoch(4)
+    keys = np.concatenate([w.unique_keys(90, 5 * bs, bs // 2), w.unique_keys(91, 0, bs // 2)])
+    vals = w.uniform_values(92, 0, bs, dim)
+    sc = distinct(8, bs)
+    t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+    o.insert_or_assign(keys, bytes_of(vals), sc)
+    assert_same_table(t, o, dim * 4)
+    # saturation of the 32-bit frequency (kernel_utils.cuh:499-512)
+    if strategy == EvictStrategy.kEpochLfu:
+        k4 = keys[:4].copy()
+        big = np.array([0xFFFFFFF0, 0xFFFFFFFF, 0x1FFFFFFFF, 5], np.uint64)
+        t.insert_or_assign(4, dev(k4), dev(vals[:4]), dev(big))
+        o.insert_or_assign(k4, bytes_of(vals[:4]), big)
+        assert_same_table(t, o, dim * 4)
+    t.close()
+
+
+def test_hybrid_mode(oracle):
+    """Config 4 at reduced size: most value rows in pinned host memory, LFU,
+    find / find* with 80 % hits and insert_or_assign with 20 % new keys."""
+    cap, dim, bs = 1 << 16, 64, 1 << 12
+    t, o, opts = make_pair(oracle, hybrid=True, init_capacity=cap, max_capacity=cap, dim=dim,
+                           max_hbm_for_vectors=cap * dim * 4 // 4, evict_strategy=EvictStrategy.kLfu)
+    assert not t.is_pure_hbm()
+    v = t.view()
+    assert v.hbm_slots == cap // 4 and v.host_values
+
+    def distinct(b, n):
+        return (np.uint64(b + 1) << np.uint64(24)) + np.random.Generator(np.random.PCG64(100 + b)).permutation(n).astype(np.uint64)
+    nb = (cap + 4 * bs) // bs
+    fill(t, o, 95, nb, bs, dim, distinct)
+    assert t.size() == o.size()
+    assert_same_table(t, o, dim * 4)
+    recent = w.unique_keys(95, (nb - 2) * bs, bs)
+    q = np.concatenate([recent[: bs * 8 // 10], w.unique_keys(96, 0, bs - bs * 8 // 10)])
+    out = torch.zeros(bs, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    sc = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    t.find(bs, dev(q), out, founds, sc)
+    ptrs = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    f2 = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.find_ptr(bs, dev(q), ptrs, f2, None)
+    torch.cuda.synchronize()
+    ov, of, osc = o.find(q)
+    gf = founds.cpu().numpy()
+    assert (gf == of).all() and (f2.cpu().numpy() == of).all()
+    assert abs(of.mean() - 0.8) < 0.02
+    assert (bytes_of(out.cpu().numpy())[of] == ov[of]).all()
+    assert (host_u64(sc)[of] == osc[of]).all()
+    gp = ptrs.cpu().numpy()
+    in_host = (gp >= v.host_values) & (gp < v.host_values + (cap - v.hbm_slots) * dim * 4)
+    in_hbm = (gp >= v.values) & (gp < v.values + v.hbm_slots * dim * 4)
+    assert (in_host | in_hbm)[of].all() and in_host[of].mean() > 0.6
+    for i in np.flatnonzero(of)[:: 151]:
+        assert (read_device(int(gp[i]), dim * 4) == ov[i]).all()
+    # insert_or_assign with 20 % new keys
+    keys = np.concatenate([recent[: bs * 8 // 10], w.unique_keys(97, 0, bs - bs * 8 // 10)])
+    vals = w.uniform_values(98, 0, bs, dim)
+    s2 = distinct(nb + 3, bs)
+    t.insert_or_assign(bs, dev(keys), dev(vals), dev(s2))
+    o.insert_or_assign(keys, bytes_of(vals), s2)
+    assert_same_table(t, o, dim * 4)
+    # find_or_insert, and the refusal of insert_and_evict (merlin_hashtable.cuh:1384-1386)
+    keys = np.concatenate([recent[bs // 2: bs], w.unique_keys(99, 0, bs // 2)])
+    io = w.uniform_values(101, 0, bs, dim)
+    d_io = dev(io)
+    s3 = distinct(nb + 4, bs)
+    t.find_or_insert(bs, dev(keys), d_io, dev(s3))
+    oio = bytes_of(io).copy()
+    o.find_or_insert(keys, oio, s3)
+    torch.cuda.synchronize()
+    assert (host_bytes(d_io, bs, dim * 4) == oio).all()
+    assert_same_table(t, o, dim * 4)
+    with pytest.raises(RuntimeError):
+        t.insert_and_evict(bs, dev(keys), dev(io), dev(s3), torch.zeros(bs, dtype=torch.int64, device=DEV),
+                           torch.zeros(bs, dim, device=DEV), torch.zeros(bs, dtype=torch.int64, device=DEV))
+    t.close()
+
+
+def test_calls_on_two_streams_are_ordered_by_role(oracle):
+    """Writers and readers on different streams: the group lock orders them the
+    way the calls were issued (group_lock.cuh:43-56), without host syncs."""
+    cap, dim, bs = 1 << 16, 32, 1 << 14
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    keep = []
+    for b in range(6):
+        keys = w.unique_keys(110, b * bs, bs)
+        vals = w.uniform_values(110, b * bs, bs, dim)
+        sc = w.monotone_scores(b + 1, bs)
+        dk, dv, ds = dev(keys), dev(vals), dev(sc)
+        torch.cuda.synchronize()
+        t.insert_or_assign(bs, dk, dv, ds, stream=s1)
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+        out = torch.zeros(bs, dim, dtype=torch.float32, device=DEV)
+        founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+        t.find(bs, dk, out, founds, None, stream=s2)  # must see the insert issued just before
+        ov, of, _ = o.find(keys)
+        outs.append((out, founds, ov, of))
+        keep.append((dk, dv, ds))
+    torch.cuda.synchronize()
+    for out, founds, ov, of in outs:
+        gf = founds.cpu().numpy()
+        assert (gf == of).all()
+        assert (bytes_of(out.cpu().numpy())[of] == ov[of]).all()
+    assert_same_table(t, o, dim * 4)
+    t.close()
+
+
+def test_error_classes(oracle):
+    t = HashTable()
+    t.init(default_options(init_capacity=1024, max_capacity=1024, max_hbm_for_vectors=1 << 30, dim=4,
+                           evict_strategy=EvictStrategy.kLru))
+    k = dev(w.unique_keys(1, 0, 8))
+    v = dev(np.zeros((8, 4), np.float32))
+    with pytest.raises(MerlinException):  # LRU takes no scores (merlin_hashtable.cuh:3834-3839)
+        t.insert_or_assign(8, k, v, dev(np.ones(8, np.uint64)))
+    t.insert_or_assign(8, k, v, dev(np.ones(8, np.uint64)), ignore_evict_strategy=True)
+    assert t.size() == 8
+    with pytest.raises(ValueError):
+        t.export_batch_if(99, 0, 0, 10, 0, torch.zeros(1, dtype=torch.int64, device=DEV), k, v)
+    t2 = HashTable()
+    t2.init(default_options(init_capacity=1024, max_capacity=1024, max_hbm_for_vectors=1 << 30, dim=4,
+                            value_kind=ValueKind.kBytes, evict_strategy=EvictStrategy.kLru))
+    with pytest.raises(ValueError):
+        t2.accum_or_assign(8, k, v, torch.zeros(8, dtype=torch.bool, device=DEV))
+    t.close()
+    t2.close()
