@@ -158,8 +158,11 @@ def test_non_power_of_two_capacity_and_reserved_bit(oracle):
     assert t.bucket_count() == o.bucket_count() == 1000
     assert t.capacity() == 128000
     fill(t, o, 70, 20, bs, dim, lambda b, n: w.monotone_scores(b + 1, n))
-    # with start bit 17 the default sentinels are ordinary keys, the relocated ones are reserved
-    special = np.array([M64, M64 - 1, M64 - 2] + oracle.reserved_keys(17)[:3], np.uint64)
+    # with start bit 17 the sentinels move: EMPTY is all ones but bit 0 (the old RECLAIM
+    # value), while the old EMPTY and LOCKED values become ordinary keys
+    rk = oracle.reserved_keys(17)
+    assert rk[0] == M64 - 1
+    special = np.array([M64, M64 - 2, M64 - 4] + rk[:3], np.uint64)
     vals = w.uniform_values(71, 0, 6, dim)
     sc = w.monotone_scores(30, 6)
     t.insert_or_assign(6, dev(special), dev(vals), dev(sc))
