@@ -105,7 +105,9 @@ __device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
         s = (desired & kEpochMask) | kLow32;
     }
   }
-  st_u8(v.digests + slot, (uint8_t)digest);
+  /* a hit keeps its digest: the byte is only written when the slot changes
+   * owner (the reference rewrites the same value, kernel_utils.cuh:296-300) */
+  if (new_insert) st_u8(v.digests + slot, (uint8_t)digest);
   st_u64(v.scores + slot, s);
 }
 
@@ -170,7 +172,11 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
   if constexpr (!TABLE) {
     reinterpret_cast<T*>(row)[u] = x;
   } else if constexpr (VEC == 16) {
+#ifdef HKV_EXP_PLAIN_ROW_STORES
+    reinterpret_cast<T*>(row)[u] = x;
+#else
     st_u128(row + 16 * (size_t)u, x);
+#endif
   } else if constexpr (VEC == 4) {
     st_u32(reinterpret_cast<uint32_t*>(row) + u, x);
   } else {
@@ -183,8 +189,18 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
 #ifdef HKV_STATS
 __device__ unsigned long long g_hkv_stats[16];
 #define HKV_COUNT(slot, n) atomicAdd(&g_hkv_stats[slot], (unsigned long long)(n))
+/* phase timing: lane 0 adds the cycles since the previous mark to a counter */
+#define HKV_MARK_INIT() unsigned long long hkv_t_ = wall_clock64()
+#define HKV_MARK(slot)                                                   \
+  do {                                                                   \
+    const unsigned long long now_ = wall_clock64();                      \
+    if (threadIdx.x == 0) atomicAdd(&g_hkv_stats[slot], now_ - hkv_t_);  \
+    hkv_t_ = now_;                                                       \
+  } while (0)
 #else
 #define HKV_COUNT(slot, n) ((void)0)
+#define HKV_MARK_INIT() ((void)0)
+#define HKV_MARK(slot) ((void)0)
 #endif
 
 #ifndef HKV_SCAN_PAIR
@@ -453,12 +469,14 @@ upsert_kernel(View v, UpsertArgs a) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
 
+  HKV_MARK_INIT();
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
   s_unsure[lane] = 0;
   __syncthreads();
   probe_wave<true>(v, s_meta, s_slot, s_em, s_unsure, lane);
   __syncthreads();
+  HKV_MARK(9); /* probe */
 
   /* ---- state of the key this lane owns ---------------------------------------------- */
   const KeyMeta me = s_meta[lane];
@@ -537,6 +555,7 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
+    HKV_MARK(10); /* step 1 */
     /* ---- step 2: full buckets: min-score scan by the tile, two buckets in flight ------------ */
     uint64_t best = kMaxScore;
     uint32_t bpos = 0;
@@ -571,6 +590,7 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
+    HKV_MARK(11); /* scans */
     /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
     bool refused_now = false;
     if (want_scan) {
@@ -598,6 +618,7 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
+    HKV_MARK(12); /* victim lock */
     /* ---- step 4: critical sections of every lock taken in this trip ------------------------------ */
     const bool locked = got != kStNone && got != kStRefused;
     const uint64_t slot = bslot + pos;
@@ -659,8 +680,10 @@ upsert_kernel(View v, UpsertArgs a) {
             move, row, usr, units, a.value_kind, lane);
     }
 
+    HKV_MARK(13); /* meta + bulk issue */
     /* ---- step 5: everything written under the locks is out; release them --------------------------- */
     wait_stores();
+    HKV_MARK(14); /* store drain */
     if (locked) st_unlock(v.keys + slot, commit ? key : victim);
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
