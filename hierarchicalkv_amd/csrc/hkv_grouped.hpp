@@ -1,0 +1,901 @@
+/*
+ * Two-phase upserts: the large-batch path of insert_or_assign,
+ * insert_and_evict, find_or_insert and accum_or_assign.
+ *
+ * Same per-key semantics as the slot-lock kernel (hkv_upsert.hpp, after
+ * upsert.cuh:52-233, upsert_and_evict.cuh:27-1099, find_or_insert.cuh:27-1050,
+ * accum_or_assign.cuh:83-174); what changes is who may touch a slot.  An
+ * inserter runs alone on the table (the API-level group lock, as
+ * group_lock.cuh:43-56), so the only conflicts are between keys of the same
+ * batch, and only between keys that are absent: a key that is present owns its
+ * slot (keys of a batch are unique), absent keys of one bucket compete for its
+ * free slots and victims.  Hence two phases, each a kernel:
+ *
+ *   upsert_hits_kernel   every key is probed as in find.  A key that is present
+ *                        gets its new score and row at once, without a lock;
+ *                        an absent key goes to a list.
+ *   grouped_miss_kernel  the absent keys, partitioned by bucket.  Each bucket
+ *                        is owned by one 8-lane tile, which reads the digest
+ *                        line once and the 128 scores once, keeps both in
+ *                        registers, places its keys one after the other there
+ *                        (free slot, else minimum score, ties to the lowest
+ *                        slot), and writes back whole 64-byte pieces.
+ *
+ * The serial order this amounts to - all present keys, then the absent ones
+ * bucket by bucket - is one of the orders the slot-lock kernel could have
+ * produced.  What is saved: on this memory system an atomic on a random line
+ * costs about as much as moving two and a half full 128-byte lines and a
+ * scattered 8-byte store about one and a half, and the slot-lock protocol
+ * spends a CAS, an unlock store and two small loads per key on top of the
+ * score and digest stores; a bucket that takes several keys of a batch is
+ * scanned once instead of once per key.
+ *
+ * Partition of the absent keys: bins are aligned runs of 2^s buckets.
+ *   bin_hist_kernel      per-block histogram of the keys' bins (LDS)
+ *   bin_colscan_kernel   per bin: running sum over the blocks
+ *   bin_scatter_kernel   per block: scan of the bin totals, then every key's
+ *                        index goes to its place in `order`
+ * grouped_miss_kernel then runs one 256-thread workgroup per bin: counting
+ * sort of the bin's keys by bucket in LDS, and its 32 tiles take buckets from
+ * a work list.
+ */
+#ifndef HKV_GROUPED_HPP_
+#define HKV_GROUPED_HPP_
+
+#include "hkv_upsert.hpp"
+
+namespace hkv {
+
+constexpr int kBinThreads = 1024;   /* histogram / scatter workgroup */
+constexpr int kMaxBins = 8192;      /* LDS histogram: 32 KB */
+constexpr int kGrpThreads = 256;    /* grouped_upsert_kernel workgroup */
+constexpr int kGrpChunk = 512;      /* keys of a bin staged per pass */
+constexpr int kGrpMaxBpbShift = 10; /* at most 1024 buckets per bin */
+constexpr int kGrpMaxBpb = 1 << kGrpMaxBpbShift;
+constexpr int kGrpKeys = 2;         /* keys of one bucket handled per pass of a tile */
+
+struct BinArgs {
+  const uint64_t* keys;
+  const uint8_t* absent; /* per key of the batch: 1 = goes to the second phase */
+  uint64_t n;
+  uint32_t bpb_shift; /* buckets per bin = 1 << bpb_shift */
+  uint32_t nbins;
+  uint32_t blocks;    /* histogram blocks */
+  uint32_t slice;     /* keys per histogram block */
+  uint32_t* hist;     /* [blocks][nbins] */
+  uint32_t* total;    /* [nbins] */
+  uint32_t* bin_start; /* [nbins + 1] */
+  uint32_t* order;    /* [n] key indices grouped by bin */
+};
+
+/* bin of key i of the batch (never a reserved key: the probe filtered those) */
+__device__ __forceinline__ uint32_t bin_of(const View& v, const BinArgs& b, uint64_t key) {
+  uint32_t bkt, start, digest;
+  locate(v, key, bkt, start, digest);
+  return bkt >> b.bpb_shift;
+}
+
+constexpr int kBinUnroll = 8; /* keys a thread has in flight */
+
+__global__ void __launch_bounds__(kBinThreads)
+bin_hist_kernel(View v, BinArgs b) {
+  extern __shared__ uint32_t s_hist[];
+  for (uint32_t t = threadIdx.x; t < b.nbins; t += kBinThreads) s_hist[t] = 0;
+  __syncthreads();
+  const uint64_t lo = (uint64_t)blockIdx.x * b.slice;
+  const uint64_t hi = lo + b.slice < b.n ? lo + b.slice : b.n;
+  for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += (uint64_t)kBinThreads * kBinUnroll) {
+    uint64_t key[kBinUnroll];
+    uint8_t take[kBinUnroll];
+#pragma unroll
+    for (int e = 0; e < kBinUnroll; e++) {
+      const uint64_t i = i0 + (uint64_t)e * kBinThreads;
+      take[e] = 0;
+      key[e] = 0;
+      if (i < hi) {
+        take[e] = b.absent[i];
+        key[e] = b.keys[i];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < kBinUnroll; e++)
+      if (take[e]) atomicAdd(&s_hist[bin_of(v, b, key[e])], 1u);
+  }
+  __syncthreads();
+  uint32_t* out = b.hist + (uint64_t)blockIdx.x * b.nbins;
+  for (uint32_t t = threadIdx.x; t < b.nbins; t += kBinThreads) out[t] = s_hist[t];
+}
+
+/* hist[g][bin] becomes the number of keys of that bin in blocks before g.
+ * The column is read kColBatch entries at a time, loads before stores. */
+constexpr int kMaxHistBlocks = 128;
+constexpr int kColBatch = 32;
+__global__ void __launch_bounds__(256)
+bin_colscan_kernel(BinArgs b) {
+  const uint32_t bin = blockIdx.x * 256 + threadIdx.x;
+  if (bin >= b.nbins) return;
+  uint32_t run = 0;
+  for (uint32_t g0 = 0; g0 < b.blocks; g0 += kColBatch) {
+    uint32_t c[kColBatch];
+#pragma unroll
+    for (int g = 0; g < kColBatch; g++)
+      c[g] = g0 + g < b.blocks ? b.hist[(uint64_t)(g0 + g) * b.nbins + bin] : 0u;
+#pragma unroll
+    for (int g = 0; g < kColBatch; g++) {
+      if (g0 + g < b.blocks) b.hist[(uint64_t)(g0 + g) * b.nbins + bin] = run;
+      run += c[g];
+    }
+  }
+  b.total[bin] = run;
+}
+
+__global__ void __launch_bounds__(kBinThreads)
+bin_scatter_kernel(View v, BinArgs b) {
+  extern __shared__ uint32_t s_cursor[]; /* [nbins] */
+  __shared__ uint32_t s_wave[kBinThreads / kWave];
+  /* exclusive scan of total[]: thread t owns the bins [t * per, t * per + per) */
+  const uint32_t per = (b.nbins + kBinThreads - 1) / kBinThreads;
+  const uint32_t b0 = threadIdx.x * per;
+  uint32_t sum = 0;
+  for (uint32_t e = 0; e < per; e++)
+    if (b0 + e < b.nbins) sum += b.total[b0 + e];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t inc = sum;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t y = __shfl_up(inc, off);
+    if (lane >= off) inc += y;
+  }
+  if (lane == kWave - 1) s_wave[wave] = inc;
+  __syncthreads();
+  uint32_t run = inc - sum;
+  for (int w = 0; w < wave; w++) run += s_wave[w];
+  const uint32_t* rel = b.hist + (uint64_t)blockIdx.x * b.nbins;
+  for (uint32_t e = 0; e < per; e++) {
+    const uint32_t bin = b0 + e;
+    if (bin < b.nbins) {
+      if (blockIdx.x == 0) b.bin_start[bin] = run;
+      s_cursor[bin] = run + rel[bin];
+      run += b.total[bin];
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == kBinThreads - 1) b.bin_start[b.nbins] = run;
+  __syncthreads();
+  const uint64_t lo = (uint64_t)blockIdx.x * b.slice;
+  const uint64_t hi = lo + b.slice < b.n ? lo + b.slice : b.n;
+  for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += (uint64_t)kBinThreads * kBinUnroll) {
+    uint64_t key[kBinUnroll];
+    uint8_t take[kBinUnroll];
+#pragma unroll
+    for (int e = 0; e < kBinUnroll; e++) {
+      const uint64_t i = i0 + (uint64_t)e * kBinThreads;
+      take[e] = 0;
+      key[e] = 0;
+      if (i < hi) {
+        take[e] = b.absent[i];
+        key[e] = b.keys[i];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < kBinUnroll; e++)
+      if (take[e])
+        b.order[atomicAdd(&s_cursor[bin_of(v, b, key[e])], 1u)] =
+            (uint32_t)(i0 + (uint64_t)e * kBinThreads);
+  }
+}
+
+/* ---- register-resident bucket state ------------------------------------------------ */
+
+/* byte `p` (0..15) of the 16 digest bytes a lane holds; selects and shifts
+ * only, so that the four words stay in registers */
+__device__ __forceinline__ uint32_t dg_byte(const uint4& d, uint32_t p) {
+  const uint32_t a = (p & 8u) ? d.z : d.x;
+  const uint32_t b = (p & 8u) ? d.w : d.y;
+  const uint32_t x = (p & 4u) ? b : a;
+  return (x >> ((p & 3u) * 8)) & 0xFFu;
+}
+__device__ __forceinline__ void dg_set(uint4& d, uint32_t p, uint32_t byte) {
+  const uint32_t sh = (p & 3u) * 8;
+  const uint32_t clr = 0xFFu << sh, put = byte << sh;
+  const uint32_t w = p >> 2;
+  const uint32_t c0 = w == 0 ? clr : 0u, c1 = w == 1 ? clr : 0u, c2 = w == 2 ? clr : 0u,
+                 c3 = w == 3 ? clr : 0u;
+  d.x = (d.x & ~c0) | (put & c0);
+  d.y = (d.y & ~c1) | (put & c1);
+  d.z = (d.z & ~c2) | (put & c2);
+  d.w = (d.w & ~c3) | (put & c3);
+}
+
+/* The 128 scores of a bucket over the 8 lanes of a tile: lane j holds the
+ * positions {16 it + 2 j, 16 it + 2 j + 1}, the layout of scan_reduce. */
+__device__ __forceinline__ void scores_load(const View& v, uint64_t bslot, int j, uint64_t* sc) {
+#pragma unroll
+  for (int it = 0; it < kTile; it++) {
+    const uint4 t = *reinterpret_cast<const uint4*>(v.scores + bslot + it * 16 + j * 2);
+    sc[2 * it] = t.x | ((uint64_t)t.y << 32);
+    sc[2 * it + 1] = t.z | ((uint64_t)t.w << 32);
+  }
+}
+__device__ __forceinline__ void scores_patch(uint64_t* sc, int j, uint32_t pos, uint64_t s) {
+  const bool mine = (int)((pos & 15u) >> 1) == j;
+  const uint32_t e = 2 * (pos >> 4) + (pos & 1u);
+#pragma unroll
+  for (uint32_t q = 0; q < 2 * kTile; q++)
+    if (mine && q == e) sc[q] = s;
+}
+/* write back the 64-byte pieces named in `dirty` (bit c: positions 8c..8c+7) */
+__device__ __forceinline__ void scores_flush(const View& v, uint64_t bslot, int j,
+                                             const uint64_t* sc, uint32_t dirty) {
+#pragma unroll
+  for (int it = 0; it < kTile; it++) {
+    if ((dirty >> (2 * it + (j >> 2))) & 1u) {
+      const uint4 t = make_uint4((uint32_t)sc[2 * it], (uint32_t)(sc[2 * it] >> 32),
+                                 (uint32_t)sc[2 * it + 1], (uint32_t)(sc[2 * it + 1] >> 32));
+      st_u128(v.scores + bslot + it * 16 + j * 2, t);
+    }
+  }
+}
+
+/* ScoreFunctor<Strategy>::update_with_digest (kernel_utils.cuh:291-302,
+ * 353-371, 422-434, 490-517, 581-593) as a value: the score an accepted key
+ * leaves in its slot; false when the score stays as it is. */
+__device__ __forceinline__ bool final_score(const UpsertArgs& a, bool new_insert, uint64_t desired,
+                                            uint64_t in_score, uint64_t old, uint64_t& s) {
+  const int STRATEGY = a.strategy;
+  s = desired;
+  if (STRATEGY == HKV_LFU) {
+    if (!a.scores) return false;
+    s = new_insert ? in_score : in_score + old;
+  } else if (STRATEGY == HKV_EPOCH_LFU) {
+    if (!new_insert) {
+      s = old & kLow32;
+      if (kLow32 - s > (desired & kLow32))
+        s += desired;
+      else
+        s = (desired & kEpochMask) | kLow32;
+    }
+  }
+  return true;
+}
+
+struct GroupArgs {
+  const uint32_t* order;
+  const uint32_t* bin_start;
+  uint32_t bpb_shift;
+  uint32_t locked_rule; /* refuse when score <= min, not < (upsert.cuh:1478-1524) */
+};
+
+struct HitArgs {
+  uint8_t* absent; /* [n] out: 1 = the key goes to the second phase */
+};
+
+/*
+ * Phase 1.  One wavefront per 64 keys, as lookup_kernel: probe, then
+ *   present  new score (update_with_digest with the slot's old score where the
+ *            strategy needs it) and the row traffic of the operation, the whole
+ *            wavefront moving the rows of its keys, VEC bytes per lane;
+ *   absent   flagged for the second phase.
+ * accum_or_assign drops the keys whose flag disagrees with what was found
+ * (accum_or_assign.cuh:139-156).
+ */
+template <int OP, int VEC>
+__global__ void __launch_bounds__(kWave)
+upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
+  __shared__ KeyMeta s_meta[kWave];
+  __shared__ int64_t s_slot[kWave];
+  const int lane = threadIdx.x;
+  const uint64_t base = (uint64_t)blockIdx.x * kWave;
+  const uint64_t i = base + lane;
+  stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
+  const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
+  __syncthreads();
+  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  __syncthreads();
+
+  const bool valid = (s_meta[lane].info & 0x100u) != 0;
+  const int64_t slot = s_slot[lane];
+  bool hit = valid && slot >= 0;
+  bool miss = valid && slot < 0;
+  if (OP == kOpAccumOrAssign && valid) {
+    const bool is_accum = a.accum_flags[i] != 0;
+    if (hit && !is_accum) hit = false;
+    if (miss && is_accum) miss = false;
+  }
+  if (i < a.n) h.absent[i] = miss;
+  if (hit) {
+    const uint64_t desired = desired_when_missed(a, in_score, i);
+    const bool needs_old = a.strategy == HKV_LFU || a.strategy == HKV_EPOCH_LFU;
+    const uint64_t old = needs_old ? v.scores[slot] : 0;
+    uint64_t snew;
+    if (final_score(a, false, desired, in_score, old, snew)) v.scores[slot] = snew;
+  }
+  if (OP == kOpAccumOrAssign) {
+    /* rows move for the keys that stay "present" only */
+    __syncthreads();
+    if (!hit) s_slot[lane] = -1;
+    __syncthreads();
+  }
+
+  /* rows: 64 rows x units-per-row spread over the 64 lanes; all loads of a
+   * batch are issued before the first store */
+  using T = typename VecType<VEC>::type;
+  const uint32_t units = v.value_bytes / VEC;
+  const uint32_t total = units * kWave;
+  const bool pow2 = (units & (units - 1)) == 0;
+  const uint32_t sh = 31 - __clz(units);
+  constexpr int kBatch = VEC == 16 ? (OP == kOpAccumOrAssign ? 8 : 16) : 4;
+  uint8_t* usr_base = (OP == kOpFindOrInsert ? a.values_io : const_cast<uint8_t*>(a.values_in)) +
+                      base * v.value_bytes;
+  for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
+    T buf[kBatch];
+    T tab[OP == kOpAccumOrAssign ? kBatch : 1];
+#pragma unroll
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * kWave;
+      buf[b] = T{};
+      if (OP == kOpAccumOrAssign) tab[b] = T{};
+      if (idx < total) {
+        const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
+        const uint32_t c = idx - kk * units;
+        const int64_t sl = s_slot[kk];
+        if (sl >= 0) {
+          if (OP == kOpFindOrInsert) {
+            buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
+          } else {
+            buf[b] = reinterpret_cast<const T*>(usr_base + (uint64_t)kk * v.value_bytes)[c];
+            if (OP == kOpAccumOrAssign)
+              tab[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * kWave;
+      if (idx < total) {
+        const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
+        const uint32_t c = idx - kk * units;
+        const int64_t sl = s_slot[kk];
+        if (sl >= 0) {
+          if (OP == kOpFindOrInsert) {
+            reinterpret_cast<T*>(usr_base + (uint64_t)kk * v.value_bytes)[c] = buf[b];
+          } else if (OP == kOpAccumOrAssign) {
+            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, add_unit(tab[b], buf[b], a.value_kind));
+          } else {
+            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
+          }
+        }
+      }
+    }
+  }
+}
+
+/* ---- cross-lane moves inside an 8-lane tile without the LDS permute unit -------------------- */
+
+/* value of the partner lane (lane ^ 1, lane ^ 2: data-parallel moves inside a
+ * quad; lane ^ 4: one swizzle) */
+__device__ __forceinline__ uint32_t xor1_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, true); /* quad_perm [1,0,3,2] */
+}
+__device__ __forceinline__ uint32_t xor2_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true); /* quad_perm [2,3,0,1] */
+}
+__device__ __forceinline__ uint32_t xor4_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x101F); /* and 0x1f, or 0, xor 4 */
+}
+/* lane 0 of the tile to all its lanes */
+__device__ __forceinline__ uint32_t tile_first_u32(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x0018); /* and 0x18, or 0, xor 0 */
+}
+
+/* minimum score of the bucket and its slot; ties go to the lowest slot, as the
+ * reference's sequential scan with a strict '<' (upsert.cuh:166-183) */
+__device__ __forceinline__ void tile_min(const uint64_t* sc, int j, uint64_t& best, uint32_t& bpos) {
+  best = sc[0];
+  uint32_t e = 0;
+#pragma unroll
+  for (uint32_t q = 1; q < 2 * kTile; q++) {
+    /* register q holds slot 16 (q >> 1) + 2 j + (q & 1): slots grow with q */
+    if (sc[q] < best) {
+      best = sc[q];
+      e = q;
+    }
+  }
+  bpos = (e >> 1) * 16 + 2 * (uint32_t)j + (e & 1u);
+#define HKV_TILE_MIN_STEP(FN)                                                  \
+  {                                                                            \
+    const uint64_t ob = (uint64_t)FN((uint32_t)best) | ((uint64_t)FN((uint32_t)(best >> 32)) << 32); \
+    const uint32_t op = FN(bpos);                                              \
+    if (ob < best || (ob == best && op < bpos)) {                              \
+      best = ob;                                                               \
+      bpos = op;                                                               \
+    }                                                                          \
+  }
+  HKV_TILE_MIN_STEP(xor1_u32)
+  HKV_TILE_MIN_STEP(xor2_u32)
+  HKV_TILE_MIN_STEP(xor4_u32)
+#undef HKV_TILE_MIN_STEP
+}
+
+/*
+ * Phase 2, one bucket: the absent keys of the batch that fall into bucket
+ * `bkt` are the entries [sb, se) of the sorted LDS arrays.  Called by the 8
+ * lanes of a tile together; `lane` is the lane inside the wavefront.  `dg` is
+ * the lane's 16 bytes of the bucket's digest line; `sc` holds the bucket's scores
+ * already when sc_loaded says so (the caller asks for them ahead of time when
+ * the digest line shows no free slot).
+ *
+ * Everything that steers the work (which key goes where, what it displaces) is
+ * computed by all 8 lanes alike from the same LDS entries, so the lanes agree
+ * without talking; only the minimum search and the free-slot mask cross lanes.
+ */
+template <int OP, int VEC, int UPL>
+__device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
+                                             const GroupArgs& g, uint32_t bkt, uint32_t sb,
+                                             uint32_t se, const uint64_t* s_key,
+                                             const uint32_t* s_idx, const uint32_t* s_info,
+                                             uint32_t units, int lane, uint4 dg, uint64_t* sc,
+                                             bool sc_loaded) {
+  const int j = lane & (kTile - 1);
+  const int tile = lane >> 3;
+  const int tile_base = lane & ~(kTile - 1);
+  const uint64_t bslot = (uint64_t)bkt * kBucketSize;
+  const uint8_t* rows_in = OP == kOpFindOrInsert ? a.values_io : a.values_in;
+
+  bool dg_dirty = false;
+  int size_delta = 0;
+
+  /* free slots of the bucket, bit p for slot p */
+  uint64_t em_lo = 0, em_hi = 0;
+  {
+    const uint32_t m16 = match16_natural(dg, v.empty_digest * 0x01010101u);
+    if (tile_ballot(m16 != 0, tile)) {
+#pragma unroll
+      for (int q = 0; q < kTile; q++) {
+        const uint64_t m = __shfl(m16, tile_base + q) & 0xFFFFu;
+        if (q < 4)
+          em_lo |= m << (16 * q);
+        else
+          em_hi |= m << (16 * (q - 4));
+      }
+    }
+  }
+
+  for (uint32_t q0 = sb; q0 < se; q0 += kGrpKeys) {
+    const int mg = (int)(se - q0) < kGrpKeys ? (int)(se - q0) : kGrpKeys;
+    /* a later pass may read what an earlier one wrote (a victim's key and row) */
+    if (q0 != sb) wait_stores();
+
+    /* ---- the rows the keys came with: asked for now, stored when the slot is known ------------ */
+    constexpr bool kPre = VEC == 16 && UPL <= 2;
+    using T = typename VecType<VEC>::type;
+    T xin[kPre ? kGrpKeys : 1][kPre ? UPL : 1];
+    if constexpr (kPre) {
+#pragma unroll
+      for (int q = 0; q < kGrpKeys; q++) {
+        const uint8_t* us = rows_in + (uint64_t)s_idx[q < mg ? q0 + q : sb] * v.value_bytes;
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = j + w * kTile;
+          xin[q][w] = T{};
+          if (q < mg && u < units) xin[q][w] = ld_unit<VEC, false>(us, u);
+        }
+      }
+    }
+
+    /* outcome of key q of the pass, the same in every lane of the tile */
+    int got[kGrpKeys];
+    uint32_t pos[kGrpKeys];
+    uint64_t snew[kGrpKeys];
+    uint64_t best_seen[kGrpKeys];
+    bool wrs[kGrpKeys], cancelled[kGrpKeys], need_vk[kGrpKeys];
+    int vic_from[kGrpKeys];
+    uint32_t dirty = 0; /* 64-byte score pieces changed in this pass */
+
+    /* ---- the keys of the pass, one after the other -------------------------------------------------- */
+#pragma unroll
+    for (int q = 0; q < kGrpKeys; q++) {
+      got[q] = kStNone;
+      pos[q] = 0;
+      snew[q] = 0;
+      best_seen[q] = 0;
+      wrs[q] = false;
+      cancelled[q] = false;
+      need_vk[q] = false;
+      vic_from[q] = -1;
+      if (q >= mg) continue;
+      const uint64_t kq = s_key[q0 + q];
+      const uint64_t iq = s_idx[q0 + q];
+      const uint32_t info = s_info[q0 + q];
+      const uint64_t in_score = a.scores ? a.scores[iq] : 0;
+      const uint64_t dq = desired_when_missed(a, in_score, iq);
+      wrs[q] = final_score(a, true, dq, in_score, 0, snew[q]);
+      const uint64_t sq = snew[q];
+      /* the same key earlier in this pass (batches are meant to hold unique
+       * keys): the first one wins, this one changes nothing */
+      bool dup = false;
+#pragma unroll
+      for (int p = 0; p < q; p++)
+        dup |= (got[p] == kStEmpty || got[p] == kStEvict) && s_key[q0 + p] == kq;
+      if (dup) {
+        got[q] = kStDuplicate;
+        cancelled[q] = true;
+        continue;
+      }
+      if (em_lo | em_hi) {
+        const uint32_t p = first_from(em_lo, em_hi, (info >> 8) & 0x7Fu);
+        if (p < 64)
+          em_lo &= ~(UINT64_C(1) << p);
+        else
+          em_hi &= ~(UINT64_C(1) << (p - 64));
+        got[q] = kStEmpty;
+        pos[q] = p;
+        if (j == (int)(p >> 4)) dg_set(dg, p & 15u, info & 0xFFu);
+        dg_dirty = true;
+        size_delta++;
+        if (sc_loaded && wrs[q]) {
+          scores_patch(sc, j, p, sq);
+          dirty |= 1u << (p >> 3);
+        }
+        continue;
+      }
+      if (!sc_loaded) {
+        /* scores stored one by one earlier in this call must have landed */
+        wait_stores();
+        scores_load(v, bslot, j, sc);
+        sc_loaded = true;
+        /* keys of this pass that went into free slots have not stored their
+         * scores yet: the registers are the truth from here on */
+#pragma unroll
+        for (int r = 0; r < q; r++) {
+          if (got[r] == kStEmpty && wrs[r]) {
+            scores_patch(sc, j, pos[r], snew[r]);
+            dirty |= 1u << (pos[r] >> 3);
+          }
+        }
+      }
+      uint64_t best;
+      uint32_t bpos;
+      tile_min(sc, j, best, bpos);
+      const bool refuse = g.locked_rule ? (dq <= best) : (dq < best);
+      if (refuse) {
+        got[q] = kStRefused;
+        continue;
+      }
+      /* the slot may belong to a key of this very pass (one that has just been
+       * inserted with a low score): that key's writes are dropped, it leaves
+       * through the eviction */
+#pragma unroll
+      for (int p = 0; p < q; p++) {
+        if (!cancelled[p] && pos[p] == bpos && (got[p] == kStEmpty || got[p] == kStEvict)) {
+          cancelled[p] = true;
+          vic_from[q] = p;
+        }
+      }
+      /* kStReclaimed is told apart from kStEvict by the key word, which is read
+       * only when somebody needs it: a tombstone always carries the tombstone digest */
+      const bool tomb_digest =
+          tile_ballot(j == (int)(bpos >> 4) && dg_byte(dg, bpos & 15u) == v.reclaim_digest, tile) != 0;
+      got[q] = kStEvict;
+      need_vk[q] = vic_from[q] < 0 && (OP == kOpInsertAndEvict || tomb_digest);
+      pos[q] = bpos;
+      best_seen[q] = best;
+      /* a strategy that leaves the score alone still has to hide the slot from
+       * the next scan of this pass; the piece is written back only if it changed */
+      scores_patch(sc, j, bpos, wrs[q] ? sq : kMaxScore);
+      if (wrs[q]) dirty |= 1u << (bpos >> 3);
+      if (j == (int)(bpos >> 4)) dg_set(dg, bpos & 15u, info & 0xFFu);
+      dg_dirty = true;
+    }
+
+    /* ---- victims: live key or tombstone ------------------------------------------------------------- */
+    uint64_t victim[kGrpKeys];
+#pragma unroll
+    for (int q = 0; q < kGrpKeys; q++) {
+      victim[q] = 0;
+      if (got[q] == kStEvict && need_vk[q]) victim[q] = v.keys[bslot + pos[q]];
+    }
+#pragma unroll
+    for (int q = 0; q < kGrpKeys; q++) {
+      if (got[q] == kStEvict && need_vk[q] && victim[q] == v.reclaim_key) {
+        got[q] = kStReclaimed;
+        size_delta++;
+      }
+#pragma unroll
+      for (int p = 0; p < q; p++)
+        if (vic_from[q] == p) victim[q] = s_key[q0 + p];
+    }
+
+    /* ---- what leaves the table (upsert_and_evict.cuh:188-194, 218-224, 236-245) ------------------------ */
+    if (OP == kOpInsertAndEvict) {
+      int emits = 0;
+#pragma unroll
+      for (int q = 0; q < kGrpKeys; q++) emits += (got[q] == kStRefused || got[q] == kStEvict);
+      if (emits) {
+        uint32_t lo = 0, hi = 0;
+        if (j == 0) {
+          const unsigned long long b = atomicAdd(a.evicted_counter, (unsigned long long)emits);
+          lo = (uint32_t)b;
+          hi = (uint32_t)(b >> 32);
+        }
+        unsigned long long idx = tile_first_u32(lo) | ((unsigned long long)tile_first_u32(hi) << 32);
+#pragma unroll
+        for (int q = 0; q < kGrpKeys; q++) {
+          const bool refused_now = got[q] == kStRefused;
+          if (!(refused_now || got[q] == kStEvict)) continue;
+          const uint64_t iq = s_idx[q0 + q];
+          if (j == 0) {
+            a.evicted_keys[idx] = refused_now ? s_key[q0 + q] : victim[q];
+            if (a.evicted_scores) {
+              const uint64_t in_score = a.scores ? a.scores[iq] : 0;
+              a.evicted_scores[idx] = refused_now ? desired_when_missed(a, in_score, iq) : best_seen[q];
+            }
+          }
+          /* a refused key leaves with its own row, a victim that is a key of this
+           * pass with the row it came with, any other victim with its table row */
+          const uint8_t* src;
+          bool table = false;
+          if (refused_now) {
+            src = a.values_in + iq * v.value_bytes;
+          } else if (vic_from[q] >= 0) {
+            uint64_t ifrom = 0;
+#pragma unroll
+            for (int p = 0; p < q; p++)
+              if (vic_from[q] == p) ifrom = s_idx[q0 + p];
+            src = a.values_in + ifrom * v.value_bytes;
+          } else {
+            src = value_row(v, bslot + pos[q]);
+            table = true;
+          }
+          uint8_t* dst = a.evicted_values + idx * v.value_bytes;
+          for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
+            T x[UPL];
+#pragma unroll
+            for (int w = 0; w < UPL; w++) {
+              const uint32_t u = u0 + j + w * kTile;
+              x[w] = T{};
+              if (u < units) x[w] = table ? ld_unit<VEC, true>(src, u) : ld_unit<VEC, false>(src, u);
+            }
+#pragma unroll
+            for (int w = 0; w < UPL; w++) {
+              const uint32_t u = u0 + j + w * kTile;
+              if (u < units) st_unit<VEC, false>(dst, u, x[w]);
+            }
+          }
+          idx++;
+        }
+      }
+    }
+
+    /* ---- key, score, row of every key that stays -------------------------------------------------------- */
+#pragma unroll
+    for (int q = 0; q < kGrpKeys; q++) {
+      const bool writes =
+          (got[q] == kStEmpty || got[q] == kStReclaimed || got[q] == kStEvict) && !cancelled[q];
+      if (!writes) continue;
+      const uint64_t slot = bslot + pos[q];
+      if (j == 0) {
+        v.keys[slot] = s_key[q0 + q];
+        if (wrs[q] && !sc_loaded) v.scores[slot] = snew[q];
+      }
+      uint8_t* tb = value_row(v, slot);
+      if constexpr (kPre) {
+#pragma unroll
+        for (int w = 0; w < UPL; w++) {
+          const uint32_t u = j + w * kTile;
+          if (u < units) st_unit<VEC, true>(tb, u, xin[q][w]);
+        }
+      } else {
+        const uint8_t* us = rows_in + (uint64_t)s_idx[q0 + q] * v.value_bytes;
+        for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
+          T x[UPL];
+#pragma unroll
+          for (int w = 0; w < UPL; w++) {
+            const uint32_t u = u0 + j + w * kTile;
+            x[w] = T{};
+            if (u < units) x[w] = ld_unit<VEC, false>(us, u);
+          }
+#pragma unroll
+          for (int w = 0; w < UPL; w++) {
+            const uint32_t u = u0 + j + w * kTile;
+            if (u < units) st_unit<VEC, true>(tb, u, x[w]);
+          }
+        }
+      }
+    }
+    if (sc_loaded && dirty) scores_flush(v, bslot, j, sc, dirty);
+  }
+
+  if (dg_dirty) st_u128(v.digests + bslot + j * 16, dg);
+  if (size_delta && j == 0) atomicAdd(v.sizes + bkt, size_delta);
+}
+
+#ifndef HKV_GROUPED_MIN_WAVES
+#define HKV_GROUPED_MIN_WAVES 1
+#endif
+template <int OP, int VEC, int UPL>
+__global__ void __launch_bounds__(kGrpThreads, HKV_GROUPED_MIN_WAVES)
+grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
+  __shared__ uint64_t s_key[kGrpChunk];
+  __shared__ uint32_t s_idx[kGrpChunk];
+  __shared__ uint32_t s_info[kGrpChunk]; /* digest | start << 8 | bucket inside the bin << 16 */
+  __shared__ uint32_t s_seg[kGrpMaxBpb + 1];
+  __shared__ uint32_t s_cur[kGrpMaxBpb];
+  __shared__ uint16_t s_work[kGrpMaxBpb];
+  __shared__ uint32_t s_wsum[kGrpThreads / kWave];
+  __shared__ uint32_t s_nwork, s_next;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const uint32_t bin = blockIdx.x;
+  const uint32_t bpb = 1u << g.bpb_shift;
+  const uint32_t first = g.bin_start[bin], last = g.bin_start[bin + 1];
+  const uint32_t units = v.value_bytes / VEC;
+
+#ifdef HKV_STATS
+  const unsigned long long t_begin = wall_clock64();
+  unsigned long long t_setup = 0, t_loop = 0;
+#endif
+  for (uint32_t c0 = first; c0 < last; c0 += kGrpChunk) {
+#ifdef HKV_STATS
+    const unsigned long long t_c0 = wall_clock64();
+#endif
+    const uint32_t cn = last - c0 < (uint32_t)kGrpChunk ? last - c0 : (uint32_t)kGrpChunk;
+    for (uint32_t t = tid; t <= bpb; t += kGrpThreads) s_seg[t] = 0;
+    if (tid == 0) {
+      s_nwork = 0;
+      s_next = 0;
+    }
+    __syncthreads();
+
+    /* ---- stage: two keys per thread, counted by bucket ----------------------------------------- */
+    uint64_t mk[2];
+    uint32_t mi[2], minfo[2];
+    bool have[2];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      const uint32_t p = tid + e * kGrpThreads;
+      have[e] = p < cn;
+      mk[e] = 0;
+      mi[e] = 0;
+      minfo[e] = 0;
+      if (have[e]) {
+        mi[e] = g.order[c0 + p];
+        mk[e] = a.keys[mi[e]];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      if (have[e]) {
+        uint32_t bkt, start, digest;
+        locate(v, mk[e], bkt, start, digest);
+        const uint32_t lb = bkt - (bin << g.bpb_shift);
+        minfo[e] = digest | (start << 8) | (lb << 16);
+        atomicAdd(&s_seg[lb], 1u);
+      }
+    }
+    __syncthreads();
+
+    /* ---- exclusive scan of the counts; list of the buckets that have keys ---------------------------- */
+    {
+      uint32_t c[4], sum = 0;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t t = tid * 4 + e;
+        c[e] = t < bpb ? s_seg[t] : 0;
+        sum += c[e];
+      }
+      uint32_t inc = sum;
+#pragma unroll
+      for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t y = __shfl_up(inc, off);
+        if (lane >= off) inc += y;
+      }
+      if (lane == kWave - 1) s_wsum[tid >> 6] = inc;
+      __syncthreads();
+      uint32_t run = inc - sum;
+      for (int w = 0; w < (tid >> 6); w++) run += s_wsum[w];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t t = tid * 4 + e;
+        if (t < bpb) {
+          s_seg[t] = run;
+          s_cur[t] = run;
+          if (c[e]) s_work[atomicAdd(&s_nwork, 1u)] = (uint16_t)t;
+          run += c[e];
+        }
+      }
+      if (tid == kGrpThreads - 1) s_seg[bpb] = run;
+    }
+    __syncthreads();
+
+    /* ---- place ------------------------------------------------------------------------------------------ */
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+      if (have[e]) {
+        const uint32_t p = atomicAdd(&s_cur[minfo[e] >> 16], 1u);
+        s_key[p] = mk[e];
+        s_idx[p] = mi[e];
+        s_info[p] = minfo[e];
+      }
+    }
+    __syncthreads();
+
+    /* ---- tiles take buckets from the work list; the digest line of the next
+     * bucket is asked for before the current one is worked on ---------------------------------------------- */
+    const uint32_t nwork = s_nwork;
+    const int tile_base = lane & ~(kTile - 1);
+    const int j = lane & (kTile - 1);
+    const uint32_t bkt0 = bin << g.bpb_shift;
+    auto take = [&]() {
+      uint32_t w = 0;
+      if (j == 0) w = atomicAdd(&s_next, 1u);
+      return (uint32_t)__shfl(w, tile_base);
+    };
+    auto digests_of = [&](uint32_t w) {
+      return *reinterpret_cast<const uint4*>(v.digests + (uint64_t)(bkt0 + s_work[w]) * kBucketSize +
+                                             j * 16);
+    };
+#ifdef HKV_STATS
+    const unsigned long long t_c1 = wall_clock64();
+    t_setup += t_c1 - t_c0;
+#endif
+    /* Software pipeline over the tile's buckets: digest lines are asked for two
+     * buckets ahead, and once a digest line shows no free slot the bucket's
+     * scores are asked for one bucket ahead, so that a bucket's turn starts
+     * with its data in registers. */
+    const auto no_free_slot = [&](const uint4& d) {
+      return tile_ballot(match16_natural(d, v.empty_digest * 0x01010101u) != 0, lane >> 3) == 0;
+    };
+    uint32_t w0 = take();
+    uint32_t w1 = take();
+    uint4 dg0 = make_uint4(0, 0, 0, 0), dg1 = dg0;
+    if (w0 < nwork) dg0 = digests_of(w0);
+    if (w1 < nwork) dg1 = digests_of(w1);
+    uint64_t sc0[2 * kTile], sc1[2 * kTile];
+#pragma unroll
+    for (int q = 0; q < 2 * kTile; q++) sc0[q] = sc1[q] = 0;
+    bool have0 = false;
+    if (w0 < nwork && no_free_slot(dg0)) {
+      scores_load(v, (uint64_t)(bkt0 + s_work[w0]) * kBucketSize, j, sc0);
+      have0 = true;
+    }
+    while (w0 < nwork) {
+      const uint32_t w2 = take();
+      uint4 dg2 = make_uint4(0, 0, 0, 0);
+      if (w2 < nwork) dg2 = digests_of(w2);
+      bool have1 = false;
+      if (w1 < nwork && no_free_slot(dg1)) {
+        scores_load(v, (uint64_t)(bkt0 + s_work[w1]) * kBucketSize, j, sc1);
+        have1 = true;
+      }
+      const uint32_t lb = s_work[w0];
+      group_bucket<OP, VEC, UPL>(v, a, g, bkt0 + lb, s_seg[lb], s_seg[lb + 1], s_key, s_idx, s_info,
+                                 units, lane, dg0, sc0, have0);
+      HKV_COUNT(4, (lane == 0));
+      w0 = w1;
+      dg0 = dg1;
+      have0 = have1;
+#pragma unroll
+      for (int q = 0; q < 2 * kTile; q++) sc0[q] = sc1[q];
+      w1 = w2;
+      dg1 = dg2;
+    }
+#ifdef HKV_STATS
+    const unsigned long long t_c2 = wall_clock64();
+    t_loop += t_c2 - t_c1;
+#endif
+    __syncthreads();
+  }
+#ifdef HKV_STATS
+  if (tid == 0 && first < last) {
+    HKV_COUNT(0, wall_clock64() - t_begin);
+    HKV_COUNT(1, t_setup);
+    HKV_COUNT(2, t_loop);
+    HKV_COUNT(3, 1);
+  }
+#endif
+}
+
+}  // namespace hkv
+#endif

@@ -12,6 +12,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -22,6 +23,7 @@
 #include "hkv_c_api.h"
 #include "hkv_misc.hpp"
 #include "hkv_upsert.hpp"
+#include "hkv_grouped.hpp"
 
 using namespace hkv;
 
@@ -151,6 +153,11 @@ struct hkv_table {
   uint64_t epoch;
   Clock clock;
   mutable StreamGroupLock lock;
+  /* bucket-grouped upserts: partition scratch (histograms, bin starts, key
+   * order), grown on demand; only ever used under the inserter role */
+  void* d_scratch;
+  uint64_t scratch_bytes;
+  int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
 };
 
 namespace {
@@ -272,6 +279,114 @@ void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   }
 }
 
+/* Geometry of a two-phase upsert, or feasible == false when the batch is
+ * better served by the slot-lock kernel. */
+struct GroupPlan {
+  bool feasible;
+  uint32_t bpb_shift, nbins, blocks, slice;
+  uint64_t off_total, off_start, off_order, off_absent, bytes;
+};
+
+GroupPlan plan_grouped(const hkv_table* t, uint64_t n) {
+  GroupPlan p{};
+  const uint64_t buckets = t->view.buckets_num;
+  /* the second phase has no locks: it needs the inserter's exclusivity */
+  if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return p;
+  /* bins of about 256 keys if every key of the batch were absent */
+  uint32_t shift = 0;
+  while (shift < (uint32_t)kGrpMaxBpbShift && (n << (shift + 1)) <= 256 * buckets) shift++;
+  p.bpb_shift = shift;
+  p.nbins = (uint32_t)((buckets + (UINT64_C(1) << shift) - 1) >> shift);
+  if (p.nbins > (uint32_t)kMaxBins) return p;
+  if (t->upsert_path == 0 && (n < 32768 || n < 64 * (uint64_t)p.nbins)) return p;
+  p.blocks = (uint32_t)std::min<uint64_t>(kMaxHistBlocks, (n + 8191) / 8192);
+  p.slice = (uint32_t)((n + p.blocks - 1) / p.blocks);
+  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
+  p.off_total = up((uint64_t)p.blocks * p.nbins * 4);
+  p.off_start = p.off_total + up((uint64_t)p.nbins * 4);
+  p.off_order = p.off_start + up(((uint64_t)p.nbins + 1) * 4);
+  p.off_absent = p.off_order + up(n * 4);
+  p.bytes = p.off_absent + up(n);
+  p.feasible = true;
+  return p;
+}
+
+template <template <int, int, int> class Launcher, int OP, class... Args>
+void dispatch_vec_upl(int vec, uint32_t value_bytes, Args&&... args) {
+  if (vec == 16) {
+    switch (pick_upl(value_bytes, 16)) {
+      case 1: Launcher<OP, 16, 1>::go(args...); break;
+      case 2: Launcher<OP, 16, 2>::go(args...); break;
+      case 4: Launcher<OP, 16, 4>::go(args...); break;
+      default: Launcher<OP, 16, 8>::go(args...); break;
+    }
+  } else if (vec == 4) {
+    Launcher<OP, 4, 8>::go(args...);
+  } else {
+    Launcher<OP, 1, 8>::go(args...);
+  }
+}
+
+template <int OP, int VEC, int UPL>
+struct LaunchHits {
+  static void go(const View& v, const UpsertArgs& a, const HitArgs& h, hipStream_t s) {
+    hipLaunchKernelGGL((upsert_hits_kernel<OP, VEC>), dim3(grid_for(a.n)), dim3(kWave), 0, s, v, a,
+                       h);
+  }
+};
+template <int OP, int VEC, int UPL>
+struct LaunchMisses {
+  static void go(const View& v, const UpsertArgs& a, const GroupArgs& g, uint32_t nbins,
+                 hipStream_t s) {
+    hipLaunchKernelGGL((grouped_miss_kernel<OP, VEC, UPL>), dim3(nbins), dim3(kGrpThreads), 0, s,
+                       v, a, g);
+  }
+};
+
+/* Caller holds the inserter role on `s`. */
+template <int OP>
+int run_grouped(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule,
+                const GroupPlan& p, hipStream_t s) {
+  if (p.bytes > t->scratch_bytes) {
+    /* kernels of earlier calls may still use the old block */
+    HKV_HIP(hipDeviceSynchronize());
+    table_free(t, 0, t->d_scratch);
+    t->d_scratch = nullptr;
+    t->scratch_bytes = 0;
+    const uint64_t want = p.bytes + p.bytes / 4;
+    HKV_TRY(table_alloc(t, 0, &t->d_scratch, want));
+    t->scratch_bytes = want;
+  }
+  uint8_t* base = (uint8_t*)t->d_scratch;
+  HitArgs h{};
+  h.absent = base + p.off_absent;
+  dispatch_vec_upl<LaunchHits, OP>(vec, t->view.value_bytes, t->view, a, h, s);
+
+  BinArgs b{};
+  b.keys = a.keys;
+  b.absent = h.absent;
+  b.n = a.n;
+  b.bpb_shift = p.bpb_shift;
+  b.nbins = p.nbins;
+  b.blocks = p.blocks;
+  b.slice = p.slice;
+  b.hist = (uint32_t*)base;
+  b.total = (uint32_t*)(base + p.off_total);
+  b.bin_start = (uint32_t*)(base + p.off_start);
+  b.order = (uint32_t*)(base + p.off_order);
+  const size_t lds = (size_t)p.nbins * 4;
+  hipLaunchKernelGGL(bin_hist_kernel, dim3(p.blocks), dim3(kBinThreads), lds, s, t->view, b);
+  hipLaunchKernelGGL(bin_colscan_kernel, dim3((p.nbins + 255) / 256), dim3(256), 0, s, b);
+  hipLaunchKernelGGL(bin_scatter_kernel, dim3(p.blocks), dim3(kBinThreads), lds, s, t->view, b);
+  GroupArgs g{};
+  g.order = b.order;
+  g.bin_start = b.bin_start;
+  g.bpb_shift = p.bpb_shift;
+  g.locked_rule = locked_rule;
+  dispatch_vec_upl<LaunchMisses, OP>(vec, t->view.value_bytes, t->view, a, g, p.nbins, s);
+  return HKV_SUCCESS;
+}
+
 template <int OP>
 int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
                hipStream_t s) {
@@ -281,7 +396,12 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
-    if constexpr (OP == kOpFindOrInsertPtr) {
+    GroupPlan plan{};
+    if constexpr (OP != kOpFindOrInsertPtr) plan = plan_grouped(t, a.n);
+    if (plan.feasible) {
+      if constexpr (OP != kOpFindOrInsertPtr)
+        HKV_TRY(run_grouped<OP>(t, a, vec, locked_rule, plan, s));
+    } else if constexpr (OP == kOpFindOrInsertPtr) {
       launch_upsert<OP, true>(vec, t->view, a, s);
     } else if constexpr (OP == kOpInsertOrAssign || OP == kOpFindOrInsert) {
       if (locked_rule)
@@ -394,6 +514,17 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->d_meta = nullptr;
   t->d_counters = nullptr;
   t->h_values = nullptr;
+  t->d_scratch = nullptr;
+  t->scratch_bytes = 0;
+  /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default while the
+   * two-phase path is being tuned), "auto" = two-phase for large batches,
+   * "grouped" = two-phase whenever it is possible (tests) */
+  t->upsert_path = 1;
+  if (const char* e = getenv("HKV_UPSERT_PATH")) {
+    if (!strcmp(e, "auto")) t->upsert_path = 0;
+    if (!strcmp(e, "locked")) t->upsert_path = 1;
+    if (!strcmp(e, "grouped")) t->upsert_path = 2;
+  }
   t->counter_next = 0;
   memset(&t->view, 0, sizeof t->view);
   t->epoch = kIgnoredEpoch;
@@ -547,6 +678,7 @@ int hkv_table_destroy(hkv_table* t) {
   (void)hipDeviceSynchronize();
   table_free(t, 0, t->d_meta);
   table_free(t, 0, t->d_counters);
+  table_free(t, 0, t->d_scratch);
   table_free(t, 0, t->view.values);
   table_free(t, 1, t->h_values);
   delete t;
@@ -954,6 +1086,15 @@ int hkv_debug_stats(uint64_t* out16) {
   HKV_HIP(hipMemcpyFromSymbol(out16, HIP_SYMBOL(g_hkv_stats), 16 * sizeof(uint64_t)));
   uint64_t z[16] = {0};
   HKV_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_hkv_stats), z, sizeof z));
+  return HKV_SUCCESS;
+}
+#endif
+
+#ifdef HKV_EXP
+/* tuning builds only: select the phases the upsert kernel skips */
+int hkv_debug_set_exp(int flags) {
+  HKV_HIP(hipDeviceSynchronize());
+  HKV_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_hkv_exp), &flags, sizeof flags));
   return HKV_SUCCESS;
 }
 #endif

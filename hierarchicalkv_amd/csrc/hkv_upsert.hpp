@@ -203,6 +203,15 @@ __device__ unsigned long long g_hkv_stats[16];
 #define HKV_MARK(slot) ((void)0)
 #endif
 
+/* Knock-out switches for tuning builds (-DHKV_EXP): a device word selects
+ * phases to skip, to apportion a launch's time.  Results are wrong by design. */
+#ifdef HKV_EXP
+__device__ int g_hkv_exp;
+#define HKV_EXP_FLAG(bit) ((g_hkv_exp & (bit)) != 0)
+#else
+#define HKV_EXP_FLAG(bit) false
+#endif
+
 #ifndef HKV_SCAN_PAIR
 #define HKV_SCAN_PAIR 1
 #endif
@@ -491,6 +500,7 @@ upsert_kernel(View v, UpsertArgs a) {
     em_hi = e.z | ((uint64_t)e.w << 32);
   }
   bool pending = (me.info & 0x100u) != 0;
+  if (HKV_EXP_FLAG(4)) pending = false;
   bool reprobe = pending && hit < 0 && s_unsure[lane];
 
   /* The trip loop is controlled by a wavefront-uniform value only: all 64
@@ -550,7 +560,10 @@ upsert_kernel(View v, UpsertArgs a) {
           }
         }
       } else {
-        want_scan = true;
+        if (HKV_EXP_FLAG(2))
+          got = kStRefused;
+        else
+          want_scan = true;
         HKV_COUNT(6, 1); /* scans */
       }
     }
@@ -594,7 +607,7 @@ upsert_kernel(View v, UpsertArgs a) {
     /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
     bool refused_now = false;
     if (want_scan) {
-      const bool refuse = LOCKED_RULE ? (desired <= best) : (desired < best);
+      const bool refuse = (LOCKED_RULE ? (desired <= best) : (desired < best)) || HKV_EXP_FLAG(16);
       if (refuse) {
         refused_now = true;
         got = kStRefused;
@@ -656,7 +669,7 @@ upsert_kernel(View v, UpsertArgs a) {
       a.out_ptrs[i] = locked ? row : nullptr;
       a.founds[i] = got == kStDuplicate;
     }
-    if (commit) {
+    if (commit && !HKV_EXP_FLAG(8)) {
       write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
       if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
     }
@@ -675,6 +688,7 @@ upsert_kernel(View v, UpsertArgs a) {
           usr = const_cast<uint8_t*>(a.values_in) + i * v.value_bytes;
         }
       }
+      if (HKV_EXP_FLAG(1)) move = kMoveNone;
       if (__ballot(move != kMoveNone))
         bulk_rows<VEC, UPL, OP == kOpFindOrInsert, OP == kOpAccumOrAssign>(
             move, row, usr, units, a.value_kind, lane);
