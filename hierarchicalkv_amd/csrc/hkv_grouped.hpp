@@ -35,21 +35,37 @@
  *   bin_colscan_kernel   per bin: running sum over the blocks
  *   bin_scatter_kernel   per block: scan of the bin totals, then every key's
  *                        index goes to its place in `order`
- * grouped_miss_kernel then runs one 256-thread workgroup per bin: counting
- * sort of the bin's keys by bucket in LDS, and its 32 tiles take buckets from
- * a work list.
+ * grouped_miss_kernel then runs one wavefront per bin: counting sort of the
+ * bin's keys by bucket in LDS, and its 8 tiles take buckets from a work list.
  */
 #ifndef HKV_GROUPED_HPP_
 #define HKV_GROUPED_HPP_
 
 #include "hkv_upsert.hpp"
 
+/* phase timing of tuning builds: the first lane of a workgroup adds the ticks
+ * since the previous mark to a slot in LDS; one atomic per slot and workgroup
+ * at the end */
+#ifdef HKV_STATS
+#define HKV_LMARK_INIT() unsigned long long hkv_lt_ = wall_clock64()
+#define HKV_LMARK(acc, slot)                                  \
+  do {                                                        \
+    const unsigned long long now_ = wall_clock64();           \
+    if (threadIdx.x == 0) (acc)[slot] += now_ - hkv_lt_;      \
+    hkv_lt_ = now_;                                           \
+  } while (0)
+#else
+#define HKV_LMARK_INIT() ((void)0)
+#define HKV_LMARK(acc, slot) ((void)0)
+#endif
+
 namespace hkv {
 
 constexpr int kBinThreads = 1024;   /* histogram / scatter workgroup */
 constexpr int kMaxBins = 8192;      /* LDS histogram: 32 KB */
-constexpr int kGrpThreads = 256;    /* grouped_upsert_kernel workgroup */
-constexpr int kGrpChunk = 512;      /* keys of a bin staged per pass */
+constexpr int kGrpThreads = 64;     /* grouped_miss_kernel workgroup: one wavefront, no barriers to wait at */
+constexpr int kGrpChunk = 256;      /* keys of a bin staged per pass */
+constexpr int kGrpStage = kGrpChunk / kGrpThreads; /* keys a thread stages */
 constexpr int kGrpMaxBpbShift = 10; /* at most 1024 buckets per bin */
 constexpr int kGrpMaxBpb = 1 << kGrpMaxBpbShift;
 constexpr int kGrpKeys = 2;         /* keys of one bucket handled per pass of a tile */
@@ -206,36 +222,6 @@ __device__ __forceinline__ void dg_set(uint4& d, uint32_t p, uint32_t byte) {
   d.w = (d.w & ~c3) | (put & c3);
 }
 
-/* The 128 scores of a bucket over the 8 lanes of a tile: lane j holds the
- * positions {16 it + 2 j, 16 it + 2 j + 1}, the layout of scan_reduce. */
-__device__ __forceinline__ void scores_load(const View& v, uint64_t bslot, int j, uint64_t* sc) {
-#pragma unroll
-  for (int it = 0; it < kTile; it++) {
-    const uint4 t = *reinterpret_cast<const uint4*>(v.scores + bslot + it * 16 + j * 2);
-    sc[2 * it] = t.x | ((uint64_t)t.y << 32);
-    sc[2 * it + 1] = t.z | ((uint64_t)t.w << 32);
-  }
-}
-__device__ __forceinline__ void scores_patch(uint64_t* sc, int j, uint32_t pos, uint64_t s) {
-  const bool mine = (int)((pos & 15u) >> 1) == j;
-  const uint32_t e = 2 * (pos >> 4) + (pos & 1u);
-#pragma unroll
-  for (uint32_t q = 0; q < 2 * kTile; q++)
-    if (mine && q == e) sc[q] = s;
-}
-/* write back the 64-byte pieces named in `dirty` (bit c: positions 8c..8c+7) */
-__device__ __forceinline__ void scores_flush(const View& v, uint64_t bslot, int j,
-                                             const uint64_t* sc, uint32_t dirty) {
-#pragma unroll
-  for (int it = 0; it < kTile; it++) {
-    if ((dirty >> (2 * it + (j >> 2))) & 1u) {
-      const uint4 t = make_uint4((uint32_t)sc[2 * it], (uint32_t)(sc[2 * it] >> 32),
-                                 (uint32_t)sc[2 * it + 1], (uint32_t)(sc[2 * it + 1] >> 32));
-      st_u128(v.scores + bslot + it * 16 + j * 2, t);
-    }
-  }
-}
-
 /* ScoreFunctor<Strategy>::update_with_digest (kernel_utils.cuh:291-302,
  * 353-371, 422-434, 490-517, 581-593) as a value: the score an accepted key
  * leaves in its slot; false when the score stays as it is. */
@@ -388,42 +374,87 @@ __device__ __forceinline__ uint32_t tile_first_u32(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x0018); /* and 0x18, or 0, xor 0 */
 }
 
-/* minimum score of the bucket and its slot; ties go to the lowest slot, as the
- * reference's sequential scan with a strict '<' (upsert.cuh:166-183) */
-__device__ __forceinline__ void tile_min(const uint64_t* sc, int j, uint64_t& best, uint32_t& bpos) {
-  best = sc[0];
-  uint32_t e = 0;
+/* (score, slot) pairs order by score, then by slot: the reference's sequential
+ * scan with a strict '<' keeps the lowest slot among equal scores
+ * (upsert.cuh:166-183) */
+__device__ __forceinline__ bool pair_lt(uint64_t s, uint32_t p, uint64_t t, uint32_t q) {
+  return s < t || (s == t && p < q);
+}
+
+/* The two smallest (score, slot) pairs of a bucket. */
+struct Top2 {
+  uint64_t s1, s2;
+  uint32_t p1, p2;
+};
+
+constexpr uint32_t kNoSlot = 255;
+
+/*
+ * Scan of a bucket's 128 scores by the 8 lanes of a tile: lane j reads the
+ * slots {16 it + 2 j, 16 it + 2 j + 1}, one coalesced 128-byte line per `it`
+ * and tile, keeps its two smallest pairs, and three exchange steps merge the
+ * lanes' pairs.  Slot `skip` does not take part (a slot a key of this pass has
+ * just moved into: its score is still on its way).  Two pairs are enough for
+ * a pass of two keys; the scores themselves are not kept, which is what keeps
+ * the kernel's register count low.
+ */
+__device__ __forceinline__ Top2 tile_top2(const View& v, uint64_t bslot, int j, uint32_t skip) {
+  uint4 raw[kTile];
 #pragma unroll
-  for (uint32_t q = 1; q < 2 * kTile; q++) {
-    /* register q holds slot 16 (q >> 1) + 2 j + (q & 1): slots grow with q */
-    if (sc[q] < best) {
-      best = sc[q];
-      e = q;
+  for (int it = 0; it < kTile; it++)
+    raw[it] = *reinterpret_cast<const uint4*>(v.scores + bslot + it * 16 + j * 2);
+  Top2 t;
+  t.s1 = t.s2 = kMaxScore;
+  t.p1 = t.p2 = kNoSlot;
+#pragma unroll
+  for (int q = 0; q < 2 * kTile; q++) {
+    const uint4& r = raw[q >> 1];
+    const uint64_t x = (q & 1) ? (r.z | ((uint64_t)r.w << 32)) : (r.x | ((uint64_t)r.y << 32));
+    const uint32_t px = (q >> 1) * 16 + 2 * (uint32_t)j + (q & 1);
+    if (px == skip) continue;
+    if (pair_lt(x, px, t.s1, t.p1)) {
+      t.s2 = t.s1;
+      t.p2 = t.p1;
+      t.s1 = x;
+      t.p1 = px;
+    } else if (pair_lt(x, px, t.s2, t.p2)) {
+      t.s2 = x;
+      t.p2 = px;
     }
   }
-  bpos = (e >> 1) * 16 + 2 * (uint32_t)j + (e & 1u);
-#define HKV_TILE_MIN_STEP(FN)                                                  \
-  {                                                                            \
-    const uint64_t ob = (uint64_t)FN((uint32_t)best) | ((uint64_t)FN((uint32_t)(best >> 32)) << 32); \
-    const uint32_t op = FN(bpos);                                              \
-    if (ob < best || (ob == best && op < bpos)) {                              \
-      best = ob;                                                               \
-      bpos = op;                                                               \
-    }                                                                          \
+#define HKV_TOP2_STEP(FN)                                                                      \
+  {                                                                                            \
+    const uint64_t a1 = (uint64_t)FN((uint32_t)t.s1) | ((uint64_t)FN((uint32_t)(t.s1 >> 32)) << 32); \
+    const uint64_t a2 = (uint64_t)FN((uint32_t)t.s2) | ((uint64_t)FN((uint32_t)(t.s2 >> 32)) << 32); \
+    const uint32_t q1 = FN(t.p1), q2 = FN(t.p2);                                               \
+    Top2 m;                                                                                    \
+    if (pair_lt(a1, q1, t.s1, t.p1)) {                                                         \
+      m.s1 = a1;                                                                               \
+      m.p1 = q1;                                                                               \
+      const bool second = pair_lt(a2, q2, t.s1, t.p1);                                         \
+      m.s2 = second ? a2 : t.s1;                                                               \
+      m.p2 = second ? q2 : t.p1;                                                               \
+    } else {                                                                                   \
+      m.s1 = t.s1;                                                                             \
+      m.p1 = t.p1;                                                                             \
+      const bool second = pair_lt(a1, q1, t.s2, t.p2);                                         \
+      m.s2 = second ? a1 : t.s2;                                                               \
+      m.p2 = second ? q1 : t.p2;                                                               \
+    }                                                                                          \
+    t = m;                                                                                     \
   }
-  HKV_TILE_MIN_STEP(xor1_u32)
-  HKV_TILE_MIN_STEP(xor2_u32)
-  HKV_TILE_MIN_STEP(xor4_u32)
-#undef HKV_TILE_MIN_STEP
+  HKV_TOP2_STEP(xor1_u32)
+  HKV_TOP2_STEP(xor2_u32)
+  HKV_TOP2_STEP(xor4_u32)
+#undef HKV_TOP2_STEP
+  return t;
 }
 
 /*
  * Phase 2, one bucket: the absent keys of the batch that fall into bucket
  * `bkt` are the entries [sb, se) of the sorted LDS arrays.  Called by the 8
  * lanes of a tile together; `lane` is the lane inside the wavefront.  `dg` is
- * the lane's 16 bytes of the bucket's digest line; `sc` holds the bucket's scores
- * already when sc_loaded says so (the caller asks for them ahead of time when
- * the digest line shows no free slot).
+ * the lane's 16 bytes of the bucket's digest line.
  *
  * Everything that steers the work (which key goes where, what it displaces) is
  * computed by all 8 lanes alike from the same LDS entries, so the lanes agree
@@ -434,13 +465,15 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
                                              const GroupArgs& g, uint32_t bkt, uint32_t sb,
                                              uint32_t se, const uint64_t* s_key,
                                              const uint32_t* s_idx, const uint32_t* s_info,
-                                             uint32_t units, int lane, uint4 dg, uint64_t* sc,
-                                             bool sc_loaded) {
+                                             uint32_t units, int lane, uint4 dg,
+                                             unsigned long long* acc) {
+  static_assert(kGrpKeys == 2, "tile_top2 serves a pass of two keys");
   const int j = lane & (kTile - 1);
   const int tile = lane >> 3;
   const int tile_base = lane & ~(kTile - 1);
   const uint64_t bslot = (uint64_t)bkt * kBucketSize;
   const uint8_t* rows_in = OP == kOpFindOrInsert ? a.values_io : a.values_in;
+  HKV_LMARK_INIT();
 
   bool dg_dirty = false;
   int size_delta = 0;
@@ -483,6 +516,7 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       }
     }
 
+    HKV_LMARK(acc, 5); /* free-slot mask, row loads issued */
     /* outcome of key q of the pass, the same in every lane of the tile */
     int got[kGrpKeys];
     uint32_t pos[kGrpKeys];
@@ -490,7 +524,8 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
     uint64_t best_seen[kGrpKeys];
     bool wrs[kGrpKeys], cancelled[kGrpKeys], need_vk[kGrpKeys];
     int vic_from[kGrpKeys];
-    uint32_t dirty = 0; /* 64-byte score pieces changed in this pass */
+    bool scanned = false;
+    Top2 top{};
 
     /* ---- the keys of the pass, one after the other -------------------------------------------------- */
 #pragma unroll
@@ -510,7 +545,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       const uint64_t in_score = a.scores ? a.scores[iq] : 0;
       const uint64_t dq = desired_when_missed(a, in_score, iq);
       wrs[q] = final_score(a, true, dq, in_score, 0, snew[q]);
-      const uint64_t sq = snew[q];
       /* the same key earlier in this pass (batches are meant to hold unique
        * keys): the first one wins, this one changes nothing */
       bool dup = false;
@@ -533,30 +567,48 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
         if (j == (int)(p >> 4)) dg_set(dg, p & 15u, info & 0xFFu);
         dg_dirty = true;
         size_delta++;
-        if (sc_loaded && wrs[q]) {
-          scores_patch(sc, j, p, sq);
-          dirty |= 1u << (p >> 3);
-        }
         continue;
       }
-      if (!sc_loaded) {
-        /* scores stored one by one earlier in this call must have landed */
-        wait_stores();
-        scores_load(v, bslot, j, sc);
-        sc_loaded = true;
-        /* keys of this pass that went into free slots have not stored their
-         * scores yet: the registers are the truth from here on */
+      if (!scanned) {
+        /* a key of this pass that has just taken the last free slot is not
+         * part of the scan: it competes with its new score below */
+        uint32_t skip = kNoSlot;
+#pragma unroll
+        for (int r = 0; r < q; r++)
+          if (got[r] == kStEmpty) skip = pos[r];
+        top = tile_top2(v, bslot, j, skip);
+        scanned = true;
+      }
+      /* minimum over what the scan saw, less the slots this pass has already
+       * taken over, plus the keys this pass has placed */
+      uint64_t best = kMaxScore;
+      uint32_t bpos = kNoSlot;
+      {
+        bool used1 = false, used2 = false;
 #pragma unroll
         for (int r = 0; r < q; r++) {
-          if (got[r] == kStEmpty && wrs[r]) {
-            scores_patch(sc, j, pos[r], snew[r]);
-            dirty |= 1u << (pos[r] >> 3);
+          if (got[r] == kStEvict) {
+            used1 |= pos[r] == top.p1;
+            used2 |= pos[r] == top.p2;
+          }
+        }
+        if (!used1 && pair_lt(top.s1, top.p1, best, bpos)) {
+          best = top.s1;
+          bpos = top.p1;
+        }
+        if (!used2 && pair_lt(top.s2, top.p2, best, bpos)) {
+          best = top.s2;
+          bpos = top.p2;
+        }
+#pragma unroll
+        for (int r = 0; r < q; r++) {
+          if ((got[r] == kStEmpty || got[r] == kStEvict) && !cancelled[r] && wrs[r] &&
+              pair_lt(snew[r], pos[r], best, bpos)) {
+            best = snew[r];
+            bpos = pos[r];
           }
         }
       }
-      uint64_t best;
-      uint32_t bpos;
-      tile_min(sc, j, best, bpos);
       const bool refuse = g.locked_rule ? (dq <= best) : (dq < best);
       if (refuse) {
         got[q] = kStRefused;
@@ -580,14 +632,11 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       need_vk[q] = vic_from[q] < 0 && (OP == kOpInsertAndEvict || tomb_digest);
       pos[q] = bpos;
       best_seen[q] = best;
-      /* a strategy that leaves the score alone still has to hide the slot from
-       * the next scan of this pass; the piece is written back only if it changed */
-      scores_patch(sc, j, bpos, wrs[q] ? sq : kMaxScore);
-      if (wrs[q]) dirty |= 1u << (bpos >> 3);
       if (j == (int)(bpos >> 4)) dg_set(dg, bpos & 15u, info & 0xFFu);
       dg_dirty = true;
     }
 
+    HKV_LMARK(acc, 6); /* placement */
     /* ---- victims: live key or tombstone ------------------------------------------------------------- */
     uint64_t victim[kGrpKeys];
 #pragma unroll
@@ -674,16 +723,16 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
           (got[q] == kStEmpty || got[q] == kStReclaimed || got[q] == kStEvict) && !cancelled[q];
       if (!writes) continue;
       const uint64_t slot = bslot + pos[q];
-      if (j == 0) {
+      if (j == 0 && !HKV_EXP_FLAG(128)) {
         v.keys[slot] = s_key[q0 + q];
-        if (wrs[q] && !sc_loaded) v.scores[slot] = snew[q];
+        if (wrs[q]) v.scores[slot] = snew[q];
       }
       uint8_t* tb = value_row(v, slot);
       if constexpr (kPre) {
 #pragma unroll
         for (int w = 0; w < UPL; w++) {
           const uint32_t u = j + w * kTile;
-          if (u < units) st_unit<VEC, true>(tb, u, xin[q][w]);
+          if (u < units && !HKV_EXP_FLAG(64)) st_unit<VEC, true>(tb, u, xin[q][w]);
         }
       } else {
         const uint8_t* us = rows_in + (uint64_t)s_idx[q0 + q] * v.value_bytes;
@@ -703,32 +752,43 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
         }
       }
     }
-    if (sc_loaded && dirty) scores_flush(v, bslot, j, sc, dirty);
+    HKV_LMARK(acc, 7); /* victims, keys, rows */
   }
 
-  if (dg_dirty) st_u128(v.digests + bslot + j * 16, dg);
+  if (dg_dirty && !HKV_EXP_FLAG(32)) st_u128(v.digests + bslot + j * 16, dg);
   if (size_delta && j == 0) atomicAdd(v.sizes + bkt, size_delta);
+  HKV_LMARK(acc, 8); /* score and digest write-back */
 }
 
-#ifndef HKV_GROUPED_MIN_WAVES
-#define HKV_GROUPED_MIN_WAVES 1
+#ifndef HKV_GROUPED_WAVES_PER_EU
+#define HKV_GROUPED_WAVES_PER_EU 3
 #endif
 template <int OP, int VEC, int UPL>
-__global__ void __launch_bounds__(kGrpThreads, HKV_GROUPED_MIN_WAVES)
+__global__ void __launch_bounds__(kGrpThreads)
+__attribute__((amdgpu_waves_per_eu(HKV_GROUPED_WAVES_PER_EU)))
 grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
   __shared__ uint64_t s_key[kGrpChunk];
   __shared__ uint32_t s_idx[kGrpChunk];
   __shared__ uint32_t s_info[kGrpChunk]; /* digest | start << 8 | bucket inside the bin << 16 */
-  __shared__ uint32_t s_seg[kGrpMaxBpb + 1];
-  __shared__ uint32_t s_cur[kGrpMaxBpb];
-  __shared__ uint16_t s_work[kGrpMaxBpb];
+  /* sized by the launch: (bpb + 1) segment starts, bpb cursors, bpb work items */
+  extern __shared__ uint32_t s_dyn[];
   __shared__ uint32_t s_wsum[kGrpThreads / kWave];
   __shared__ uint32_t s_nwork, s_next;
+#ifdef HKV_STATS
+  __shared__ unsigned long long s_acc[16];
+  if (threadIdx.x < 16) s_acc[threadIdx.x] = 0;
+  __syncthreads();
+#else
+  unsigned long long* const s_acc = nullptr;
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const uint32_t bin = blockIdx.x;
   const uint32_t bpb = 1u << g.bpb_shift;
+  uint32_t* const s_seg = s_dyn;
+  uint32_t* const s_cur = s_dyn + bpb + 1;
+  uint16_t* const s_work = reinterpret_cast<uint16_t*>(s_dyn + 2 * bpb + 1);
   const uint32_t first = g.bin_start[bin], last = g.bin_start[bin + 1];
   const uint32_t units = v.value_bytes / VEC;
 
@@ -748,12 +808,12 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
     }
     __syncthreads();
 
-    /* ---- stage: two keys per thread, counted by bucket ----------------------------------------- */
-    uint64_t mk[2];
-    uint32_t mi[2], minfo[2];
-    bool have[2];
+    /* ---- stage: kGrpStage keys per thread, counted by bucket ------------------------------------- */
+    uint64_t mk[kGrpStage];
+    uint32_t mi[kGrpStage], minfo[kGrpStage];
+    bool have[kGrpStage];
 #pragma unroll
-    for (int e = 0; e < 2; e++) {
+    for (int e = 0; e < kGrpStage; e++) {
       const uint32_t p = tid + e * kGrpThreads;
       have[e] = p < cn;
       mk[e] = 0;
@@ -765,7 +825,7 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
       }
     }
 #pragma unroll
-    for (int e = 0; e < 2; e++) {
+    for (int e = 0; e < kGrpStage; e++) {
       if (have[e]) {
         uint32_t bkt, start, digest;
         locate(v, mk[e], bkt, start, digest);
@@ -778,13 +838,11 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
 
     /* ---- exclusive scan of the counts; list of the buckets that have keys ---------------------------- */
     {
-      uint32_t c[4], sum = 0;
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const uint32_t t = tid * 4 + e;
-        c[e] = t < bpb ? s_seg[t] : 0;
-        sum += c[e];
-      }
+      const uint32_t per = (bpb + kGrpThreads - 1) / kGrpThreads;
+      const uint32_t t0 = tid * per;
+      uint32_t sum = 0;
+      for (uint32_t e = 0; e < per; e++)
+        if (t0 + e < bpb) sum += s_seg[t0 + e];
       uint32_t inc = sum;
 #pragma unroll
       for (int off = 1; off < kWave; off <<= 1) {
@@ -795,14 +853,14 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
       __syncthreads();
       uint32_t run = inc - sum;
       for (int w = 0; w < (tid >> 6); w++) run += s_wsum[w];
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const uint32_t t = tid * 4 + e;
+      for (uint32_t e = 0; e < per; e++) {
+        const uint32_t t = t0 + e;
         if (t < bpb) {
+          const uint32_t c = s_seg[t];
           s_seg[t] = run;
           s_cur[t] = run;
-          if (c[e]) s_work[atomicAdd(&s_nwork, 1u)] = (uint16_t)t;
-          run += c[e];
+          if (c) s_work[atomicAdd(&s_nwork, 1u)] = (uint16_t)t;
+          run += c;
         }
       }
       if (tid == kGrpThreads - 1) s_seg[bpb] = run;
@@ -811,7 +869,7 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
 
     /* ---- place ------------------------------------------------------------------------------------------ */
 #pragma unroll
-    for (int e = 0; e < 2; e++) {
+    for (int e = 0; e < kGrpStage; e++) {
       if (have[e]) {
         const uint32_t p = atomicAdd(&s_cur[minfo[e] >> 16], 1u);
         s_key[p] = mk[e];
@@ -840,46 +898,26 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
     const unsigned long long t_c1 = wall_clock64();
     t_setup += t_c1 - t_c0;
 #endif
-    /* Software pipeline over the tile's buckets: digest lines are asked for two
-     * buckets ahead, and once a digest line shows no free slot the bucket's
-     * scores are asked for one bucket ahead, so that a bucket's turn starts
-     * with its data in registers. */
-    const auto no_free_slot = [&](const uint4& d) {
-      return tile_ballot(match16_natural(d, v.empty_digest * 0x01010101u) != 0, lane >> 3) == 0;
-    };
+    /* the digest line of the next bucket is asked for before the current one is
+     * worked on */
     uint32_t w0 = take();
-    uint32_t w1 = take();
-    uint4 dg0 = make_uint4(0, 0, 0, 0), dg1 = dg0;
+    uint4 dg0 = make_uint4(0, 0, 0, 0);
     if (w0 < nwork) dg0 = digests_of(w0);
-    if (w1 < nwork) dg1 = digests_of(w1);
-    uint64_t sc0[2 * kTile], sc1[2 * kTile];
-#pragma unroll
-    for (int q = 0; q < 2 * kTile; q++) sc0[q] = sc1[q] = 0;
-    bool have0 = false;
-    if (w0 < nwork && no_free_slot(dg0)) {
-      scores_load(v, (uint64_t)(bkt0 + s_work[w0]) * kBucketSize, j, sc0);
-      have0 = true;
-    }
+    HKV_LMARK_INIT();
     while (w0 < nwork) {
-      const uint32_t w2 = take();
-      uint4 dg2 = make_uint4(0, 0, 0, 0);
-      if (w2 < nwork) dg2 = digests_of(w2);
-      bool have1 = false;
-      if (w1 < nwork && no_free_slot(dg1)) {
-        scores_load(v, (uint64_t)(bkt0 + s_work[w1]) * kBucketSize, j, sc1);
-        have1 = true;
-      }
+      const uint32_t w1 = take();
+      uint4 dg1 = make_uint4(0, 0, 0, 0);
+      if (w1 < nwork) dg1 = digests_of(w1);
       const uint32_t lb = s_work[w0];
+      HKV_LMARK(s_acc, 9); /* take + prefetch issue */
       group_bucket<OP, VEC, UPL>(v, a, g, bkt0 + lb, s_seg[lb], s_seg[lb + 1], s_key, s_idx, s_info,
-                                 units, lane, dg0, sc0, have0);
-      HKV_COUNT(4, (lane == 0));
+                                 units, lane, dg0, s_acc);
+      HKV_LMARK(s_acc, 10); /* bucket */
+#ifdef HKV_STATS
+      if (tid == 0) s_acc[4] += 1; /* buckets per workgroup */
+#endif
       w0 = w1;
       dg0 = dg1;
-      have0 = have1;
-#pragma unroll
-      for (int q = 0; q < 2 * kTile; q++) sc0[q] = sc1[q];
-      w1 = w2;
-      dg1 = dg2;
     }
 #ifdef HKV_STATS
     const unsigned long long t_c2 = wall_clock64();
@@ -893,6 +931,7 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
     HKV_COUNT(1, t_setup);
     HKV_COUNT(2, t_loop);
     HKV_COUNT(3, 1);
+    for (int k = 4; k < 12; k++) HKV_COUNT(k, s_acc[k]);
   }
 #endif
 }

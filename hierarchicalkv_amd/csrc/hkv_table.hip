@@ -292,13 +292,13 @@ GroupPlan plan_grouped(const hkv_table* t, uint64_t n) {
   const uint64_t buckets = t->view.buckets_num;
   /* the second phase has no locks: it needs the inserter's exclusivity */
   if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return p;
-  /* bins of about 256 keys if every key of the batch were absent */
+  /* bins of about 128 keys if every key of the batch were absent */
   uint32_t shift = 0;
-  while (shift < (uint32_t)kGrpMaxBpbShift && (n << (shift + 1)) <= 256 * buckets) shift++;
+  while (shift < (uint32_t)kGrpMaxBpbShift && (n << (shift + 1)) <= 128 * buckets) shift++;
   p.bpb_shift = shift;
   p.nbins = (uint32_t)((buckets + (UINT64_C(1) << shift) - 1) >> shift);
   if (p.nbins > (uint32_t)kMaxBins) return p;
-  if (t->upsert_path == 0 && (n < 32768 || n < 64 * (uint64_t)p.nbins)) return p;
+  if (t->upsert_path == 0 && (n < 32768 || n < 32 * (uint64_t)p.nbins)) return p;
   p.blocks = (uint32_t)std::min<uint64_t>(kMaxHistBlocks, (n + 8191) / 8192);
   p.slice = (uint32_t)((n + p.blocks - 1) / p.blocks);
   auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
@@ -338,7 +338,9 @@ template <int OP, int VEC, int UPL>
 struct LaunchMisses {
   static void go(const View& v, const UpsertArgs& a, const GroupArgs& g, uint32_t nbins,
                  hipStream_t s) {
-    hipLaunchKernelGGL((grouped_miss_kernel<OP, VEC, UPL>), dim3(nbins), dim3(kGrpThreads), 0, s,
+    const size_t bpb = (size_t)1 << g.bpb_shift;
+    const size_t lds = (2 * bpb + 1) * 4 + bpb * 2;
+    hipLaunchKernelGGL((grouped_miss_kernel<OP, VEC, UPL>), dim3(nbins), dim3(kGrpThreads), lds, s,
                        v, a, g);
   }
 };
