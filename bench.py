@@ -40,6 +40,14 @@ def upsert_bytes(vb, new_fraction):
     return (1.0 - new_fraction) * (161 + 2 * vb) + new_fraction * (1185 + 2 * vb)
 
 
+# HBM bytes per launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (KiB per dispatch, each scaled by what the same counter reads for a
+# 1 GiB device-to-device copy: 2.000 and 1.000).  Counters cannot be read from inside
+# this process, so the figures of the committed profile summary are reported; they
+# apply to the default workload and the default (slot-lock) upsert path only.
+MEASURED_TRAFFIC = {"upsert_kernel": 1639.5e6, "lookup_kernel": 868.7e6}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -175,6 +183,11 @@ def main():
     find_gbs = fb / (find_avg * 1e-3) / 1e9
     ups_gbs = ub / (ups_avg * 1e-3) / 1e9
 
+    default_workload = (args.capacity_log2 == 26 and dim == 64 and args.batch_log2 == 20
+                        and not args.warm_keys)
+    path = os.environ.get("HKV_UPSERT_PATH", "locked")
+    ups_traffic = MEASURED_TRAFFIC["upsert_kernel"] if default_workload and path == "locked" else None
+    find_traffic = MEASURED_TRAFFIC["lookup_kernel"] if default_workload else None
     result = {
         "metric": "billion-KV/s for find & insert_or_assign, dim 64, load factor 1.0, 1 GPU",
         "value": round(value, 4),
@@ -197,18 +210,20 @@ def main():
             "size_after": size1,
             "prefill_s": round(prefill_s, 1),
             "resident_keys": "warm (previous step)" if args.warm_keys else "cold (old pre-fill batches)",
+            "upsert_path": path,
         },
         "find": {"ms": round(find_avg, 4), "bkvs": round(n / (find_avg * 1e-3) / 1e9, 4),
                  "bkvs_2p30": round(n / (find_avg * 1e-3) / 2**30, 4)},
         "insert_or_assign": {"ms": round(ups_avg, 4), "bkvs": round(n / (ups_avg * 1e-3) / 1e9, 4),
                              "bkvs_2p30": round(n / (ups_avg * 1e-3) / 2**30, 4)},
-        "roofline": {"kernel": "upsert_kernel<insert_or_assign>", "bound": "hbm",
+        "roofline": {"kernel": "upsert_kernel<insert_or_assign>" if path == "locked" else
+                     "two-phase upsert: upsert_hits_kernel + bin_* + grouped_miss_kernel", "bound": "hbm",
                      "achieved": round(ups_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": ups_traffic,
                      "bytes_per_key": upsert_bytes(vb, 0.5)},
         "roofline_find": {"kernel": "lookup_kernel<values>", "bound": "hbm",
                           "achieved": round(find_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": round(find_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                          "frac": round(find_gbs / HBM_PEAK_GBS, 4), "traffic": find_traffic,
                           "bytes_per_key": find_bytes(vb)},
     }
     table.close()
@@ -239,7 +254,7 @@ def cpu_baseline(args, np, w):
         t.insert_or_assign_mt(w.unique_keys(seed, pos, n), vals, threads=threads)
         pos += n
     prev = w.unique_keys(seed, pos - n, n)
-    reps = 3
+    reps = 100  # about 10 s of host work
     tf = ti = 0.0
     out = np.zeros((n, dim * 4), np.uint8)
     for r in range(reps):
