@@ -70,6 +70,68 @@ size_kernel(View v, unsigned long long* out) {
   }
 }
 
+/*
+ * Rehash into a table with twice the buckets (rehash_kernel_for_fast_mode,
+ * core_kernels.cuh:540-591).  With g = hash modulo capacity and the bucket
+ * count doubling from B to 2B, a key of bucket b lands in bucket b or b + B
+ * of the new table, and both start out empty: every entry can keep its slot
+ * position, so no destination search and no compaction is needed (positions
+ * are not observable through the API).  Tombstones stay in bucket b.  One
+ * wavefront per 64 slots; it counts its live keys per destination bucket with
+ * two ballots and moves their rows together.
+ */
+__global__ void __launch_bounds__(256)
+rehash_kernel(View src, View dst) {
+  const int lane = lane_id();
+  const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  const uint64_t s = wave * kWave + lane;
+  if (wave * kWave >= src.capacity) return;
+  const uint64_t b = s >> 7;
+  const uint32_t p = (uint32_t)(s & 127u);
+  const uint64_t key = src.keys[s];
+  const bool tomb = key == src.reclaim_key;
+  const bool live = key != src.empty_key && !tomb;
+  uint64_t nb = b;
+  if (live) {
+    uint32_t bkt, start, digest;
+    locate(dst, key, bkt, start, digest);
+    nb = bkt;
+  }
+  const uint64_t d = nb * kBucketSize + p;
+  if (live || tomb) {
+    dst.keys[d] = key;
+    dst.digests[d] = src.digests[s];
+    dst.scores[d] = src.scores[s];
+  }
+  const unsigned long long stay = __ballot(live && nb == b);
+  const unsigned long long move = __ballot(live && nb != b);
+  if (lane == 0) {
+    /* the 64 slots of a wavefront belong to one bucket */
+    if (stay) atomicAdd(dst.sizes + b, (int)__popcll(stay));
+    if (move) atomicAdd(dst.sizes + b + src.buckets_num, (int)__popcll(move));
+  }
+  unsigned long long rest = stay | move;
+  while (rest) {
+    const int l = __ffsll(rest) - 1;
+    rest &= rest - 1;
+    const uint64_t dl = __shfl((unsigned long long)d, l);
+    wave_copy_row(value_row(dst, dl), value_row(src, wave * kWave + l), src.value_bytes, lane);
+  }
+}
+
+/* sum of the sizes of the first n buckets (fast_load_factor,
+ * merlin_hashtable.cuh:3796-3830); one workgroup */
+__global__ void __launch_bounds__(256)
+partial_size_kernel(View v, uint32_t n, unsigned long long* out) {
+  __shared__ unsigned long long s_part[4];
+  unsigned long long local = 0;
+  for (uint32_t b = threadIdx.x; b < n; b += 256) local += (unsigned long long)v.sizes[b];
+  for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
+  __syncthreads();
+  if (threadIdx.x == 0) *out = s_part[0] + s_part[1] + s_part[2] + s_part[3];
+}
+
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
 __global__ void zero_i32_kernel(int32_t* p) { *p = 0; }
 

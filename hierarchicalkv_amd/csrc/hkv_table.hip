@@ -146,6 +146,7 @@ struct hkv_table {
   hkv_allocator alloc;
   void* d_meta;          /* digests + keys + scores + sizes in one arena */
   uint64_t meta_bytes;
+  void* d_values;        /* value rows in HBM */
   void* h_values;        /* host address of the pinned value rows (hybrid) */
   unsigned long long* d_counters; /* ring of scratch words for size / size_if /
                                      the count-returning insert_and_evict */
@@ -158,6 +159,7 @@ struct hkv_table {
   void* d_scratch;
   uint64_t scratch_bytes;
   int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
+  bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
 };
 
 namespace {
@@ -389,9 +391,164 @@ int run_grouped(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule,
   return HKV_SUCCESS;
 }
 
+constexpr unsigned kCounterRing = 32;
+
+/* Calls that return a count synchronise before they return, so at most one
+ * word per concurrently calling host thread is in use. */
+unsigned long long* take_counter(const hkv_table* t) {
+  return t->d_counters + (t->counter_next.fetch_add(1) % kCounterRing);
+}
+
+int read_counter(unsigned long long* d, hipStream_t s, uint64_t* out) {
+  unsigned long long h = 0;
+  HKV_HIP(hipMemcpyAsync(&h, d, sizeof h, hipMemcpyDeviceToHost, s));
+  HKV_HIP(hipStreamSynchronize(s));
+  *out = h;
+  return HKV_SUCCESS;
+}
+
+/* The memory of one table geometry. */
+struct TableMem {
+  void* d_meta;
+  uint64_t meta_bytes;
+  void* d_values;
+  void* h_values;
+};
+
+void free_arenas(hkv_table* t, TableMem& m) {
+  table_free(t, 0, m.d_meta);
+  table_free(t, 0, m.d_values);
+  table_free(t, 1, m.h_values);
+  m = TableMem{};
+}
+
+/* Arenas for `buckets_num` buckets, filled with EMPTY: the geometry fields of
+ * `v` (everything that does not depend on the bucket count is taken as is).
+ * On failure the caller frees what `m` holds. */
+int alloc_arenas(hkv_table* t, uint64_t buckets_num, View& v, TableMem& m) {
+  v.buckets_num = buckets_num;
+  v.capacity = buckets_num * kBucketSize;
+  v.pow2_buckets = ispow2(buckets_num);
+  /* metadata arena: digests | keys | scores | sizes, each 256-byte aligned */
+  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
+  const uint64_t off_keys = up(v.capacity);
+  const uint64_t off_scores = off_keys + up(v.capacity * 8);
+  const uint64_t off_sizes = off_scores + up(v.capacity * 8);
+  m.meta_bytes = off_sizes + up(v.buckets_num * 4);
+  HKV_TRY(table_alloc(t, 0, &m.d_meta, m.meta_bytes));
+  uint8_t* base = (uint8_t*)m.d_meta;
+  v.digests = base;
+  v.keys = (uint64_t*)(base + off_keys);
+  v.scores = (uint64_t*)(base + off_scores);
+  v.sizes = (int32_t*)(base + off_sizes);
+  /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
+   * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
+  const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
+  const uint64_t hbm_buckets =
+      std::min<uint64_t>(v.buckets_num, t->opts.max_hbm_for_vectors / bucket_bytes);
+  v.hbm_slots = hbm_buckets * kBucketSize;
+  v.values = nullptr;
+  v.host_values = nullptr;
+  if (hbm_buckets) {
+    HKV_TRY(table_alloc(t, 0, &m.d_values, hbm_buckets * bucket_bytes));
+    v.values = (uint8_t*)m.d_values;
+  }
+  if (hbm_buckets != v.buckets_num) {
+    HKV_TRY(table_alloc(t, 1, &m.h_values, (v.buckets_num - hbm_buckets) * bucket_bytes));
+    void* dp = nullptr;
+    hipError_t e = hipHostGetDevicePointer(&dp, m.h_values, 0);
+    if (e != hipSuccess)
+      return fail(HKV_ERROR_HIP, "hipHostGetDevicePointer: %s", hipGetErrorString(e));
+    v.host_values = (uint8_t*)dp;
+  }
+  const uint64_t groups = v.capacity / 16;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, 0, v, 1);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e != hipSuccess) return fail(HKV_ERROR_HIP, "table fill: %s", hipGetErrorString(e));
+  return HKV_SUCCESS;
+}
+
+/* One doubling: new arenas, rehash, swap.  Caller holds the inserter role and
+ * the device is idle. */
+int double_table(hkv_table* t, hipStream_t s) {
+  View nv = t->view;
+  TableMem mem{};
+  int rc = alloc_arenas(t, t->view.buckets_num * 2, nv, mem);
+  if (rc) {
+    free_arenas(t, mem);
+    return rc;
+  }
+  const uint64_t waves = t->view.capacity / kWave;
+  hipLaunchKernelGGL(rehash_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, t->view, nv);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e != hipSuccess) {
+    free_arenas(t, mem);
+    return fail(HKV_ERROR_HIP, "rehash: %s", hipGetErrorString(e));
+  }
+  TableMem old{t->d_meta, t->meta_bytes, t->d_values, t->h_values};
+  t->d_meta = mem.d_meta;
+  t->meta_bytes = mem.meta_bytes;
+  t->d_values = mem.d_values;
+  t->h_values = mem.h_values;
+  t->view = nv;
+  t->pure_hbm = nv.hbm_slots == nv.capacity;
+  free_arenas(t, old);
+  return HKV_SUCCESS;
+}
+
+/* reserve, merlin_hashtable.cuh:3503-3541 */
+int reserve_impl(hkv_table* t, uint64_t new_capacity, hipStream_t s) {
+  if (t->reach_max_capacity || new_capacity > t->opts.max_capacity) {
+    t->reach_max_capacity = t->view.capacity * 2 > t->opts.max_capacity;
+    return HKV_SUCCESS;
+  }
+  {
+    LockGuard g(t, StreamGroupLock::kInserter, s);
+    HKV_HIP(g.acquire());
+    /* with exclusive access, wait for everything that still uses the arenas */
+    HKV_HIP(hipDeviceSynchronize());
+    while (t->view.capacity < new_capacity && t->view.capacity * 2 <= t->opts.max_capacity)
+      HKV_TRY(double_table(t, s));
+    t->reach_max_capacity = t->view.capacity * 2 > t->opts.max_capacity;
+  }
+  return HKV_SUCCESS;
+}
+
+/* fast_load_factor, merlin_hashtable.cuh:3796-3830: the first min(buckets,
+ * 1024) buckets stand for the table; the incoming batch counts as all new */
+int fast_load_factor(hkv_table* t, uint64_t delta, hipStream_t s, float* out) {
+  const uint32_t n = (uint32_t)std::min<uint64_t>(t->view.buckets_num, 1024);
+  unsigned long long* d = take_counter(t);
+  {
+    LockGuard g(t, StreamGroupLock::kReader, s);
+    HKV_HIP(g.acquire());
+    hipLaunchKernelGGL(partial_size_kernel, dim3(1), dim3(256), 0, s, t->view, n, d);
+    HKV_HIP(hipGetLastError());
+  }
+  uint64_t sum = 0;
+  HKV_TRY(read_counter(d, s, &sum));
+  *out = (float)((delta * 1.0) / (t->view.capacity * 1.0) + (sum * 1.0) / (kBucketSize * n * 1.0));
+  return HKV_SUCCESS;
+}
+
+/* the growth loop at the head of every inserting call
+ * (merlin_hashtable.cuh:1151-1154, 1369-1372, 1604-1607, 1712-1715, 1898-1901) */
+int grow_for(hkv_table* t, uint64_t n, hipStream_t s) {
+  while (!t->reach_max_capacity) {
+    float lf = 0.f;
+    HKV_TRY(fast_load_factor(t, n, s, &lf));
+    if (!(lf > t->opts.max_load_factor)) break;
+    HKV_TRY(reserve_impl(t, t->view.capacity * 2, s));
+  }
+  return HKV_SUCCESS;
+}
+
 template <int OP>
 int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
                hipStream_t s) {
+  HKV_TRY(grow_for(t, a.n, s));
   a.epoch = t->epoch;
   a.clock = t->clock;
   a.value_kind = t->opts.value_kind;
@@ -450,22 +607,6 @@ void launch_size_if(const hkv_table* t, uint64_t pattern, uint64_t threshold,
                      t->view, Pred(), pattern, threshold, d_out);
 }
 
-constexpr unsigned kCounterRing = 32;
-
-/* Calls that return a count synchronise before they return, so at most one
- * word per concurrently calling host thread is in use. */
-unsigned long long* take_counter(const hkv_table* t) {
-  return t->d_counters + (t->counter_next.fetch_add(1) % kCounterRing);
-}
-
-int read_counter(unsigned long long* d, hipStream_t s, uint64_t* out) {
-  unsigned long long h = 0;
-  HKV_HIP(hipMemcpyAsync(&h, d, sizeof h, hipMemcpyDeviceToHost, s));
-  HKV_HIP(hipStreamSynchronize(s));
-  *out = h;
-  return HKV_SUCCESS;
-}
-
 int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) {
   if (!o || !out) return fail(HKV_ERROR_ARGUMENT, "null argument");
   /* HashTable::init, merlin_hashtable.cuh:1016-1048 */
@@ -483,12 +624,6 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
                 "initial required buckets number");
   if (o->max_bucket_size != kBucketSize)
     return fail(HKV_ERROR_UNSUPPORTED, "only max_bucket_size == 128 is supported");
-  /* a table with init_capacity * 2 <= max_capacity grows by rehashing in the
-   * reference (merlin_hashtable.cuh:1151-1154); refuse rather than never grow */
-  if (o->init_capacity * 2 <= std::max(o->init_capacity, o->max_capacity))
-    return fail(HKV_ERROR_UNSUPPORTED,
-                "growable tables (init_capacity * 2 <= max_capacity) need rehash, "
-                "which is not supported: set init_capacity == max_capacity");
   if (o->io_by_cpu && o->max_hbm_for_vectors != 0)
     return fail(HKV_ERROR_CHECK,
                 "[HierarchicalKV] `io_by_cpu` should not be true when "
@@ -514,6 +649,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->own_alloc = al == nullptr;
   if (al) t->alloc = *al;
   t->d_meta = nullptr;
+  t->d_values = nullptr;
   t->d_counters = nullptr;
   t->h_values = nullptr;
   t->d_scratch = nullptr;
@@ -587,54 +723,26 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   v.empty_digest = (uint8_t)(fmix64(v.empty_key) >> 32);
   v.reclaim_digest = (uint8_t)(fmix64(v.reclaim_key) >> 32);
 
-  /* metadata arena: digests | keys | scores | sizes, each 256-byte aligned */
-  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
-  const uint64_t off_keys = up(v.capacity);
-  const uint64_t off_scores = off_keys + up(v.capacity * 8);
-  const uint64_t off_sizes = off_scores + up(v.capacity * 8);
-  t->meta_bytes = off_sizes + up(v.buckets_num * 4);
-  int rc = table_alloc(t, 0, &t->d_meta, t->meta_bytes);
-  if (rc) return bail(rc);
-  uint8_t* m = (uint8_t*)t->d_meta;
-  v.digests = m;
-  v.keys = (uint64_t*)(m + off_keys);
-  v.scores = (uint64_t*)(m + off_scores);
-  v.sizes = (int32_t*)(m + off_sizes);
-  void* cnt = nullptr;
-  rc = table_alloc(t, 0, &cnt, kCounterRing * sizeof(unsigned long long));
-  if (rc) return bail(rc);
-  t->d_counters = (unsigned long long*)cnt;
-
-  /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
-   * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
-  const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
-  uint64_t hbm_buckets = std::min<uint64_t>(v.buckets_num, o->max_hbm_for_vectors / bucket_bytes);
-  v.hbm_slots = hbm_buckets * kBucketSize;
-  t->pure_hbm = hbm_buckets == v.buckets_num;
-  if (hbm_buckets) {
-    void* p = nullptr;
-    rc = table_alloc(t, 0, &p, hbm_buckets * bucket_bytes);
-    if (rc) return bail(rc);
-    v.values = (uint8_t*)p;
-  }
-  if (!t->pure_hbm) {
-    void* p = nullptr;
-    rc = table_alloc(t, 1, &p, (v.buckets_num - hbm_buckets) * bucket_bytes);
-    if (rc) return bail(rc);
-    t->h_values = p;
-    void* dp = nullptr;
-    hipError_t e = hipHostGetDevicePointer(&dp, p, 0);
-    if (e != hipSuccess) {
-      return bail(fail(HKV_ERROR_HIP, "hipHostGetDevicePointer: %s", hipGetErrorString(e)));
+  TableMem mem{};
+  {
+    int rc = alloc_arenas(t, v.buckets_num, v, mem);
+    if (rc) {
+      free_arenas(t, mem);
+      return bail(rc);
     }
-    v.host_values = (uint8_t*)dp;
   }
-
-  const uint64_t groups = v.capacity / 16;
-  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, 0, v, 1);
-  hipError_t e = hipGetLastError();
-  if (e == hipSuccess) e = hipDeviceSynchronize();
-  if (e != hipSuccess) return bail(fail(HKV_ERROR_HIP, "table fill: %s", hipGetErrorString(e)));
+  t->d_meta = mem.d_meta;
+  t->meta_bytes = mem.meta_bytes;
+  t->d_values = mem.d_values;
+  t->h_values = mem.h_values;
+  t->pure_hbm = v.hbm_slots == v.capacity;
+  void* cnt = nullptr;
+  {
+    int rc = table_alloc(t, 0, &cnt, kCounterRing * sizeof(unsigned long long));
+    if (rc) return bail(rc);
+  }
+  t->d_counters = (unsigned long long*)cnt;
+  t->reach_max_capacity = o->init_capacity * 2 > o->max_capacity; /* merlin_hashtable.cuh:1064 */
   *out = t;
   return HKV_SUCCESS;
 }
@@ -681,7 +789,7 @@ int hkv_table_destroy(hkv_table* t) {
   table_free(t, 0, t->d_meta);
   table_free(t, 0, t->d_counters);
   table_free(t, 0, t->d_scratch);
-  table_free(t, 0, t->view.values);
+  table_free(t, 0, t->d_values);
   table_free(t, 1, t->h_values);
   delete t;
   return HKV_SUCCESS;
@@ -940,6 +1048,10 @@ int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t strea
   hipLaunchKernelGGL(erase_kernel, dim3(grid_for(n)), dim3(kWave), 0, s, t->view, keys, n);
   HKV_HIP(hipGetLastError());
   return HKV_SUCCESS;
+}
+
+int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream) {
+  return reserve_impl(t, new_capacity, (hipStream_t)stream);
 }
 
 int hkv_clear(hkv_table* t, hkv_stream_t stream) {

@@ -175,6 +175,9 @@ class HashTable:
     def clear(self, stream=None):
         _check(lib.hkv_clear(self._h, _stream(stream)))
 
+    def reserve(self, new_capacity, stream=None):
+        _check(lib.hkv_reserve(self._h, new_capacity, _stream(stream)))
+
     # -- readers ---------------------------------------------------------------
     def find(self, n, keys, values, founds, scores=None, stream=None):
         _check(lib.hkv_find(self._h, n, _ptr(keys), _ptr(values), _ptr(founds), _ptr(scores),

@@ -227,6 +227,12 @@ int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys,
               hkv_stream_t stream);
 /* HashTable::clear, merlin_hashtable.cuh:3059-3078 */
 int hkv_clear(hkv_table* t, hkv_stream_t stream);
+/* HashTable::reserve, merlin_hashtable.cuh:3503-3541: doubles the bucket count
+ * (rehash) until capacity >= new_capacity or max_capacity would be passed.
+ * Tables created with init_capacity * 2 <= max_capacity also grow by
+ * themselves at the head of every inserting call, as the reference's do
+ * (merlin_hashtable.cuh:1151-1154).  Synchronises the device. */
+int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream);
 
 /* HashTable::export_batch (device counter), merlin_hashtable.cuh:3099-3147 */
 int hkv_export_batch(const hkv_table* t, uint64_t n, uint64_t offset,

@@ -21,8 +21,7 @@
  *   GB / MB / KB ......... merlin/utils.cuh:338-342
  *
  * Not provided (outside this build's scope, the call throws
- * std::runtime_error): reserve() to a larger capacity and automatic growth,
- * lock_keys / unlock_keys, find_and_update, the *_v2 predicate forms and
+ * std::runtime_error): lock_keys / unlock_keys, find_and_update, the *_v2 predicate forms and
  * for_each, TableMode::kMemory, S = uint32_t.
  */
 #ifndef MERLIN_HASHTABLE_HPP_
@@ -686,9 +685,9 @@ class HashTable : public HashTableBase<K, V, S> {
 
   size_type capacity() const override { return hkv_capacity(table_); }
 
-  void reserve(const size_type new_capacity, hipStream_t = 0) override {
-    if (new_capacity <= capacity()) return;
-    throw std::runtime_error("reserve() to a larger capacity (rehash) is not supported");
+  /* merlin_hashtable.cuh:3503-3541 */
+  void reserve(const size_type new_capacity, hipStream_t stream = 0) override {
+    throw_on_error_(hkv_reserve(table_, new_capacity, stream));
   }
 
   float load_factor(hipStream_t stream = 0) const override {

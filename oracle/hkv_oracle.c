@@ -79,6 +79,7 @@ struct hkvo_table {
   uint64_t epoch;
   int clock_mode;
   uint64_t clock_base;
+  int reach_max_capacity; /* merlin_hashtable.cuh:1064 */
 };
 
 static __thread char g_err[512];
@@ -206,6 +207,7 @@ int hkvo_create(const hkv_options* o, int hybrid_refusal, hkvo_table** out) {
   t->empty_digest = (uint8_t)(hkvo_murmur3_fmix64(t->empty_key) >> 32);
   t->reclaim_digest = (uint8_t)(hkvo_murmur3_fmix64(t->reclaim_key) >> 32);
   t->epoch = IGNORED_EPOCH;
+  t->reach_max_capacity = o->init_capacity * 2 > o->max_capacity;
   t->digests = (uint8_t*)malloc(t->capacity);
   t->keys = (uint64_t*)malloc(t->capacity * 8);
   t->scores = (uint64_t*)calloc(t->capacity, 8);
@@ -491,6 +493,101 @@ static void commit_meta(hkvo_table* t, int strategy, const occupy_t* r,
   if (r->result == OCC_EMPTY || r->result == OCC_RECLAIMED) t->sizes[r->bkt]++;
 }
 
+/* ---- growth -------------------------------------------------------------------
+ * reserve (merlin_hashtable.cuh:3503-3541): while capacity < new_capacity and
+ * doubling stays within max_capacity, double the number of buckets
+ * (double_capacity, core_kernels.cuh:386-401) and move every live key whose
+ * bucket changed (rehash_kernel_for_fast_mode, core_kernels.cuh:540-591; the
+ * key goes to the first EMPTY slot of its new bucket at or after its start
+ * position, move_key_to_new_bucket :494-537).  Tombstones stay where they are.
+ * The reference also compacts the old bucket towards start positions
+ * (defragmentation_for_rehash :445-492); slot positions are not observable
+ * through the API and lookups here scan the whole bucket, so that step is left
+ * out. */
+static int double_capacity(hkvo_table* t) {
+  const uint64_t ob = t->buckets_num, nb = ob * 2, ncap = nb * BUCKET;
+  uint8_t* dg = (uint8_t*)realloc(t->digests, ncap);
+  if (dg) t->digests = dg;
+  uint64_t* ks = (uint64_t*)realloc(t->keys, ncap * 8);
+  if (ks) t->keys = ks;
+  uint64_t* sc = (uint64_t*)realloc(t->scores, ncap * 8);
+  if (sc) t->scores = sc;
+  int32_t* sz = (int32_t*)realloc(t->sizes, nb * 4);
+  if (sz) t->sizes = sz;
+  uint8_t* vs = (uint8_t*)realloc(t->values, ncap * (uint64_t)t->vb);
+  if (vs) t->values = vs;
+  if (!dg || !ks || !sc || !sz || !vs) return fail(HKV_ERROR_RUNTIME, "out of memory");
+  memset(t->digests + t->capacity, t->empty_digest, ncap - t->capacity);
+  for (uint64_t i = t->capacity; i < ncap; i++) t->keys[i] = t->empty_key;
+  memset(t->scores + t->capacity, 0, (ncap - t->capacity) * 8);
+  memset(t->sizes + ob, 0, ob * 4);
+  memset(t->values + t->capacity * (uint64_t)t->vb, 0, (ncap - t->capacity) * (uint64_t)t->vb);
+  t->buckets_num = nb;
+  t->capacity = ncap;
+  for (uint64_t b = 0; b < ob; b++) {
+    for (uint64_t p = 0; p < BUCKET; p++) {
+      const uint64_t s = b * BUCKET + p;
+      const uint64_t k = t->keys[s];
+      if (k == t->empty_key || k == t->reclaim_key) continue;
+      uint64_t nbkt;
+      uint32_t start;
+      uint8_t digest;
+      hkvo_locate(k, nb, &nbkt, &start, &digest);
+      if (nbkt == b) continue;
+      uint64_t d = UINT64_MAX;
+      for (uint64_t off = 0; off < BUCKET; off++) {
+        const uint64_t q = nbkt * BUCKET + ((start + off) & (BUCKET - 1));
+        if (t->keys[q] == t->empty_key) {
+          d = q;
+          break;
+        }
+      }
+      if (d == UINT64_MAX) return fail(HKV_ERROR_RUNTIME, "rehash: new bucket is full");
+      t->keys[d] = k;
+      t->digests[d] = t->digests[s];
+      t->scores[d] = t->scores[s];
+      memcpy(t->values + d * t->vb, t->values + s * t->vb, t->vb);
+      t->sizes[nbkt]++;
+      t->keys[s] = t->empty_key;
+      t->digests[s] = t->empty_digest;
+      t->sizes[b]--;
+    }
+  }
+  return HKV_SUCCESS;
+}
+
+int hkvo_reserve(hkvo_table* t, uint64_t new_capacity) {
+  if (t->reach_max_capacity || new_capacity > t->opts.max_capacity) {
+    t->reach_max_capacity = t->capacity * 2 > t->opts.max_capacity;
+    return HKV_SUCCESS;
+  }
+  while (t->capacity < new_capacity && t->capacity * 2 <= t->opts.max_capacity) {
+    int rc = double_capacity(t);
+    if (rc) return rc;
+  }
+  t->reach_max_capacity = t->capacity * 2 > t->opts.max_capacity;
+  return HKV_SUCCESS;
+}
+
+/* fast_load_factor, merlin_hashtable.cuh:3796-3830: sizes of the first
+ * min(buckets, 1024) buckets, plus the incoming batch as if it were all new */
+static float fast_load_factor(const hkvo_table* t, uint64_t delta) {
+  const uint64_t N = t->buckets_num < 1024 ? t->buckets_num : 1024;
+  int64_t sum = 0;
+  for (uint64_t b = 0; b < N; b++) sum += t->sizes[b];
+  return (float)((delta * 1.0) / (t->capacity * 1.0) + (sum * 1.0) / (BUCKET * N * 1.0));
+}
+
+/* the growth loop at the head of every inserting call
+ * (merlin_hashtable.cuh:1151-1154, 1369-1372, 1604-1607, 1712-1715, 1898-1901) */
+static int grow_for(hkvo_table* t, uint64_t n) {
+  while (!t->reach_max_capacity && fast_load_factor(t, n) > t->opts.max_load_factor) {
+    int rc = hkvo_reserve(t, t->capacity * 2);
+    if (rc) return rc;
+  }
+  return HKV_SUCCESS;
+}
+
 static inline int strategy_of(const hkvo_table* t, int ignore) {
   return ignore ? HKV_CUSTOMIZED : t->strategy;
 }
@@ -559,6 +656,10 @@ int hkvo_insert_or_assign(hkvo_table* t, uint64_t n, const uint64_t* keys,
                           const void* values, const uint64_t* scores,
                           int ignore) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   int strategy = strategy_of(t, ignore);
   if (!ignore) {
     int rc = check_scores_arg(t, strategy, scores);
@@ -580,6 +681,10 @@ int hkvo_insert_and_evict(hkvo_table* t, uint64_t n, const uint64_t* keys,
                           uint64_t* ek, void* ev_, uint64_t* es,
                           uint64_t* counter, int ignore) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   if (t->hybrid_refusal) /* merlin_hashtable.cuh:1384-1386 */
     return fail(HKV_ERROR_RUNTIME,
                 "insert_and_evict is not supported in hybrid mode");
@@ -620,6 +725,10 @@ int hkvo_insert_and_evict(hkvo_table* t, uint64_t n, const uint64_t* keys,
 int hkvo_find_or_insert(hkvo_table* t, uint64_t n, const uint64_t* keys,
                         void* values_, const uint64_t* scores, int ignore) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   int strategy = strategy_of(t, ignore);
   if (!ignore) {
     int rc = check_scores_arg(t, strategy, scores);
@@ -654,6 +763,10 @@ int hkvo_find_or_insert_slot(hkvo_table* t, uint64_t n, const uint64_t* keys,
                              uint64_t* slots, uint8_t* founds,
                              const uint64_t* scores, int ignore) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   int strategy = strategy_of(t, ignore);
   if (!ignore) {
     int rc = check_scores_arg(t, strategy, scores);
@@ -713,6 +826,10 @@ int hkvo_accum_or_assign(hkvo_table* t, uint64_t n, const uint64_t* keys,
                          const void* vd_, const uint8_t* flags,
                          const uint64_t* scores, int ignore) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   if (t->opts.value_kind == HKV_VALUE_BYTES)
     return fail(HKV_ERROR_ARGUMENT, "accum_or_assign needs an arithmetic value_kind");
   int strategy = strategy_of(t, ignore);
@@ -983,6 +1100,10 @@ int hkvo_insert_or_assign_mt(hkvo_table* t, uint64_t n, const uint64_t* keys,
                              const void* values, const uint64_t* scores,
                              int ignore, int threads) {
   if (n == 0) return HKV_SUCCESS;
+  {
+    int grc = grow_for(t, n);
+    if (grc) return grc;
+  }
   if (threads <= 0) threads = hkvo_online_cores();
   int strategy = strategy_of(t, ignore);
   if (!ignore) {

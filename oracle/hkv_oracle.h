@@ -84,6 +84,10 @@ int hkvo_find_slot(const hkvo_table* t, uint64_t n, const uint64_t* keys,
 int hkvo_contains(const hkvo_table* t, uint64_t n, const uint64_t* keys,
                   uint8_t* founds);
 int hkvo_erase(hkvo_table* t, uint64_t n, const uint64_t* keys);
+/* reserve + rehash (merlin_hashtable.cuh:3503-3541).  Every inserting call
+ * above also runs the reference's growth loop first (fast_load_factor >
+ * max_load_factor => reserve(2 * capacity), merlin_hashtable.cuh:1151-1154). */
+int hkvo_reserve(hkvo_table* t, uint64_t new_capacity);
 int hkvo_clear(hkvo_table* t);
 int hkvo_export_batch_if(const hkvo_table* t, int predicate, uint64_t pattern,
                          uint64_t threshold, uint64_t n, uint64_t offset,

@@ -49,8 +49,6 @@ def test_option_checks_need_no_gpu():
             t.init(default_options(init_capacity=1024, max_capacity=1024, **bad))
     t = HashTable()
     with pytest.raises(NotImplementedError):
-        t.init(default_options(init_capacity=1024, max_capacity=4096))  # growable
-    with pytest.raises(NotImplementedError):
         t.init(default_options(init_capacity=1024, max_capacity=1024, table_mode=1))
     with pytest.raises(NotImplementedError):
         t.init(default_options(init_capacity=1024, max_capacity=1024, score_size=4))

@@ -374,3 +374,53 @@ def test_error_classes(oracle):
         t2.accum_or_assign(8, k, v, torch.zeros(8, dtype=torch.bool, device=DEV))
     t.close()
     t2.close()
+
+
+def test_growth_reserve_and_rehash(oracle):
+    # reserve / rehash and the growth loop at the head of the inserting calls
+    # (merlin_hashtable.cuh:3503-3541, 1151-1154); scenario of test_rehash
+    # (merlin_hashtable_test.cc.cu:1078-1200) at a larger size, plus evictions once
+    # max_capacity is reached
+    dim, bs = 8, 3000
+    t, o, _ = make_pair(oracle, init_capacity=1 << 12, max_capacity=1 << 15, dim=dim,
+                        max_load_factor=0.5, evict_strategy=EvictStrategy.kCustomized)
+    assert t.capacity() == o.capacity() == 1 << 12
+    caps = []
+    for b in range(16):  # 48000 keys into at most 32768 slots
+        keys = w.unique_keys(77, b * bs, bs)
+        vals = w.values_from_keys(keys, dim)
+        sc = w.monotone_scores(b + 1, bs)
+        t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+        o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1), sc)
+        assert t.capacity() == o.capacity()
+        assert t.size() == o.size()
+        caps.append(t.capacity())
+    assert caps[0] > 1 << 12 and caps[-1] == 1 << 15 and sorted(caps) == caps
+    assert_same_table(t, o, dim * 4)
+    t.close()
+    # explicit reserve on a table that does not grow by itself
+    t, o, _ = make_pair(oracle, init_capacity=1 << 12, max_capacity=1 << 14, dim=dim,
+                        max_load_factor=4.0, evict_strategy=EvictStrategy.kLru)
+    t.set_clock(1, 1 << 40)
+    o.set_clock(1, 1 << 40)
+    for b in range(2):  # 6000 keys into 4096 slots: evictions, then tombstones
+        keys = w.unique_keys(78, b * bs, bs)
+        vals = w.values_from_keys(keys, dim)
+        t.insert_or_assign(bs, dev(keys), dev(vals))
+        o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1))
+    gone = w.unique_keys(78, bs, 500)
+    t.erase(500, dev(gone))
+    o.erase(gone)
+    for want in (5000, 1 << 14, 1 << 20):
+        t.reserve(want)
+        o.reserve(want)
+        assert t.capacity() == o.capacity()
+        assert t.size() == o.size()
+        assert_same_table(t, o, dim * 4)
+    assert t.capacity() == 1 << 14
+    keys = w.unique_keys(78, 2 * bs, bs)
+    vals = w.values_from_keys(keys, dim)
+    t.insert_or_assign(bs, dev(keys), dev(vals))
+    o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1))
+    assert_same_table(t, o, dim * 4)
+    t.close()

@@ -544,3 +544,65 @@ def test_multithreaded_baseline_equals_sequential(oracle):
     assert (f1 == f2).all() and (v1 == v2).all() and (s1 == s2).all()
     a.close()
     b.close()
+
+
+# ---- growth ----------------------------------------------------------------------
+
+def test_rehash_scenario_of_the_reference_test(oracle):
+    # tests/merlin_hashtable_test.cc.cu:1078-1200 (test_rehash): one bucket to start with, room
+    # for four; 256 keys arrive at once.  The growth loop at the head of insert_or_assign
+    # (fast_load_factor = 256/128 > 0.5, then 256/256 > 0.5) takes the table to 512 slots
+    # before the first key goes in, so nothing is evicted.
+    o = default_options(init_capacity=128, max_capacity=512, dim=4, reserved_key_start_bit=5,
+                        evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    assert t.capacity() == 128
+    keys = w.unique_keys(7, 0, 256)
+    keys = keys[(keys & np.uint64(0x60)) != np.uint64(0x60)][:200]  # keep clear of the reserved patterns at bit 5
+    t.insert_or_assign(keys, vals_of(keys, 4), keys.copy())
+    assert t.capacity() == 512
+    per_bucket = np.bincount([int(oracle.locate(int(k), 4)[0]) for k in keys], minlength=4)
+    assert per_bucket.max() <= 128  # so every key fits: the size is the number of keys
+    assert t.size() == len(keys)
+    t.reserve(512)
+    assert t.capacity() == 512 and t.size() == len(keys)
+    v, f, sc = t.find(keys)
+    assert f.all() and (sc == keys).all() and (v == vals_of(keys, 4)).all()
+    t.close()
+
+
+def test_reserve_keeps_the_map_and_doubles_until_the_limit(oracle):
+    # reserve (merlin_hashtable.cuh:3503-3541) against a python dict: same entries before and
+    # after, every key in the bucket its hash names for the new bucket count, tombstones
+    # still not counted, and no doubling past max_capacity.
+    o = default_options(init_capacity=1024, max_capacity=8192, dim=2, max_load_factor=2.0,
+                        evict_strategy=EvictStrategy.kCustomized)  # load factor 2: no growth on its own
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(11, 0, 900)
+    sc = w.monotone_scores(1, 900)
+    t.insert_or_assign(keys, vals_of(keys, 2), sc)
+    t.erase(keys[:50])
+    before = dict(zip(*[x.tolist() for x in (t.export_all()[0], t.export_all()[2])]))
+    assert t.capacity() == 1024 and t.size() == len(before)
+    t.reserve(2048)
+    assert t.capacity() == 2048
+    t.reserve(3000)  # next power of two
+    assert t.capacity() == 4096
+    t.reserve(1 << 20)  # beyond max_capacity: ignored (merlin_hashtable.cuh:3508-3511)
+    assert t.capacity() == 4096
+    t.reserve(8192)
+    assert t.capacity() == 8192
+    t.reserve(16384)
+    assert t.capacity() == 8192
+    k, v, s = t.export_all()
+    assert dict(zip(k.tolist(), s.tolist())) == before
+    assert (v == vals_of(k, 2)).all()
+    assert t.size() == len(before)
+    sizes = np.zeros(64, np.int64)
+    for key in k.tolist():
+        sizes[oracle.locate(key, 64)[0]] += 1
+    assert [t.bucket_size(b) for b in range(64)] == sizes.tolist()
+    _, f, _ = t.find(keys)
+    assert not f[:50].any()
+    assert f.tolist() == [k_ in before for k_ in keys.tolist()]  # (a few were evicted at 1024 slots)
+    t.close()
