@@ -97,6 +97,9 @@ SIGNATURES = {
     "hkv_contains": (_i, [_T, _u64, _p, _p, _p]),
     "hkv_erase": (_i, [_T, _u64, _p, _p]),
     "hkv_clear": (_i, [_T, _p]),
+    "hkv_lock_keys": (_i, [_T, _u64, _p, _p, _p, _p, _p]),
+    "hkv_unlock_keys": (_i, [_T, _u64, _p, _p, _p, _p]),
+    "hkv_find_and_update": (_i, [_T, _u64, _p, _p, _p, _p, _p]),
     "hkv_reserve": (_i, [_T, C.c_uint64, _p]),
     "hkv_export_batch": (_i, [_T, _u64, _u64, _p, _p, _p, _p, _p]),
     "hkv_export_batch_if": (_i, [_T, _i, _u64, _u64, _u64, _u64, _p, _p, _p, _p, _p]),

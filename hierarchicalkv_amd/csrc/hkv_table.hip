@@ -24,6 +24,7 @@
 #include "hkv_misc.hpp"
 #include "hkv_upsert.hpp"
 #include "hkv_grouped.hpp"
+#include "hkv_keylocks.hpp"
 
 using namespace hkv;
 
@@ -160,6 +161,7 @@ struct hkv_table {
   uint64_t scratch_bytes;
   int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
+  bool keys_may_be_locked; /* lock_keys has been called: LOCKED key words may sit in the table */
 };
 
 namespace {
@@ -294,6 +296,7 @@ GroupPlan plan_grouped(const hkv_table* t, uint64_t n) {
   const uint64_t buckets = t->view.buckets_num;
   /* the second phase has no locks: it needs the inserter's exclusivity */
   if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return p;
+  if (t->keys_may_be_locked) return p; /* the second phase does not look at key words */
   /* bins of about 128 keys if every key of the batch were absent */
   uint32_t shift = 0;
   while (shift < (uint32_t)kGrpMaxBpbShift && (n << (shift + 1)) <= 128 * buckets) shift++;
@@ -545,13 +548,17 @@ int grow_for(hkv_table* t, uint64_t n, hipStream_t s) {
   return HKV_SUCCESS;
 }
 
+/* `hybrid_rule`: the operation follows the lock-key kernels of hybrid mode when
+ * the table is not pure HBM (insert_or_assign, find_or_insert); the pointer
+ * overload always does. */
 template <int OP>
-int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
-               hipStream_t s) {
+int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_t s) {
   HKV_TRY(grow_for(t, a.n, s));
   a.epoch = t->epoch;
   a.clock = t->clock;
   a.value_kind = t->opts.value_kind;
+  const bool refuse_equal = OP == kOpFindOrInsertPtr || (hybrid_rule && !t->pure_hbm);
+  a.refuse_equal = refuse_equal;
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
@@ -559,14 +566,9 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool locked_rule,
     if constexpr (OP != kOpFindOrInsertPtr) plan = plan_grouped(t, a.n);
     if (plan.feasible) {
       if constexpr (OP != kOpFindOrInsertPtr)
-        HKV_TRY(run_grouped<OP>(t, a, vec, locked_rule, plan, s));
-    } else if constexpr (OP == kOpFindOrInsertPtr) {
+        HKV_TRY(run_grouped<OP>(t, a, vec, refuse_equal, plan, s));
+    } else if (refuse_equal || t->keys_may_be_locked) {
       launch_upsert<OP, true>(vec, t->view, a, s);
-    } else if constexpr (OP == kOpInsertOrAssign || OP == kOpFindOrInsert) {
-      if (locked_rule)
-        launch_upsert<OP, true>(vec, t->view, a, s);
-      else
-        launch_upsert<OP, false>(vec, t->view, a, s);
     } else {
       launch_upsert<OP, false>(vec, t->view, a, s);
     }
@@ -654,6 +656,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->h_values = nullptr;
   t->d_scratch = nullptr;
   t->scratch_bytes = 0;
+  t->keys_may_be_locked = false;
   /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default while the
    * two-phase path is being tuned), "auto" = two-phase for large batches,
    * "grouped" = two-phase whenever it is possible (tests) */
@@ -809,7 +812,7 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.n = n;
   a.strategy = strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
-  return run_upsert<kOpInsertOrAssign>(t, a, vec, !t->pure_hbm, (hipStream_t)stream);
+  return run_upsert<kOpInsertOrAssign>(t, a, vec, true, (hipStream_t)stream);
 }
 
 int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
@@ -888,7 +891,7 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.n = n;
   a.strategy = strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
-  return run_upsert<kOpFindOrInsert>(t, a, vec, !t->pure_hbm, (hipStream_t)stream);
+  return run_upsert<kOpFindOrInsert>(t, a, vec, true, (hipStream_t)stream);
 }
 
 int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
@@ -1040,6 +1043,68 @@ int hkv_contains(const hkv_table* t, uint64_t n, const uint64_t* keys,
   return HKV_SUCCESS;
 }
 
+int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys, uint64_t** locked_key_ptrs,
+                  uint8_t* success, const uint64_t* scores, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
+  hipStream_t s = (hipStream_t)stream;
+  TouchArgs a{};
+  a.keys = keys;
+  a.scores = const_cast<uint64_t*>(scores);
+  a.key_ptrs = locked_key_ptrs;
+  a.flags = success;
+  a.n = n;
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.strategy = t->opts.evict_strategy;
+  {
+    LockGuard g(t, StreamGroupLock::kInserter, s);
+    HKV_HIP(g.acquire());
+    t->keys_may_be_locked = true;
+    hipLaunchKernelGGL((touch_kernel<true>), dim3(grid_for(n)), dim3(kWave), 0, s, t->view, a);
+    HKV_HIP(hipGetLastError());
+  }
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
+}
+
+int hkv_unlock_keys(hkv_table* t, uint64_t n, uint64_t** locked_key_ptrs, const uint64_t* keys,
+                    uint8_t* success, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  hipStream_t s = (hipStream_t)stream;
+  LockGuard g(t, StreamGroupLock::kInserter, s);
+  HKV_HIP(g.acquire());
+  hipLaunchKernelGGL(unlock_keys_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, t->view,
+                     n, locked_key_ptrs, keys, success);
+  HKV_HIP(hipGetLastError());
+  return HKV_SUCCESS;
+}
+
+int hkv_find_and_update(hkv_table* t, uint64_t n, const uint64_t* keys, void** values,
+                        uint8_t* founds, uint64_t* scores, hkv_stream_t stream) {
+  if (n == 0) return HKV_SUCCESS;
+  HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
+  hipStream_t s = (hipStream_t)stream;
+  TouchArgs a{};
+  a.keys = keys;
+  a.scores = scores;
+  a.value_ptrs = values;
+  a.flags = founds;
+  a.n = n;
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.strategy = t->opts.evict_strategy;
+  {
+    /* it writes scores, so it runs with the updaters, not with the readers */
+    LockGuard g(t, StreamGroupLock::kUpdater, s);
+    HKV_HIP(g.acquire());
+    hipLaunchKernelGGL((touch_kernel<false>), dim3(grid_for(n)), dim3(kWave), 0, s, t->view, a);
+    HKV_HIP(hipGetLastError());
+  }
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
+}
+
 int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t stream) {
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
@@ -1055,6 +1120,7 @@ int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream) {
 }
 
 int hkv_clear(hkv_table* t, hkv_stream_t stream) {
+  t->keys_may_be_locked = false;
   hipStream_t s = (hipStream_t)stream;
   LockGuard g(t, StreamGroupLock::kInserter, s);
   HKV_HIP(g.acquire());

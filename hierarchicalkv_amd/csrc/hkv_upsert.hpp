@@ -61,6 +61,8 @@ struct UpsertArgs {
   Clock clock;
   int32_t value_kind;
   int32_t strategy; /* hkv_evict_strategy; uniform, so a scalar branch */
+  int32_t refuse_equal; /* refuse when score <= min instead of < (hybrid and
+                           pointer kernels, upsert.cuh:1524, find_or_insert.cuh:1593) */
 };
 
 /* ScoreFunctor<Strategy>::desired_when_missed, kernel_utils.cuh:275-279,
@@ -422,10 +424,11 @@ __device__ __forceinline__ void bulk_evicted(int kind, const uint8_t* src, uint8
  * candidate, `hit` is the key's slot or -1, and (em_lo, em_hi) is the fresh
  * 128-bit mask of EMPTY digests.  Every lane of the wavefront must call this.
  */
+constexpr int kMaxLockedWaits = 64;
 __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uint32_t bkt,
                                                 uint32_t digest, bool pending, bool& reprobe,
                                                 int64_t& hit, uint64_t& em_lo, uint64_t& em_hi,
-                                                int lane) {
+                                                int& waited, int lane) {
   const int tile = lane >> 3, j = lane & 7;
   const int lane_base = lane & ~(kTile - 1);
 #pragma unroll 1
@@ -447,10 +450,13 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
         hi |= m << (16 * (q - 4));
     }
     if (j == r) {
-      if (found == -2) {
+      if (found == -2 && ++waited < kMaxLockedWaits) {
         __builtin_amdgcn_s_sleep(2);
       } else {
-        hit = found;
+        /* a slot that stays LOCKED this long is held by lock_keys, not by a
+         * wavefront of this launch: the key is not there to be found (the
+         * reference reads LOCKED as "another key", lookup_ptr.cuh:93-110) */
+        hit = found == -2 ? -1 : found;
         reprobe = false;
         em_lo = lo;
         em_hi = hi;
@@ -460,10 +466,12 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
 }
 
 /*
- * LOCKED_RULE: behaviour of the lock-key kernels used by the pointer overload
- * and by hybrid mode (find_ptr_or_insert.cuh:170-200, upsert.cuh:1478-1524):
- * slots whose key is LOCKED or EMPTY are invisible to the victim scan and a
- * key is refused when score <= min instead of score < min.
+ * LOCKED_RULE: the victim scan of the lock-key kernels used by the pointer
+ * overload and by hybrid mode (find_ptr_or_insert.cuh:170-200,
+ * upsert.cuh:1478-1524): slots whose key is LOCKED or EMPTY are invisible to
+ * it.  Also used once lock_keys may have left LOCKED slots in the table, which
+ * the plain scan would pick and wait for without end.  Whether a key is
+ * refused at score == min is a separate switch (UpsertArgs::refuse_equal).
  */
 template <int OP, int VEC, int UPL, bool LOCKED_RULE>
 __global__ void __launch_bounds__(kWave, HKV_UPSERT_MIN_WAVES)
@@ -502,6 +510,7 @@ upsert_kernel(View v, UpsertArgs a) {
   bool pending = (me.info & 0x100u) != 0;
   if (HKV_EXP_FLAG(4)) pending = false;
   bool reprobe = pending && hit < 0 && s_unsure[lane];
+  int waited = 0;
 
   /* The trip loop is controlled by a wavefront-uniform value only: all 64
    * lanes take part in every trip (the tile-cooperative steps read registers
@@ -509,7 +518,7 @@ upsert_kernel(View v, UpsertArgs a) {
   unsigned long long pend_mask = __ballot(pending);
   while (pend_mask) {
     if (__ballot(pending && reprobe))
-      settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, lane);
+      settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, waited, lane);
 
     const bool active = pending && !reprobe;
     const uint64_t desired = desired_when_missed(a, in_score, i);
@@ -607,7 +616,7 @@ upsert_kernel(View v, UpsertArgs a) {
     /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
     bool refused_now = false;
     if (want_scan) {
-      const bool refuse = (LOCKED_RULE ? (desired <= best) : (desired < best)) || HKV_EXP_FLAG(16);
+      const bool refuse = (a.refuse_equal ? (desired <= best) : (desired < best)) || HKV_EXP_FLAG(16);
       if (refuse) {
         refused_now = true;
         got = kStRefused;
@@ -765,11 +774,12 @@ assign_kernel(View v, AssignArgs a) {
   int64_t hit = s_slot[lane];
   bool reprobe = hit < 0 && s_unsure[lane];
   bool pending = (me.info & 0x100u) && (hit >= 0 || reprobe);
+  int waited = 0;
   uint64_t em_lo = 0, em_hi = 0;
   unsigned long long pend_mask = __ballot(pending);
   while (pend_mask) {
     if (__ballot(pending && reprobe))
-      settle_reprobes(v, key, me.bkt, me.info & 0xFFu, pending, reprobe, hit, em_lo, em_hi, lane);
+      settle_reprobes(v, key, me.bkt, me.info & 0xFFu, pending, reprobe, hit, em_lo, em_hi, waited, lane);
     int got = kStNone;
     if (pending && !reprobe) {
       if (hit < 0) {

@@ -169,6 +169,18 @@ class HashTable:
         _check(lib.hkv_assign_values(self._h, n, _ptr(keys), _ptr(values), _stream(stream),
                                      int(unique_key)))
 
+    def lock_keys(self, n, keys, locked_key_ptrs, success=None, stream=None, scores=None):
+        _check(lib.hkv_lock_keys(self._h, n, _ptr(keys), _ptr(locked_key_ptrs), _ptr(success),
+                                 _ptr(scores), _stream(stream)))
+
+    def unlock_keys(self, n, locked_key_ptrs, keys, success=None, stream=None):
+        _check(lib.hkv_unlock_keys(self._h, n, _ptr(locked_key_ptrs), _ptr(keys), _ptr(success),
+                                   _stream(stream)))
+
+    def find_and_update(self, n, keys, value_ptrs, founds, scores=None, stream=None, unique_key=True):
+        _check(lib.hkv_find_and_update(self._h, n, _ptr(keys), _ptr(value_ptrs), _ptr(founds),
+                                       _ptr(scores), _stream(stream)))
+
     def erase(self, n, keys, stream=None):
         _check(lib.hkv_erase(self._h, n, _ptr(keys), _stream(stream)))
 

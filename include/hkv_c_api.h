@@ -222,6 +222,26 @@ int hkv_find_ptr(const hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_contains(const hkv_table* t, uint64_t n, const uint64_t* keys,
                  uint8_t* founds /* bool[n] */, hkv_stream_t stream);
 
+/* HashTable::lock_keys, merlin_hashtable.cuh:1982-2012: every key that is
+ * present has its key word set to LOCKED and its score touched;
+ * locked_key_ptrs[i] = address of that key word, or null.  While keys are
+ * locked they are invisible to lookups, and slots holding them are never
+ * chosen as eviction victims.  Unlike the reference, the `scores` argument is
+ * checked against the eviction strategy as in the other calls. */
+int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys,
+                  uint64_t** locked_key_ptrs, uint8_t* success /* bool[n], may be null */,
+                  const uint64_t* scores, hkv_stream_t stream);
+/* HashTable::unlock_keys, merlin_hashtable.cuh:2026-2044 */
+int hkv_unlock_keys(hkv_table* t, uint64_t n, uint64_t** locked_key_ptrs,
+                    const uint64_t* keys, uint8_t* success /* may be null */,
+                    hkv_stream_t stream);
+/* HashTable::find_and_update, merlin_hashtable.cuh:2811-2843: find* that also
+ * touches the score of every key it finds; with `scores` given, scores[i] is
+ * the input of the score rule and receives the score after the touch. */
+int hkv_find_and_update(hkv_table* t, uint64_t n, const uint64_t* keys,
+                        void** values, uint8_t* founds, uint64_t* scores,
+                        hkv_stream_t stream);
+
 /* HashTable::erase, merlin_hashtable.cuh:2904-2930 */
 int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys,
               hkv_stream_t stream);

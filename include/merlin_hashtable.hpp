@@ -21,7 +21,7 @@
  *   GB / MB / KB ......... merlin/utils.cuh:338-342
  *
  * Not provided (outside this build's scope, the call throws
- * std::runtime_error): lock_keys / unlock_keys, find_and_update, the *_v2 predicate forms and
+ * std::runtime_error): the *_v2 predicate forms and
  * for_each, TableMode::kMemory, S = uint32_t.
  */
 #ifndef MERLIN_HASHTABLE_HPP_
@@ -516,13 +516,19 @@ class HashTable : public HashTableBase<K, V, S> {
                                            unique_key, ignore_evict_strategy));
   }
 
-  void lock_keys(const size_type, key_type const*, key_type**, bool* = nullptr, hipStream_t = 0,
-                 score_type const* = nullptr) override {
-    throw std::runtime_error("lock_keys is not supported");
+  /* merlin_hashtable.cuh:1982-2012 */
+  void lock_keys(const size_type n, key_type const* keys, key_type** locked_key_ptrs,
+                 bool* succeededs = nullptr, hipStream_t stream = 0,
+                 score_type const* scores = nullptr) override {
+    throw_on_error_(hkv_lock_keys(table_, n, u64(keys),
+                                  reinterpret_cast<uint64_t**>(locked_key_ptrs),
+                                  reinterpret_cast<uint8_t*>(succeededs), scores, stream));
   }
-  void unlock_keys(const size_type, key_type**, const key_type*, bool* = nullptr,
-                   hipStream_t = 0) override {
-    throw std::runtime_error("unlock_keys is not supported");
+  /* merlin_hashtable.cuh:2026-2044 */
+  void unlock_keys(const size_type n, key_type** locked_key_ptrs, const key_type* keys,
+                   bool* succeededs = nullptr, hipStream_t stream = 0) override {
+    throw_on_error_(hkv_unlock_keys(table_, n, reinterpret_cast<uint64_t**>(locked_key_ptrs),
+                                    u64(keys), reinterpret_cast<uint8_t*>(succeededs), stream));
   }
 
   void assign(const size_type n, const key_type* keys, const value_type* values,
@@ -561,9 +567,15 @@ class HashTable : public HashTableBase<K, V, S> {
     throw_on_error_(hkv_find_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
                                  reinterpret_cast<uint8_t*>(founds), scores, stream, unique_key));
   }
-  void find_and_update(const size_type, const key_type*, value_type**, bool*,
-                       score_type* = nullptr, hipStream_t = 0, bool = true) override {
-    throw std::runtime_error("find_and_update is not supported");
+  /* merlin_hashtable.cuh:2811-2843 */
+  void find_and_update(const size_type n, const key_type* keys, value_type** values, bool* founds,
+                       score_type* scores = nullptr, hipStream_t stream = 0,
+                       bool unique_key = true) override {
+    if (!unique_key)
+      throw std::runtime_error(
+          "Not support update score when keys are not unique or bucket capacity is small.");
+    throw_on_error_(hkv_find_and_update(table_, n, u64(keys), reinterpret_cast<void**>(values),
+                                        reinterpret_cast<uint8_t*>(founds), scores, stream));
   }
   void contains(const size_type n, const key_type* keys, bool* founds,
                 hipStream_t stream = 0) const override {

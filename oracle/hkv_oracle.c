@@ -462,7 +462,10 @@ static void decide(const hkvo_table* t, int strategy, uint64_t key,
   int min_pos = -1;
   for (uint32_t p = 0; p < BUCKET; p++) {
     if (s[p] < min_score) {
-      if (ptr_rule && (k[p] == t->locked_key || k[p] == t->empty_key)) continue;
+      /* a slot that lock_keys holds is never a victim: the reference's plain
+       * kernels would retry such a slot for ever (upsert.cuh:192-222) */
+      if (k[p] == t->locked_key) continue;
+      if (ptr_rule && k[p] == t->empty_key) continue;
       min_score = s[p];
       min_pos = (int)p;
     }
@@ -931,6 +934,71 @@ int hkvo_find_slot(const hkvo_table* t, uint64_t n, const uint64_t* keys,
     slots[i] = slot >= 0 ? (uint64_t)slot : UINT64_MAX;
     if (slot >= 0 && scores) scores[i] = t->scores[slot];
   }
+  return HKV_SUCCESS;
+}
+
+/* score of a key that is present, as the upsert kernels leave it
+ * (update_with_digest with is_insert = false) */
+static void touch_score(hkvo_table* t, uint64_t slot, const uint64_t* in, uint64_t i) {
+  uint64_t ns;
+  const uint64_t desired = desired_when_missed(t, t->strategy, in, i);
+  if (score_on_upsert(t, t->strategy, in, i, desired, 0, t->scores[slot], &ns))
+    t->scores[slot] = ns;
+}
+
+/* lock_keys (merlin_hashtable.cuh:1982-2012, lock_kernel_with_filter,
+ * core_kernels.cuh:1248-1362): a key that is present has its key word replaced
+ * by LOCKED and its score touched; slots[i] = its slot (the reference returns
+ * the address of the key word) or UINT64_MAX.  The score argument is checked
+ * as in the other calls; the reference does not check it here and reads
+ * through a null pointer when a strategy needs scores that were not given. */
+int hkvo_lock_keys(hkvo_table* t, uint64_t n, const uint64_t* keys, uint64_t* slots,
+                   uint8_t* success, const uint64_t* scores) {
+  if (n == 0) return HKV_SUCCESS;
+  int rc = check_scores_arg(t, t->strategy, scores);
+  if (rc) return rc;
+  for (uint64_t i = 0; i < n; i++) {
+    int64_t slot = is_reserved(t, keys[i]) ? -1 : lookup_slot(t, keys[i]);
+    slots[i] = slot >= 0 ? (uint64_t)slot : UINT64_MAX;
+    if (success) success[i] = slot >= 0;
+    if (slot < 0) continue;
+    t->keys[slot] = t->locked_key;
+    touch_score(t, (uint64_t)slot, scores, i);
+  }
+  advance_clock(t);
+  return HKV_SUCCESS;
+}
+
+/* unlock_keys (merlin_hashtable.cuh:2026-2044, unlock_keys_kernel,
+ * core_kernels.cuh:1180-1204) */
+int hkvo_unlock_keys(hkvo_table* t, uint64_t n, const uint64_t* slots,
+                     const uint64_t* keys, uint8_t* success) {
+  for (uint64_t i = 0; i < n; i++) {
+    int ok = slots[i] != UINT64_MAX && t->keys[slots[i]] == t->locked_key;
+    if (ok) t->keys[slots[i]] = keys[i];
+    if (success) success[i] = (uint8_t)ok;
+  }
+  return HKV_SUCCESS;
+}
+
+/* find_and_update (merlin_hashtable.cuh:2811-2843,
+ * tlp_lookup_ptr_kernel_with_filter with update_score = true,
+ * lookup_ptr.cuh:25-150): find* that also touches the score of every key it
+ * finds; scores[i] returns the score after the touch. */
+int hkvo_find_and_update(hkvo_table* t, uint64_t n, const uint64_t* keys,
+                         uint64_t* slots, uint8_t* founds, uint64_t* scores) {
+  if (n == 0) return HKV_SUCCESS;
+  int rc = check_scores_arg(t, t->strategy, scores);
+  if (rc) return rc;
+  for (uint64_t i = 0; i < n; i++) {
+    int64_t slot = is_reserved(t, keys[i]) ? -1 : lookup_slot(t, keys[i]);
+    if (founds) founds[i] = slot >= 0;
+    slots[i] = slot >= 0 ? (uint64_t)slot : UINT64_MAX;
+    if (slot < 0) continue;
+    touch_score(t, (uint64_t)slot, scores, i);
+    if (scores) scores[i] = t->scores[slot];
+  }
+  advance_clock(t);
   return HKV_SUCCESS;
 }
 

@@ -83,6 +83,14 @@ int hkvo_find_slot(const hkvo_table* t, uint64_t n, const uint64_t* keys,
                    uint64_t* slots, uint8_t* founds, uint64_t* scores);
 int hkvo_contains(const hkvo_table* t, uint64_t n, const uint64_t* keys,
                   uint8_t* founds);
+/* lock_keys / unlock_keys / find_and_update (merlin_hashtable.cuh:1982-2044,
+ * 2811-2843); slot indices stand for the addresses the reference returns */
+int hkvo_lock_keys(hkvo_table* t, uint64_t n, const uint64_t* keys, uint64_t* slots,
+                   uint8_t* success, const uint64_t* scores);
+int hkvo_unlock_keys(hkvo_table* t, uint64_t n, const uint64_t* slots,
+                     const uint64_t* keys, uint8_t* success);
+int hkvo_find_and_update(hkvo_table* t, uint64_t n, const uint64_t* keys,
+                         uint64_t* slots, uint8_t* founds, uint64_t* scores);
 int hkvo_erase(hkvo_table* t, uint64_t n, const uint64_t* keys);
 /* reserve + rehash (merlin_hashtable.cuh:3503-3541).  Every inserting call
  * above also runs the reference's growth loop first (fast_load_factor >

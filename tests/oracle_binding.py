@@ -42,6 +42,9 @@ _SIG = {
     "hkvo_find": (_i, [_p, _u64, _p, _p, _p, _p]),
     "hkvo_find_slot": (_i, [_p, _u64, _p, _p, _p, _p]),
     "hkvo_contains": (_i, [_p, _u64, _p, _p]),
+    "hkvo_lock_keys": (_i, [_p, _u64, _p, _p, _p, _p]),
+    "hkvo_unlock_keys": (_i, [_p, _u64, _p, _p, _p]),
+    "hkvo_find_and_update": (_i, [_p, _u64, _p, _p, _p, _p]),
     "hkvo_erase": (_i, [_p, _u64, _p]),
     "hkvo_clear": (_i, [_p]),
     "hkvo_reserve": (_i, [_p, _u64]),
@@ -189,6 +192,27 @@ class OracleTable:
         scores = np.zeros(n, np.uint64)
         _check(_lib.hkvo_find_slot(self._h, n, _np(keys), _np(slots), _np(founds), _np(scores)))
         return slots, founds.astype(bool), scores
+
+    def lock_keys(self, keys, scores=None):
+        n = len(keys)
+        slots = np.zeros(n, np.uint64)
+        ok = np.zeros(n, np.uint8)
+        _check(_lib.hkvo_lock_keys(self._h, n, _np(keys), _np(slots), _np(ok), _np(scores)))
+        return slots, ok.astype(bool)
+
+    def unlock_keys(self, slots, keys):
+        ok = np.zeros(len(keys), np.uint8)
+        _check(_lib.hkvo_unlock_keys(self._h, len(keys), _np(slots), _np(keys), _np(ok)))
+        return ok.astype(bool)
+
+    def find_and_update(self, keys, scores=None):
+        """scores: in/out array or None; returns (slots, founds, scores)."""
+        n = len(keys)
+        slots = np.zeros(n, np.uint64)
+        founds = np.zeros(n, np.uint8)
+        sc = None if scores is None else np.ascontiguousarray(scores).copy()
+        _check(_lib.hkvo_find_and_update(self._h, n, _np(keys), _np(slots), _np(founds), _np(sc)))
+        return slots, founds.astype(bool), sc
 
     def contains(self, keys):
         founds = np.zeros(len(keys), np.uint8)

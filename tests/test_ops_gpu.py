@@ -424,3 +424,62 @@ def test_growth_reserve_and_rehash(oracle):
     o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1))
     assert_same_table(t, o, dim * 4)
     t.close()
+
+
+def test_lock_keys_unlock_keys_find_and_update(oracle):
+    # merlin_hashtable.cuh:1982-2044, 2811-2843
+    cap, dim, bs = 1 << 13, 8, 6000
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    keys = w.unique_keys(91, 0, bs)
+    vals = w.values_from_keys(keys, dim)
+    sc = w.monotone_scores(1, bs)
+    t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+    o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1), sc)
+    n = 1500
+    batch = np.concatenate([keys[:1200], w.unique_keys(92, 0, n - 1200)])
+    new_sc = w.monotone_scores(2, n)
+    ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    ok = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.lock_keys(n, dev(batch), ptrs, ok, scores=dev(new_sc))
+    oslots, ook = o.lock_keys(batch, new_sc)
+    assert (ok.cpu().numpy() == ook).all() and ook[:1200].all() and not ook[1200:].any()
+    assert bool(((ptrs != 0) == ok).all())
+    founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.contains(bs, dev(keys), founds)
+    assert (founds.cpu().numpy() == o.contains(keys)).all() and not bool(founds[:1200].any())
+    assert t.size() == o.size()
+    # inserting while keys are locked: locked slots are never victims
+    more = w.unique_keys(93, 0, 4000)
+    mv = w.values_from_keys(more, dim)
+    ms = w.monotone_scores(3, 4000)
+    t.insert_or_assign(4000, dev(more), dev(mv), dev(ms))
+    o.insert_or_assign(more, mv.view(np.uint8).reshape(4000, -1), ms)
+    assert t.size() == o.size()
+    ok2 = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.unlock_keys(n, ptrs, dev(batch), ok2)
+    assert (ok2.cpu().numpy() == o.unlock_keys(oslots, batch)).all()
+    t.unlock_keys(n, ptrs, dev(batch), ok2)
+    assert not bool(ok2.any())
+    assert_same_table(t, o, dim * 4)
+    t.close()
+    # find_and_update under LFU: rows through the returned addresses, scores after the touch
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, evict_strategy=EvictStrategy.kLfu)
+    cnt = (np.arange(bs, dtype=np.uint64) % 7) + 1
+    t.insert_or_assign(bs, dev(keys), dev(vals), dev(cnt))
+    o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1), cnt)
+    add = (np.arange(n, dtype=np.uint64) % 5) + 1
+    dsc = dev(add.copy())
+    vp = torch.zeros(n, dtype=torch.int64, device=DEV)
+    fd = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.find_and_update(n, dev(batch), vp, fd, dsc)
+    oslots, of, osc = o.find_and_update(batch, add)
+    assert (fd.cpu().numpy() == of).all() and of[:1200].all() and not of[1200:].any()
+    assert (host_u64(dsc) == osc).all()
+    vpn = vp.cpu().numpy()
+    assert (vpn[1200:] == 0).all()
+    for i in (0, 7, 1199):
+        row = read_device(int(vpn[i]), dim * 4)
+        assert (row == vals[i].view(np.uint8)).all()
+    assert_same_table(t, o, dim * 4)
+    t.close()

@@ -606,3 +606,68 @@ def test_reserve_keeps_the_map_and_doubles_until_the_limit(oracle):
     assert not f[:50].any()
     assert f.tolist() == [k_ in before for k_ in keys.tolist()]  # (a few were evicted at 1024 slots)
     t.close()
+
+
+# ---- lock_keys / unlock_keys / find_and_update ---------------------------------------
+
+def test_lock_unlock_truth_table(oracle):
+    # lock_kernel_with_filter / unlock_keys_kernel (core_kernels.cuh:1180-1204, 1248-1362):
+    # present -> LOCKED + score touched + address; absent or reserved -> null, false;
+    # unlock succeeds exactly once per locked address
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(21, 0, 300)
+    t.insert_or_assign(keys, vals_of(keys, 2), np.arange(1000, 1300, dtype=np.uint64))
+    assert t.size() == 300
+    batch = np.concatenate([keys[:60], w.unique_keys(22, 0, 10), np.array([M64, M64 - 2], np.uint64)])
+    new_sc = np.arange(5000, 5000 + len(batch), dtype=np.uint64)
+    slots, ok = t.lock_keys(batch, new_sc)
+    assert ok.tolist() == [True] * 60 + [False] * 12
+    assert (slots[60:] == np.uint64(M64)).all() and len(set(slots[:60].tolist())) == 60
+    _, f, _ = t.find(keys)
+    assert not f[:60].any() and f[60:].all()        # a locked key is invisible to lookups
+    assert t.size() == 300                          # ... but still counted
+    assert len(t.export_all()[0]) == 240            # ... and not exported (its key word is reserved)
+    again, ok2 = t.lock_keys(batch[:5], new_sc[:5])
+    assert not ok2.any()                            # cannot be found, so cannot be locked twice
+    ok3 = t.unlock_keys(slots, batch)
+    assert ok3.tolist() == [True] * 60 + [False] * 12
+    assert not t.unlock_keys(slots[:60], batch[:60]).any()
+    v, f, sc = t.find(keys)
+    assert f.all() and (v == vals_of(keys, 2)).all()
+    assert (sc[:60] == new_sc[:60]).all() and (sc[60:] == np.arange(1060, 1300, dtype=np.uint64)).all()
+    t.close()
+
+
+def test_locked_slot_is_never_the_victim(oracle):
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(23, 0, 128)
+    sc = np.arange(100, 228, dtype=np.uint64)
+    t.insert_or_assign(keys, vals_of(keys, 1), sc)
+    slots, ok = t.lock_keys(keys[:1], np.array([100], np.uint64))  # the minimum-score key
+    assert ok.all()
+    newk = w.unique_keys(24, 0, 1)
+    t.insert_or_assign(newk, vals_of(newk, 1), np.array([500], np.uint64))
+    assert t.unlock_keys(slots, keys[:1]).all()
+    _, f, s2 = t.find(np.concatenate([keys[:2], newk]))
+    assert f.tolist() == [True, False, True]        # the second lowest score went instead
+    t.close()
+
+
+def test_find_and_update_touches_scores(oracle):
+    # tlp_lookup_ptr_kernel_with_filter, update_score = true (lookup_ptr.cuh:93-110)
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kLfu)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(25, 0, 200)
+    t.insert_or_assign(keys, vals_of(keys, 2), np.full(200, 3, np.uint64))
+    q = np.concatenate([keys[:50], w.unique_keys(26, 0, 5)])
+    slots, f, sc = t.find_and_update(q, np.full(55, 4, np.uint64))
+    assert f.tolist() == [True] * 50 + [False] * 5
+    assert (sc[:50] == 7).all() and (sc[50:] == 4).all()  # LFU adds; misses keep their input
+    assert (slots[50:] == np.uint64(M64)).all()
+    _, _, s2 = t.find(keys)
+    assert (s2[:50] == 7).all() and (s2[50:] == 3).all()
+    with pytest.raises(Exception):
+        t.find_and_update(q, None)  # LFU needs scores (check_evict_strategy)
+    t.close()
