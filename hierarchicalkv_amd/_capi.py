@@ -101,6 +101,7 @@ SIGNATURES = {
     "hkv_unlock_keys": (_i, [_T, _u64, _p, _p, _p, _p]),
     "hkv_find_and_update": (_i, [_T, _u64, _p, _p, _p, _p, _p]),
     "hkv_reserve": (_i, [_T, C.c_uint64, _p]),
+    "hkv_set_max_capacity": (_i, [_T, C.c_uint64]),
     "hkv_export_batch": (_i, [_T, _u64, _u64, _p, _p, _p, _p, _p]),
     "hkv_export_batch_if": (_i, [_T, _i, _u64, _u64, _u64, _u64, _p, _p, _p, _p, _p]),
     "hkv_size_if": (_i, [_T, _i, _u64, _u64, _p, C.POINTER(_u64)]),

@@ -1119,6 +1119,15 @@ int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream) {
   return reserve_impl(t, new_capacity, (hipStream_t)stream);
 }
 
+int hkv_set_max_capacity(hkv_table* t, uint64_t new_max_capacity) {
+  if (!ispow2(new_max_capacity))
+    return fail(HKV_ERROR_ARGUMENT, "None power-of-2 new_max_capacity is not supported.");
+  if (new_max_capacity < t->view.capacity) return HKV_SUCCESS;
+  t->reach_max_capacity = false;
+  t->opts.max_capacity = new_max_capacity;
+  return HKV_SUCCESS;
+}
+
 int hkv_clear(hkv_table* t, hkv_stream_t stream) {
   t->keys_may_be_locked = false;
   hipStream_t s = (hipStream_t)stream;

@@ -187,6 +187,9 @@ class HashTable:
     def clear(self, stream=None):
         _check(lib.hkv_clear(self._h, _stream(stream)))
 
+    def set_max_capacity(self, new_max_capacity):
+        _check(lib.hkv_set_max_capacity(self._h, new_max_capacity))
+
     def reserve(self, new_capacity, stream=None):
         _check(lib.hkv_reserve(self._h, new_capacity, _stream(stream)))
 

@@ -253,6 +253,9 @@ int hkv_clear(hkv_table* t, hkv_stream_t stream);
  * themselves at the head of every inserting call, as the reference's do
  * (merlin_hashtable.cuh:1151-1154).  Synchronises the device. */
 int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream);
+/* HashTable::set_max_capacity, merlin_hashtable.cuh:3561-3579: a power of two;
+ * values below the current capacity are ignored; growth is possible again. */
+int hkv_set_max_capacity(hkv_table* t, uint64_t new_max_capacity);
 
 /* HashTable::export_batch (device counter), merlin_hashtable.cuh:3099-3147 */
 int hkv_export_batch(const hkv_table* t, uint64_t n, uint64_t offset,

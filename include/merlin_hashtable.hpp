@@ -712,9 +712,8 @@ class HashTable : public HashTableBase<K, V, S> {
   void set_max_capacity(size_type new_max_capacity) override {
     if (new_max_capacity == 0 || (new_max_capacity & (new_max_capacity - 1)) != 0)
       throw std::invalid_argument("None power-of-2 new_max_capacity is not supported.");
-    if (new_max_capacity > capacity())
-      throw std::runtime_error("growing the table (rehash) is not supported");
-    options_.max_capacity = new_max_capacity;
+    throw_on_error_(hkv_set_max_capacity(table_, new_max_capacity));
+    if (new_max_capacity >= capacity()) options_.max_capacity = new_max_capacity;
   }
 
   size_type dim() const noexcept override { return options_.dim; }

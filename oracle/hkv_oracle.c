@@ -572,6 +572,16 @@ int hkvo_reserve(hkvo_table* t, uint64_t new_capacity) {
   return HKV_SUCCESS;
 }
 
+/* set_max_capacity, merlin_hashtable.cuh:3561-3579 */
+int hkvo_set_max_capacity(hkvo_table* t, uint64_t new_max_capacity) {
+  if (!ispow2_u64(new_max_capacity))
+    return fail(HKV_ERROR_ARGUMENT, "None power-of-2 new_max_capacity is not supported.");
+  if (new_max_capacity < t->capacity) return HKV_SUCCESS;
+  t->reach_max_capacity = 0;
+  t->opts.max_capacity = new_max_capacity;
+  return HKV_SUCCESS;
+}
+
 /* fast_load_factor, merlin_hashtable.cuh:3796-3830: sizes of the first
  * min(buckets, 1024) buckets, plus the incoming batch as if it were all new */
 static float fast_load_factor(const hkvo_table* t, uint64_t delta) {

@@ -96,6 +96,8 @@ int hkvo_erase(hkvo_table* t, uint64_t n, const uint64_t* keys);
  * above also runs the reference's growth loop first (fast_load_factor >
  * max_load_factor => reserve(2 * capacity), merlin_hashtable.cuh:1151-1154). */
 int hkvo_reserve(hkvo_table* t, uint64_t new_capacity);
+/* merlin_hashtable.cuh:3561-3579 */
+int hkvo_set_max_capacity(hkvo_table* t, uint64_t new_max_capacity);
 int hkvo_clear(hkvo_table* t);
 int hkvo_export_batch_if(const hkvo_table* t, int predicate, uint64_t pattern,
                          uint64_t threshold, uint64_t n, uint64_t offset,

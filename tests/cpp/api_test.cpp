@@ -446,6 +446,83 @@ static void test_option_checks() {
   t.insert_or_assign(0, nullptr, nullptr);  // n == 0 is a no-op
 }
 
+/* test_rehash, merlin_hashtable_test.cc.cu:1078-1200, and lock_keys / unlock_keys /
+ * find_and_update through the header */
+static void test_growth_and_key_locks() {
+  constexpr size_t DIM = 16, INIT = 128, MAX = 4 * INIT, N = 2 * INIT;
+  HashTableOptions o;
+  o.init_capacity = INIT;
+  o.max_capacity = MAX;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  using Table = HashTable<K, V, S, EvictStrategy::kCustomized>;
+  Table table;
+  table.init(o);
+  CHECK(table.capacity() == INIT);
+  /* 64 keys per bucket of the final 4-bucket table: nothing can be evicted */
+  std::vector<K> keys;
+  for (size_t b = 0; b < 4; b++) {
+    auto part = keys_in_bucket(N / 4, MAX, b, 0, 0x3FFFFFFFFFFFFFFF, 11 + b);
+    keys.insert(keys.end(), part.begin(), part.end());
+  }
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  for (size_t i = 0; i < N; i++) scores[i] = static_cast<S>(keys[i]);
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM), dout(N * DIM);
+  DevBuf<S> ds(N), dso(N);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p);  // grows to MAX before the first key goes in
+  CHECK(table.capacity() == MAX);
+  CHECK(table.size() == N);
+  table.reserve(MAX);
+  CHECK(table.capacity() == MAX && table.size() == N);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  auto f = df.down(N);
+  CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  CHECK(dout.down(N * DIM) == vals);
+  CHECK(dso.down(N) == scores);
+  table.set_max_capacity(2 * MAX);
+  table.reserve(2 * MAX);
+  CHECK(table.capacity() == 2 * MAX && table.size() == N);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  CHECK(dout.down(N * DIM) == vals);
+
+  /* lock the first half; locked keys are invisible until unlocked */
+  K** dptrs = nullptr;
+  HIP(hipMalloc(reinterpret_cast<void**>(&dptrs), N * sizeof(K*)));
+  table.lock_keys(N / 2, dk.p, dptrs, df.p, 0, ds.p);
+  HIP(hipDeviceSynchronize());
+  f = df.down(N / 2);
+  CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  table.contains(N, dk.p, df.p);
+  HIP(hipDeviceSynchronize());
+  f = df.down(N);
+  for (size_t i = 0; i < N; i++) CHECK((f[i] != 0) == (i >= N / 2));
+  table.unlock_keys(N / 2, dptrs, dk.p, df.p);
+  table.contains(N, dk.p, df.p);
+  HIP(hipDeviceSynchronize());
+  f = df.down(N);
+  CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  /* find_and_update: customized scores are replaced by the ones handed in */
+  std::vector<S> ns(N);
+  for (size_t i = 0; i < N; i++) ns[i] = scores[i] + 7;
+  ds.up(ns);
+  V** vptrs = nullptr;
+  HIP(hipMalloc(reinterpret_cast<void**>(&vptrs), N * sizeof(V*)));
+  table.find_and_update(N, dk.p, vptrs, df.p, ds.p);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  CHECK(dso.down(N) == ns);
+  (void)hipFree(dptrs);
+  (void)hipFree(vptrs);
+}
+
 int main() {
   try {
     test_basic();
@@ -453,6 +530,7 @@ int main() {
     test_insert_and_evict_and_predicates();
     test_allocator_hybrid_and_checkpoint();
     test_option_checks();
+    test_growth_and_key_locks();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;

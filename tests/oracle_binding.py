@@ -48,6 +48,7 @@ _SIG = {
     "hkvo_erase": (_i, [_p, _u64, _p]),
     "hkvo_clear": (_i, [_p]),
     "hkvo_reserve": (_i, [_p, _u64]),
+    "hkvo_set_max_capacity": (_i, [_p, _u64]),
     "hkvo_export_batch_if": (_i, [_p, _i, _u64, _u64, _u64, _u64, _p, _p, _p, _p]),
     "hkvo_size_if": (_u64, [_p, _i, _u64, _u64]),
     "hkvo_size": (_u64, [_p]),
@@ -227,6 +228,9 @@ class OracleTable:
 
     def reserve(self, new_capacity):
         _check(_lib.hkvo_reserve(self._h, new_capacity))
+
+    def set_max_capacity(self, new_max_capacity):
+        _check(_lib.hkvo_set_max_capacity(self._h, new_max_capacity))
 
     def export_batch_if(self, pred=0, pattern=0, threshold=0, n=None, offset=0):
         cap = self.capacity()
