@@ -369,11 +369,6 @@ __device__ __forceinline__ uint32_t xor2_u32(uint32_t x) {
 __device__ __forceinline__ uint32_t xor4_u32(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x101F); /* and 0x1f, or 0, xor 4 */
 }
-/* lane 0 of the tile to all its lanes */
-__device__ __forceinline__ uint32_t tile_first_u32(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x0018); /* and 0x18, or 0, xor 0 */
-}
-
 /* (score, slot) pairs order by score, then by slot: the reference's sequential
  * scan with a strict '<' keeps the lowest slot among equal scores
  * (upsert.cuh:166-183) */
@@ -660,14 +655,26 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       int emits = 0;
 #pragma unroll
       for (int q = 0; q < kGrpKeys; q++) emits += (got[q] == kStRefused || got[q] == kStEvict);
-      if (emits) {
-        uint32_t lo = 0, hi = 0;
-        if (j == 0) {
-          const unsigned long long b = atomicAdd(a.evicted_counter, (unsigned long long)emits);
-          lo = (uint32_t)b;
-          hi = (uint32_t)(b >> 32);
+      /* one counter update per wavefront and pass: the tiles that have something
+       * to emit right now add up their counts (an atomic per bucket on this one
+       * word would serialise the whole launch) */
+      const unsigned long long leaders = __ballot(j == 0 && emits > 0);
+      unsigned long long idx = 0;
+      if (leaders) {
+        int before = 0, total = 0;
+        for (unsigned long long m = leaders; m; m &= m - 1) {
+          const int l = (int)__ffsll(m) - 1;
+          const int e = __shfl(emits, l);
+          total += e;
+          if (l < tile_base) before += e;
         }
-        unsigned long long idx = tile_first_u32(lo) | ((unsigned long long)tile_first_u32(hi) << 32);
+        const int first_leader = (int)__ffsll(leaders) - 1;
+        unsigned long long base = 0;
+        if (lane == first_leader) base = atomicAdd(a.evicted_counter, (unsigned long long)total);
+        base = __shfl(base, first_leader);
+        idx = base + (unsigned long long)before;
+      }
+      if (emits) {
 #pragma unroll
         for (int q = 0; q < kGrpKeys; q++) {
           const bool refused_now = got[q] == kStRefused;
