@@ -15,8 +15,11 @@
 #ifndef HKV_DEVICE_HPP_
 #define HKV_DEVICE_HPP_
 
+#include <hip/hip_cooperative_groups.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "hkv_c_api.h"
 
@@ -173,6 +176,145 @@ erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshol
   }
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
   if (lane == 0 && local) atomicAdd(counter, (unsigned long long)local);
+}
+
+/*
+ * Tile type handed to the functor forms below.  It is HIP's
+ * cooperative_groups::thread_block_tile<N> plus shuffles of pointers, which
+ * functors written for the reference use (g.shfl(value, r) on a row pointer,
+ * tests/export_batch_if_test.cc.cu:117) and HIP's own tile does not take.
+ * Everything else of cooperative_groups is visible through this namespace, so
+ * it can stand behind a `cg` alias the way merlin/utils.cuh:30 sets one up.
+ */
+namespace coop {
+using namespace cooperative_groups;
+
+template <unsigned int N>
+class thread_block_tile : public cooperative_groups::thread_block_tile<N> {
+  using Base = cooperative_groups::thread_block_tile<N>;
+
+ public:
+  template <class Parent>
+  __device__ thread_block_tile(const cooperative_groups::thread_block_tile<N, Parent>& t)
+      : Base(t) {}
+
+  template <class T>
+  __device__ T shfl(T var, int src_rank) const {
+    if constexpr (std::is_pointer<T>::value)
+      return reinterpret_cast<T>(Base::shfl(reinterpret_cast<unsigned long long>(var), src_rank));
+    else
+      return Base::shfl(var, src_rank);
+  }
+  template <class T>
+  __device__ T shfl_down(T var, unsigned int delta) const {
+    if constexpr (std::is_pointer<T>::value)
+      return reinterpret_cast<T>(Base::shfl_down(reinterpret_cast<unsigned long long>(var), delta));
+    else
+      return Base::shfl_down(var, delta);
+  }
+  template <class T>
+  __device__ T shfl_up(T var, unsigned int delta) const {
+    if constexpr (std::is_pointer<T>::value)
+      return reinterpret_cast<T>(Base::shfl_up(reinterpret_cast<unsigned long long>(var), delta));
+    else
+      return Base::shfl_up(var, delta);
+  }
+  template <class T>
+  __device__ T shfl_xor(T var, unsigned int mask) const {
+    if constexpr (std::is_pointer<T>::value)
+      return reinterpret_cast<T>(Base::shfl_xor(reinterpret_cast<unsigned long long>(var), mask));
+    else
+      return Base::shfl_xor(var, mask);
+  }
+};
+}  // namespace coop
+
+/*
+ * The functor forms that see the value row and work in cooperative-groups
+ * tiles: f.template operator()<GroupSize>(key, value, score, tile).  The tile
+ * is hkv::coop::thread_block_tile<GroupSize>; the caller picks
+ * GroupSize so that the slot count is a multiple of it (all threads of a tile
+ * take the same number of trips).  K, V, S are the caller's types over the
+ * table's 64-bit key / score words and value bytes.
+ *
+ * traverse_kernel, core_kernels.cuh:1153-1178 (for_each)
+ */
+template <class K, class V, class S, class Func, unsigned GroupSize>
+__global__ void __launch_bounds__(128)
+traverse_kernel(hkv_table_view v, uint64_t n, uint64_t offset, Func f) {
+  coop::thread_block_tile<GroupSize> g(coop::tiled_partition<GroupSize>(coop::this_thread_block()));
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint64_t slot = i + offset;
+    const K key = static_cast<K>(v.keys[slot]);
+    S* score = reinterpret_cast<S*>(v.scores + slot);
+    V* value = reinterpret_cast<V*>(value_row(v, slot));
+    f.template operator()<GroupSize>(key, value, score, g);
+  }
+}
+
+/* dump_kernel with a functor, core_kernels.cuh:1043-1112 (export_batch_if_v2):
+ * the functor alone decides, reserved keys included */
+template <class K, class V, class S, class Pred, unsigned GroupSize>
+__global__ void __launch_bounds__(128)
+export_if_v2_kernel(hkv_table_view v, uint64_t n, uint64_t offset, Pred pred,
+                    unsigned long long* counter, K* out_keys, V* out_values, S* out_scores) {
+  coop::thread_block_tile<GroupSize> g(coop::tiled_partition<GroupSize>(coop::this_thread_block()));
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  const uint32_t dim = v.value_bytes / sizeof(V);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint64_t slot = i + offset;
+    const K key = static_cast<K>(v.keys[slot]);
+    const S score = static_cast<S>(v.scores[slot]);
+    const V* value = reinterpret_cast<const V*>(value_row(v, slot));
+    const bool match = pred.template operator()<GroupSize>(key, value, score, g);
+    const unsigned long long vote = g.ballot(match);
+    const int cnt = __popcll(vote);
+    unsigned long long base = 0;
+    if (g.thread_rank() == 0 && cnt) base = atomicAdd(counter, (unsigned long long)cnt);
+    base = g.shfl(base, 0);
+    const int before = __popcll(vote & ((1ull << g.thread_rank()) - 1));
+    if (match) {
+      out_keys[base + before] = key;
+      if (out_scores) out_scores[base + before] = score;
+    }
+    for (unsigned r = 0; r < GroupSize; r++) {
+      if (!((vote >> r) & 1ull)) continue;
+      const int bias = __popcll(vote & ((1ull << r) - 1));
+      const uint64_t cur = (i / GroupSize) * GroupSize + r + offset;
+      const V* src = reinterpret_cast<const V*>(value_row(v, cur));
+      for (uint32_t d = g.thread_rank(); d < dim; d += GroupSize)
+        out_values[(base + bias) * dim + d] = src[d];
+    }
+  }
+}
+
+/* remove_kernel_v2, core_kernels.cuh:794-843 (erase_if_v2) */
+template <class K, class V, class S, class Pred, unsigned GroupSize>
+__global__ void __launch_bounds__(128)
+erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* counter) {
+  coop::thread_block_tile<GroupSize> g(coop::tiled_partition<GroupSize>(coop::this_thread_block()));
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t slot = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; slot < n; slot += stride) {
+    const uint64_t raw = v.keys[slot];
+    const K key = static_cast<K>(raw);
+    const S score = static_cast<S>(v.scores[slot]);
+    const V* value = reinterpret_cast<const V*>(value_row(v, slot));
+    bool match = pred.template operator()<GroupSize>(key, value, score, g);
+    if (is_reserved_key(v, raw)) match = false;
+    const unsigned long long vote = g.ballot(match);
+    const int cnt = __popcll(vote);
+    /* GroupSize divides 128, so the slots of a tile share a bucket */
+    if (g.thread_rank() == 0 && cnt) {
+      atomicAdd(counter, (unsigned long long)cnt);
+      atomicSub(v.sizes + (slot >> 7), cnt);
+    }
+    if (match) {
+      v.digests[slot] = v.reclaim_digest;
+      v.keys[slot] = v.reclaim_key;
+      v.scores[slot] = 0;
+    }
+  }
 }
 
 /* One-word clear as a kernel: callers may be capturing a graph, where memset

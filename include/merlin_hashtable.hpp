@@ -20,13 +20,13 @@
  *   exceptions, checks ... merlin/debug.hpp:27-72
  *   GB / MB / KB ......... merlin/utils.cuh:338-342
  *
- * Not provided (outside this build's scope, the call throws
- * std::runtime_error): the *_v2 predicate forms and
- * for_each, TableMode::kMemory, S = uint32_t.
+ * Not provided: TableMode::kMemory (dual bucket; init throws), S = uint32_t
+ * (static_assert).
  */
 #ifndef MERLIN_HASHTABLE_HPP_
 #define MERLIN_HASHTABLE_HPP_
 
+#include <hip/hip_cooperative_groups.h>
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -43,6 +43,10 @@
 
 #include "hkv_c_api.h"
 #include "hkv_device.hpp"
+
+/* as merlin/utils.cuh:30: caller functors name the tile type cg::thread_block_tile<N>;
+ * the namespace behind the alias is cooperative_groups plus pointer shuffles */
+namespace cg = hkv::coop;
 
 namespace nv {
 namespace merlin {
@@ -611,6 +615,99 @@ class HashTable : public HashTableBase<K, V, S> {
     HKV_HIP_CHECK(hipStreamSynchronize(stream));
     HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
     return static_cast<size_type>(h);
+  }
+
+  /* merlin_hashtable.cuh:3008-3052: pred.template operator()<GroupSize>(key, value, score, tile)
+   * decides; returns how many entries were erased.  Synchronises `stream`. */
+  template <typename PredFunctor>
+  size_type erase_if_v2(PredFunctor& pred, hipStream_t stream = 0) {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    unsigned long long* d_count = nullptr;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
+    hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
+                       d_count);
+    {
+      detail::RoleGuard g(table_, 2, stream);
+      const uint64_t n = v.capacity;
+      const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
+      const uint64_t dim = options_.dim;
+      if (dim >= 32 && n % 32 == 0)
+        hipLaunchKernelGGL((hkv::erase_if_v2_kernel<K, V, S, PredFunctor, 32>), dim3(blocks),
+                           dim3(128), 0, stream, v, n, pred, d_count);
+      else if (dim >= 16 && n % 16 == 0)
+        hipLaunchKernelGGL((hkv::erase_if_v2_kernel<K, V, S, PredFunctor, 16>), dim3(blocks),
+                           dim3(128), 0, stream, v, n, pred, d_count);
+      else if (dim >= 8 && n % 8 == 0)
+        hipLaunchKernelGGL((hkv::erase_if_v2_kernel<K, V, S, PredFunctor, 8>), dim3(blocks),
+                           dim3(128), 0, stream, v, n, pred, d_count);
+      else
+        hipLaunchKernelGGL((hkv::erase_if_v2_kernel<K, V, S, PredFunctor, 1>), dim3(blocks),
+                           dim3(128), 0, stream, v, n, pred, d_count);
+      HKV_HIP_CHECK(hipGetLastError());
+    }
+    unsigned long long h = 0;
+    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
+    HKV_HIP_CHECK(hipStreamSynchronize(stream));
+    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
+    return static_cast<size_type>(h);
+  }
+
+  /* merlin_hashtable.cuh:3307-3348 */
+  template <typename PredFunctor>
+  void export_batch_if_v2(PredFunctor& pred, size_type n, const size_type offset,
+                          size_type* d_counter, key_type* keys, value_type* values,
+                          score_type* scores = nullptr, hipStream_t stream = 0) const {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    detail::RoleGuard g(table_, 0, stream);
+    hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
+    if (offset >= v.capacity) return;
+    n = std::min<size_type>(v.capacity - offset, n);
+    if (n == 0) return;
+    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
+    const uint64_t dim = options_.dim;
+    auto* cnt = reinterpret_cast<unsigned long long*>(d_counter);
+    if (dim >= 32 && n % 32 == 0)
+      hipLaunchKernelGGL((hkv::export_if_v2_kernel<K, V, S, PredFunctor, 32>), dim3(blocks),
+                         dim3(128), 0, stream, v, n, offset, pred, cnt, keys, values, scores);
+    else if (dim >= 16 && n % 16 == 0)
+      hipLaunchKernelGGL((hkv::export_if_v2_kernel<K, V, S, PredFunctor, 16>), dim3(blocks),
+                         dim3(128), 0, stream, v, n, offset, pred, cnt, keys, values, scores);
+    else if (dim >= 8 && n % 8 == 0)
+      hipLaunchKernelGGL((hkv::export_if_v2_kernel<K, V, S, PredFunctor, 8>), dim3(blocks),
+                         dim3(128), 0, stream, v, n, offset, pred, cnt, keys, values, scores);
+    else
+      hipLaunchKernelGGL((hkv::export_if_v2_kernel<K, V, S, PredFunctor, 1>), dim3(blocks),
+                         dim3(128), 0, stream, v, n, offset, pred, cnt, keys, values, scores);
+    HKV_HIP_CHECK(hipGetLastError());
+  }
+
+  /* merlin_hashtable.cuh:3372-3412: f.template operator()<GroupSize>(key, value, score, tile)
+   * is applied to every slot of [first, last), reserved keys included */
+  template <typename ExecutionFunc>
+  void for_each(const size_type first, const size_type last, ExecutionFunc& f,
+                hipStream_t stream = 0) {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    if (first >= v.capacity || last > v.capacity || first >= last) return;
+    detail::RoleGuard g(table_, 2, stream);
+    const uint64_t n = last - first;
+    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
+    const uint64_t dim = options_.dim;
+    if (dim >= 32 && n % 32 == 0)
+      hipLaunchKernelGGL((hkv::traverse_kernel<K, V, S, ExecutionFunc, 32>), dim3(blocks), dim3(128),
+                         0, stream, v, n, first, f);
+    else if (dim >= 16 && n % 16 == 0)
+      hipLaunchKernelGGL((hkv::traverse_kernel<K, V, S, ExecutionFunc, 16>), dim3(blocks), dim3(128),
+                         0, stream, v, n, first, f);
+    else if (dim >= 8 && n % 8 == 0)
+      hipLaunchKernelGGL((hkv::traverse_kernel<K, V, S, ExecutionFunc, 8>), dim3(blocks), dim3(128),
+                         0, stream, v, n, first, f);
+    else
+      hipLaunchKernelGGL((hkv::traverse_kernel<K, V, S, ExecutionFunc, 1>), dim3(blocks), dim3(128),
+                         0, stream, v, n, first, f);
+    HKV_HIP_CHECK(hipGetLastError());
   }
 
   void clear(hipStream_t stream = 0) override { throw_on_error_(hkv_clear(table_, stream)); }

@@ -60,6 +60,70 @@ struct EraseIfPredFunctor {
   }
 };
 
+
+/* Functors of the tile-cooperative forms, shaped like the ones the reference's tests
+ * hand to erase_if_v2 / export_batch_if_v2 / for_each
+ * (tests/merlin_hashtable_test.cc.cu:49-97, tests/export_batch_if_test.cc.cu:34-124). */
+/* the tile-cooperative export and for_each forms see every slot, free ones included
+ * (core_kernels.cuh:1043-1112, 1153-1178): the functor tells them apart */
+template <class Kt>
+__forceinline__ __device__ bool live_key(const Kt& key) {
+  return static_cast<uint64_t>(key) < 0xFFFFFFFFFFFFFFFCull;
+}
+template <class Kt, class Vt, class St>
+struct ScoreBelowV2 {
+  St threshold;
+  template <int GroupSize>
+  __forceinline__ __device__ bool operator()(const Kt& key, const Vt* value, const St& score,
+                                             cg::thread_block_tile<GroupSize>& g) {
+    return live_key(key) && score < threshold;
+  }
+};
+/* also reads the whole value row, one row at a time by the whole tile */
+template <class Kt, class Vt, class St>
+struct ScoreBelowAndRowIntactV2 {
+  St threshold;
+  int dim;
+  template <int GroupSize>
+  __forceinline__ __device__ bool operator()(const Kt& key, const Vt* value, const St& score,
+                                             cg::thread_block_tile<GroupSize>& g) {
+    bool mine = live_key(key) && score < threshold;
+    for (int r = 0; r < static_cast<int>(g.size()); r++) {
+      const Vt* row = g.shfl(value, r);
+      const Kt k = g.shfl(key, r);
+      const bool candidate = g.shfl(mine, r);
+      if (!candidate) continue;
+      bool bad = false;
+      for (int j = g.thread_rank(); j < dim; j += g.size())
+        bad |= row[j] != static_cast<Vt>(static_cast<uint64_t>(k) * 0.00001);
+      if (g.ballot(bad) != 0 && static_cast<int>(g.thread_rank()) == r) mine = false;
+    }
+    return mine;
+  }
+};
+/* for_each body: scales every element of rows whose score is below the
+ * threshold, bumps their score by one and counts them */
+template <class Kt, class Vt, class St>
+struct BumpRowsBelow {
+  St threshold;
+  int dim;
+  Vt factor;
+  unsigned long long* counter;
+  template <int GroupSize>
+  __forceinline__ __device__ void operator()(const Kt& key, Vt* value, St* score,
+                                             cg::thread_block_tile<GroupSize>& g) {
+    const bool match = live_key(key) && *score < threshold;
+    const unsigned long long vote = g.ballot(match);
+    if (g.thread_rank() == 0 && vote) atomicAdd(counter, (unsigned long long)__popcll(vote));
+    if (match) *score += 1;
+    for (int r = 0; r < GroupSize; r++) {
+      if (!((vote >> r) & 1ull)) continue;
+      Vt* row = g.shfl(value, r);
+      for (int j = g.thread_rank(); j < dim; j += GroupSize) row[j] *= factor;
+    }
+  }
+};
+
 static std::vector<K> random_keys(size_t n, uint64_t seed) {
   std::mt19937_64 rng(seed);
   std::unordered_set<K> seen;
@@ -127,7 +191,7 @@ static void test_basic() {
   }
   // accum_or_assign: existing & flagged -> old + delta
   {
-    std::vector<V> delta(N * DIM, 0.5f);
+    std::vector<V> delta(vals);  // keys are 64-bit wide, so a small constant would vanish in fp32
     std::vector<char> flags(N, 1);
     DevBuf<V> dd(N * DIM);
     dd.up(delta);
@@ -138,7 +202,7 @@ static void test_basic() {
     HIP(hipStreamSynchronize(stream));
     auto out = dout.down(N * DIM);
     bool same = true;
-    for (size_t i = 0; i < N * DIM; i++) same &= out[i] == vals[i] + 0.5f;
+    for (size_t i = 0; i < N * DIM; i++) same &= out[i] == vals[i] * 2.0f;
     CHECK(same);
   }
   // contains, erase half, clear
@@ -166,7 +230,7 @@ static void test_basic() {
     CHECK(found == N / 2 && nulls == N / 2);
     V row[DIM];
     HIP(hipMemcpy(row, ptrs[N - 1], sizeof row, hipMemcpyDeviceToHost));
-    CHECK(row[3] == vals[(N - 1) * DIM + 3] + 0.5f);
+    CHECK(row[3] == vals[(N - 1) * DIM + 3] * 2.0f);
   }
   // export == what is resident
   {
@@ -523,6 +587,126 @@ static void test_growth_and_key_locks() {
   (void)hipFree(vptrs);
 }
 
+
+template <size_t DIM>
+static void run_functor_forms() {
+  constexpr size_t CAP = 1 << 14, N = 6000;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  using Table = HashTable<int64_t, V, S, EvictStrategy::kCustomized>;
+  Table table;
+  table.init(o);
+  auto keys = random_keys(N, 4242 + DIM);
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  for (size_t i = 0; i < N; i++) scores[i] = 1000 + i;
+  std::vector<int64_t> sk(keys.begin(), keys.end());
+  DevBuf<int64_t> dk(N);
+  DevBuf<V> dv(N * DIM);
+  DevBuf<S> ds(N);
+  dk.up(sk);
+  dv.up(vals);
+  ds.up(scores);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p);
+  CHECK(table.size() == N);
+  std::map<int64_t, size_t> at;
+  for (size_t i = 0; i < N; i++) at[sk[i]] = i;
+  const S threshold = 1000 + N / 3;
+
+  /* export_batch_if_v2: plain and row-reading predicates agree with the host's count,
+   * over the whole table and over two halves */
+  DevBuf<int64_t> xk(CAP);
+  DevBuf<V> xv(CAP * DIM);
+  DevBuf<S> xs(CAP);
+  DevBuf<size_t> dc(1);
+  auto check_export = [&](size_t got, size_t want) {
+    CHECK(got == want);
+    auto hk = xk.down(got);
+    auto hs = xs.down(got);
+    auto hv = xv.down(got * DIM);
+    std::set<int64_t> seen;
+    bool ok = true;
+    for (size_t i = 0; i < got; i++) {
+      auto it = at.find(hk[i]);
+      if (it == at.end() || hs[i] != scores[it->second] || hs[i] >= threshold) { ok = false; break; }
+      for (size_t d = 0; d < DIM; d++) ok &= hv[i * DIM + d] == vals[it->second * DIM + d];
+      seen.insert(hk[i]);
+    }
+    CHECK(ok);
+    CHECK(seen.size() == got);
+  };
+  ScoreBelowV2<int64_t, V, S> below{threshold};
+  table.template export_batch_if_v2<ScoreBelowV2<int64_t, V, S>>(below, CAP, 0, dc.p, xk.p, xv.p, xs.p);
+  HIP(hipDeviceSynchronize());
+  check_export(dc.down(1)[0], N / 3);
+  ScoreBelowAndRowIntactV2<int64_t, V, S> intact{threshold, static_cast<int>(DIM)};
+  table.template export_batch_if_v2<ScoreBelowAndRowIntactV2<int64_t, V, S>>(intact, CAP, 0, dc.p, xk.p, xv.p, xs.p);
+  HIP(hipDeviceSynchronize());
+  check_export(dc.down(1)[0], N / 3);
+  size_t halves = 0;
+  for (size_t off : {size_t(0), CAP / 2}) {
+    table.template export_batch_if_v2<ScoreBelowV2<int64_t, V, S>>(below, CAP / 2, off, dc.p, xk.p, xv.p, xs.p);
+    HIP(hipDeviceSynchronize());
+    halves += dc.down(1)[0];
+  }
+  CHECK(halves == N / 3);
+  table.template export_batch_if_v2<ScoreBelowV2<int64_t, V, S>>(below, CAP, CAP, dc.p, xk.p, xv.p, xs.p);
+  HIP(hipDeviceSynchronize());
+  CHECK(dc.down(1)[0] == 0);
+
+  /* for_each: rows below the threshold are doubled and get score +1, the others are untouched */
+  DevBuf<unsigned long long> cnt(1);
+  cnt.up({0ull});
+  BumpRowsBelow<int64_t, V, S> bump{threshold, static_cast<int>(DIM), 2.0f, cnt.p};
+  table.template for_each<BumpRowsBelow<int64_t, V, S>>(0, table.capacity(), bump);
+  HIP(hipDeviceSynchronize());
+  CHECK(cnt.down(1)[0] == N / 3);
+  DevBuf<V> dout(N * DIM);
+  DevBuf<bool> df(N);
+  DevBuf<S> dso(N);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  {
+    auto out = dout.down(N * DIM);
+    auto so = dso.down(N);
+    bool ok = true;
+    for (size_t i = 0; i < N; i++) {
+      const bool hit = scores[i] < threshold;
+      ok &= so[i] == scores[i] + (hit ? 1 : 0);
+      for (size_t d = 0; d < DIM; d++) ok &= out[i * DIM + d] == vals[i * DIM + d] * (hit ? 2.0f : 1.0f);
+    }
+    CHECK(ok);
+  }
+  /* the bumped rows no longer pass the row-reading predicate; the plain one sees the
+   * new scores (one key moved across the threshold) */
+  size_t erased = table.template erase_if_v2<ScoreBelowAndRowIntactV2<int64_t, V, S>>(intact);
+  CHECK(erased == 0);
+  CHECK(table.size() == N);
+  erased = table.template erase_if_v2<ScoreBelowV2<int64_t, V, S>>(below);
+  CHECK(erased == N / 3 - 1);
+  CHECK(table.size() == N - erased);
+  table.contains(N, dk.p, df.p);
+  HIP(hipDeviceSynchronize());
+  {
+    auto f = df.down(N);
+    bool ok = true;
+    for (size_t i = 0; i < N; i++) ok &= (f[i] != 0) == !(scores[i] + 1 < threshold);
+    CHECK(ok);
+  }
+  /* erased slots are reusable */
+  table.insert_or_assign(N, dk.p, dv.p, ds.p);
+  CHECK(table.size() == N);
+}
+
+static void test_functor_forms() {
+  run_functor_forms<64>();  // tiles of 32
+  run_functor_forms<16>();  // tiles of 16
+  run_functor_forms<8>();   // tiles of 8
+  run_functor_forms<3>();   // one thread per slot
+}
+
 int main() {
   try {
     test_basic();
@@ -531,6 +715,7 @@ int main() {
     test_allocator_hybrid_and_checkpoint();
     test_option_checks();
     test_growth_and_key_locks();
+    test_functor_forms();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
