@@ -65,7 +65,8 @@ class TableView(C.Structure):
         ("empty_digest", C.c_uint8),
         ("reclaim_digest", C.c_uint8),
         ("pow2_buckets", C.c_uint8),
-        ("pad_", C.c_uint8 * 5),
+        ("dual_bucket", C.c_uint8),
+        ("pad_", C.c_uint8 * 4),
     ]
 
 

@@ -58,6 +58,40 @@ __device__ __forceinline__ void locate(const View& v, uint64_t key,
   start = (uint32_t)(g & 127u) & ~3u;
 }
 
+/* ---- dual-bucket mode (TableMode::kMemory) ---------------------------------- */
+
+struct DualLoc {
+  uint32_t bkt[2];
+  uint32_t start[2];
+  uint32_t digest;
+};
+
+/* get_dual_bucket_indices (dual_bucket_utils.cuh:36-50), the start positions of
+ * dual_bucket_upsert.cuh:86-101 (word % capacity, then % 128, rounded down to
+ * 4: the capacity is a multiple of 128, so word % 128), digest = hash >> 56.
+ * The stored digest byte of a live key never equals the EMPTY marker, as in
+ * single-bucket mode (see locate()).  The host side guarantees
+ * buckets_num < 2^32. */
+__device__ __forceinline__ DualLoc locate_dual(const View& v, uint64_t key) {
+  const uint64_t h = fmix64(key);
+  const uint32_t lo = (uint32_t)h, hi = (uint32_t)(h >> 32);
+  const uint32_t nb = (uint32_t)v.buckets_num;
+  DualLoc d;
+  if (v.pow2_buckets) {
+    d.bkt[0] = lo & (nb - 1);
+    d.bkt[1] = hi & (nb - 1);
+  } else {
+    d.bkt[0] = lo % nb;
+    d.bkt[1] = hi % nb;
+  }
+  if (d.bkt[1] == d.bkt[0]) d.bkt[1] = d.bkt[1] + 1 == nb ? 0 : d.bkt[1] + 1;
+  d.start[0] = (lo & 127u) & ~3u;
+  d.start[1] = (hi & 127u) & ~3u;
+  d.digest = (uint32_t)(h >> 56);
+  if (d.digest == v.empty_digest) d.digest ^= 1u;
+  return d;
+}
+
 /* 0x80 in every byte of x that is zero, exactly (no borrow artefacts). */
 __device__ __forceinline__ uint32_t zero_bytes(uint32_t x) {
   const uint32_t t = (x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu;

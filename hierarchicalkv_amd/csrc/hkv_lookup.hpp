@@ -175,9 +175,37 @@ __device__ __forceinline__ uint64_t stage_keys(const View& v,
   return key;
 }
 
+/* First pass of a dual-bucket find (dual_bucket_lookup.cuh:25-140): the keys
+ * staged by stage_keys get their first bucket and the dual-mode digest. */
+__device__ __forceinline__ void restage_first_bucket(const View& v, KeyMeta* s_meta, int lane) {
+  KeyMeta m = s_meta[lane];
+  if (m.info & 0x100u) {
+    const DualLoc L = locate_dual(v, m.key);
+    m.bkt = L.bkt[0];
+    m.info = L.digest | 0x100u | (L.start[0] << 16);
+    s_meta[lane] = m;
+  }
+}
+/* Second pass of a dual-bucket find: the keys of the wavefront that b1 did not
+ * hold are staged again with their second bucket; the others are switched off. */
+__device__ __forceinline__ void restage_second_bucket(const View& v, KeyMeta* s_meta,
+                                                      const int64_t* s_slot, int lane) {
+  KeyMeta m = s_meta[lane];
+  const bool again = (m.info & 0x100u) && s_slot[lane] < 0;
+  if (again) {
+    const DualLoc L = locate_dual(v, m.key);
+    m.bkt = L.bkt[1];
+    m.info = L.digest | 0x100u | (L.start[1] << 16);
+  } else {
+    m.info &= ~0x100u;
+  }
+  s_meta[lane] = m;
+}
+
+
 enum LookupMode { kLookupValues = 0, kLookupPtr = 1, kLookupContains = 2 };
 
-template <int MODE, int VEC>
+template <int MODE, int VEC, bool DUAL = false>
 __global__ void __launch_bounds__(kWave)
 lookup_kernel(View v, FindArgs a) {
   __shared__ KeyMeta s_meta[kWave];
@@ -186,9 +214,16 @@ lookup_kernel(View v, FindArgs a) {
   const uint64_t base = (uint64_t)blockIdx.x * kWave;
   const uint64_t i = base + lane;
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
+  if (DUAL) restage_first_bucket(v, s_meta, lane);
   __syncthreads();
   probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
+  if (DUAL) {
+    restage_second_bucket(v, s_meta, s_slot, lane);
+    __syncthreads();
+    probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+    __syncthreads();
+  }
 
   const int64_t my_slot = s_slot[lane];
   if (i < a.n) {

@@ -23,6 +23,7 @@
 #include "hkv_c_api.h"
 #include "hkv_misc.hpp"
 #include "hkv_upsert.hpp"
+#include "hkv_dual.hpp"
 #include "hkv_grouped.hpp"
 #include "hkv_keylocks.hpp"
 
@@ -162,6 +163,7 @@ struct hkv_table {
   int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
   bool keys_may_be_locked; /* lock_keys has been called: LOCKED key words may sit in the table */
+  bool dual;               /* TableMode::kMemory: two candidate buckets per key */
 };
 
 namespace {
@@ -447,8 +449,11 @@ int alloc_arenas(hkv_table* t, uint64_t buckets_num, View& v, TableMem& m) {
   /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
    * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
   const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
+  /* a dual-bucket table must be created with max_hbm_for_vectors == 0 and is meant to be
+   * all-HBM (merlin_hashtable.cuh:1000-1002): its rows go to HBM */
   const uint64_t hbm_buckets =
-      std::min<uint64_t>(v.buckets_num, t->opts.max_hbm_for_vectors / bucket_bytes);
+      t->dual ? v.buckets_num
+              : std::min<uint64_t>(v.buckets_num, t->opts.max_hbm_for_vectors / bucket_bytes);
   v.hbm_slots = hbm_buckets * kBucketSize;
   v.values = nullptr;
   v.host_values = nullptr;
@@ -582,6 +587,37 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   return HKV_SUCCESS;
 }
 
+/* The calls that refuse a dual-bucket table with a MERLIN_CHECK
+ * (merlin_hashtable.cuh:1362, 1597, 1705, 1891, 2233, 2304, 2860, 2905, 3505) report
+ * HKV_ERROR_CHECK.  The calls the reference leaves unguarded although they probe one bucket
+ * only (assign, find*, the missed-keys find, lock_keys, unlock_keys, find_and_update) report
+ * HKV_ERROR_UNSUPPORTED instead of answering wrongly. */
+int refuse_dual(const hkv_table* t, const char* what, bool guarded) {
+  if (!t->dual) return HKV_SUCCESS;
+  return fail(guarded ? HKV_ERROR_CHECK : HKV_ERROR_UNSUPPORTED,
+              "[MEMORY_MODE] %s is not supported in dual-bucket mode.", what);
+}
+
+void launch_dual_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
+  const dim3 grid((unsigned)((a.n + kTilesPerWave - 1) / kTilesPerWave)), block(kWave);
+  if (vec == 16)
+    hipLaunchKernelGGL((dual_upsert_kernel<16>), grid, block, 0, s, v, a);
+  else if (vec == 4)
+    hipLaunchKernelGGL((dual_upsert_kernel<4>), grid, block, 0, s, v, a);
+  else
+    hipLaunchKernelGGL((dual_upsert_kernel<1>), grid, block, 0, s, v, a);
+}
+
+void launch_dual_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
+  const dim3 grid(grid_for(a.n)), block(kWave);
+  if (vec == 16)
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 16, true>), grid, block, 0, s, v, a);
+  else if (vec == 4)
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 4, true>), grid, block, 0, s, v, a);
+  else
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 1, true>), grid, block, 0, s, v, a);
+}
+
 template <int MODE>
 void launch_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
@@ -616,8 +652,27 @@ void launch_size_if(const hkv_table* t, uint64_t pattern, uint64_t threshold,
 int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) {
   if (!o || !out) return fail(HKV_ERROR_ARGUMENT, "null argument");
   /* HashTable::init, merlin_hashtable.cuh:1016-1048 */
-  if (o->table_mode != 0)
-    return fail(HKV_ERROR_UNSUPPORTED, "TableMode::kMemory (dual bucket) is not supported");
+  if (o->table_mode != 0 && o->table_mode != 1)
+    return fail(HKV_ERROR_ARGUMENT, "bad table_mode %d", o->table_mode);
+  if (o->table_mode == 1) {
+    /* merlin_hashtable.cuh:992-1014 */
+    if (o->init_capacity != o->max_capacity)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] init_capacity must equal max_capacity. "
+                  "Auto-rehash is not supported in dual-bucket mode.");
+    if (o->max_hbm_for_vectors != 0)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] Only pure HBM (fast mode) is supported. "
+                  "Set max_hbm_for_vectors = 0.");
+    if (o->dim * (uint64_t)o->value_size > 224 * sizeof(float))
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] dim * sizeof(V) must not exceed 896 bytes "
+                  "(i.e. dim <= 224 for float).");
+    if (o->max_bucket_size == 0 || o->init_capacity / o->max_bucket_size < 2)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] capacity must provide at least 2 buckets "
+                  "(capacity >= 2 * max_bucket_size).");
+  }
   if (o->reserved_key_start_bit < 0 || o->reserved_key_start_bit > 62)
     return fail(HKV_ERROR_CHECK, "options.reserved_key_start_bit should >= 0 and <= 62.");
   if (!ispow2(o->max_bucket_size))
@@ -661,6 +716,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->d_scratch = nullptr;
   t->scratch_bytes = 0;
   t->keys_may_be_locked = false;
+  t->dual = o->table_mode == 1;
   /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default while the
    * two-phase path is being tuned), "auto" = two-phase for large batches,
    * "grouped" = two-phase whenever it is possible (tests) */
@@ -729,6 +785,12 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   }
   v.empty_digest = (uint8_t)(fmix64(v.empty_key) >> 32);
   v.reclaim_digest = (uint8_t)(fmix64(v.reclaim_key) >> 32);
+  if (t->dual) {
+    /* dual_bucket_empty_digest, dual_bucket_utils.cuh:86-90; core_kernels.cuh:67-71 */
+    v.empty_digest = (uint8_t)(fmix64(v.empty_key) >> 56);
+    v.reclaim_digest = (uint8_t)(fmix64(v.reclaim_key) >> 56);
+  }
+  v.dual_bucket = t->dual ? 1 : 0;
 
   TableMem mem{};
   {
@@ -749,7 +811,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
     if (rc) return bail(rc);
   }
   t->d_counters = (unsigned long long*)cnt;
-  t->reach_max_capacity = o->init_capacity * 2 > o->max_capacity; /* merlin_hashtable.cuh:1064 */
+  t->reach_max_capacity = t->dual || o->init_capacity * 2 > o->max_capacity; /* merlin_hashtable.cuh:1064-1069 */
   *out = t;
   return HKV_SUCCESS;
 }
@@ -805,7 +867,6 @@ int hkv_table_destroy(hkv_table* t) {
 int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
                          const void* values, const uint64_t* scores,
                          hkv_stream_t stream, int unique_key, int ignore) {
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
   if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
@@ -816,6 +877,24 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.n = n;
   a.strategy = strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
+  if (t->dual) {
+    /* merlin_hashtable.cuh:1166-1190 */
+    if (!unique_key)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] insert_or_assign requires unique_key=true in dual-bucket mode.");
+    hipStream_t s = (hipStream_t)stream;
+    a.epoch = t->epoch;
+    a.clock = t->clock;
+    a.value_kind = t->opts.value_kind;
+    {
+      LockGuard g(t, StreamGroupLock::kInserter, s);
+      HKV_HIP(g.acquire());
+      launch_dual_upsert(vec, t->view, a, s);
+      HKV_HIP(hipGetLastError());
+    }
+    if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+    return HKV_SUCCESS;
+  }
   return run_upsert<kOpInsertOrAssign>(t, a, vec, true, (hipStream_t)stream);
 }
 
@@ -824,6 +903,7 @@ int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
                          uint64_t* evicted_keys, void* evicted_values,
                          uint64_t* evicted_scores, uint64_t* d_evicted_counter,
                          hkv_stream_t stream, int unique_key, int ignore) {
+  HKV_TRY(refuse_dual(t, "insert_and_evict()", true));
   if (n == 0) return HKV_SUCCESS;
   /* merlin_hashtable.cuh:1384-1386 */
   if (!t->pure_hbm)
@@ -851,6 +931,7 @@ int hkv_insert_and_evict_count(hkv_table* t, uint64_t n, const uint64_t* keys,
                                uint64_t* evicted_keys, void* evicted_values,
                                uint64_t* evicted_scores, hkv_stream_t stream,
                                int unique_key, int ignore, uint64_t* n_evicted) {
+  HKV_TRY(refuse_dual(t, "insert_and_evict()", true));
   *n_evicted = 0;
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
@@ -865,6 +946,7 @@ int hkv_insert_and_evict_count(hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_accum_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
                         const void* value_or_deltas, const uint8_t* flags,
                         const uint64_t* scores, hkv_stream_t stream, int ignore) {
+  HKV_TRY(refuse_dual(t, "accum_or_assign()", true));
   if (n == 0) return HKV_SUCCESS;
   if (t->opts.value_kind == HKV_VALUE_BYTES)
     return fail(HKV_ERROR_ARGUMENT, "accum_or_assign needs an arithmetic value_kind");
@@ -884,6 +966,7 @@ int hkv_accum_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
                        void* values, const uint64_t* scores, hkv_stream_t stream,
                        int unique_key, int ignore) {
+  HKV_TRY(refuse_dual(t, "find_or_insert()", true));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
@@ -901,6 +984,7 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
                            void** values, uint8_t* founds, const uint64_t* scores,
                            hkv_stream_t stream, int unique_key, int ignore) {
+  HKV_TRY(refuse_dual(t, "find_or_insert()", true));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
@@ -952,6 +1036,7 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
 
 int hkv_assign(hkv_table* t, uint64_t n, const uint64_t* keys, const void* values,
                const uint64_t* scores, hkv_stream_t stream, int unique_key) {
+  HKV_TRY(refuse_dual(t, "assign()", false));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
@@ -960,6 +1045,7 @@ int hkv_assign(hkv_table* t, uint64_t n, const uint64_t* keys, const void* value
 
 int hkv_assign_scores(hkv_table* t, uint64_t n, const uint64_t* keys,
                       const uint64_t* scores, hkv_stream_t stream, int unique_key) {
+  HKV_TRY(refuse_dual(t, "assign_scores()", true));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
@@ -968,6 +1054,7 @@ int hkv_assign_scores(hkv_table* t, uint64_t n, const uint64_t* keys,
 
 int hkv_assign_values(hkv_table* t, uint64_t n, const uint64_t* keys,
                       const void* values, hkv_stream_t stream, int unique_key) {
+  HKV_TRY(refuse_dual(t, "assign_values()", true));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   return assign_common(t, n, keys, values, nullptr, 0, (hipStream_t)stream);
@@ -986,7 +1073,10 @@ int hkv_find(const hkv_table* t, uint64_t n, const uint64_t* keys, void* values,
   const int vec = pick_vec(t->view.value_bytes, {values});
   LockGuard g(t, StreamGroupLock::kReader, s);
   HKV_HIP(g.acquire());
-  launch_lookup<kLookupValues>(vec, t->view, a, s);
+  if (t->dual)
+    launch_dual_lookup(vec, t->view, a, s);
+  else
+    launch_lookup<kLookupValues>(vec, t->view, a, s);
   HKV_HIP(hipGetLastError());
   return HKV_SUCCESS;
 }
@@ -994,6 +1084,7 @@ int hkv_find(const hkv_table* t, uint64_t n, const uint64_t* keys, void* values,
 int hkv_find_missed(const hkv_table* t, uint64_t n, const uint64_t* keys,
                     void* values, uint64_t* missed_keys, int32_t* missed_indices,
                     int32_t* missed_size, uint64_t* scores, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "find() with the missed-keys outputs", false));
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
   FindArgs a{};
@@ -1016,6 +1107,7 @@ int hkv_find_missed(const hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_find_ptr(const hkv_table* t, uint64_t n, const uint64_t* keys,
                  void** values, uint8_t* founds, uint64_t* scores,
                  hkv_stream_t stream, int unique_key) {
+  HKV_TRY(refuse_dual(t, "find() by pointer", false));
   (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
@@ -1034,6 +1126,7 @@ int hkv_find_ptr(const hkv_table* t, uint64_t n, const uint64_t* keys,
 
 int hkv_contains(const hkv_table* t, uint64_t n, const uint64_t* keys,
                  uint8_t* founds, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "contains()", true));
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
   FindArgs a{};
@@ -1049,6 +1142,7 @@ int hkv_contains(const hkv_table* t, uint64_t n, const uint64_t* keys,
 
 int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys, uint64_t** locked_key_ptrs,
                   uint8_t* success, const uint64_t* scores, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "lock_keys()", false));
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
   hipStream_t s = (hipStream_t)stream;
@@ -1074,6 +1168,7 @@ int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys, uint64_t** loc
 
 int hkv_unlock_keys(hkv_table* t, uint64_t n, uint64_t** locked_key_ptrs, const uint64_t* keys,
                     uint8_t* success, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "unlock_keys()", false));
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
   LockGuard g(t, StreamGroupLock::kInserter, s);
@@ -1086,6 +1181,7 @@ int hkv_unlock_keys(hkv_table* t, uint64_t n, uint64_t** locked_key_ptrs, const 
 
 int hkv_find_and_update(hkv_table* t, uint64_t n, const uint64_t* keys, void** values,
                         uint8_t* founds, uint64_t* scores, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "find_and_update()", false));
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
   hipStream_t s = (hipStream_t)stream;
@@ -1110,6 +1206,7 @@ int hkv_find_and_update(hkv_table* t, uint64_t n, const uint64_t* keys, void** v
 }
 
 int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "erase()", true));
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
   LockGuard g(t, StreamGroupLock::kInserter, s);
@@ -1120,6 +1217,7 @@ int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t strea
 }
 
 int hkv_reserve(hkv_table* t, uint64_t new_capacity, hkv_stream_t stream) {
+  HKV_TRY(refuse_dual(t, "reserve()", true));
   return reserve_impl(t, new_capacity, (hipStream_t)stream);
 }
 

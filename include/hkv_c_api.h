@@ -92,7 +92,7 @@ typedef struct hkv_options {
   int32_t reserved_key_start_bit;
   uint64_t num_of_buckets_per_alloc;
   int32_t api_lock;
-  int32_t table_mode; /* 0 = kThroughput (only mode supported) */
+  int32_t table_mode; /* 0 = kThroughput, 1 = kMemory (dual bucket; insert_or_assign and find only) */
   /* template parameters of HashTable<K,V,S,Strategy> */
   int32_t evict_strategy; /* hkv_evict_strategy */
   int32_t value_kind;     /* hkv_value_kind */
@@ -119,7 +119,8 @@ typedef struct hkv_table_view {
   uint64_t reserved_mask1, reserved_mask2; /* reserved <=> (k & mask1) == mask2 */
   uint8_t empty_digest, reclaim_digest;
   uint8_t pow2_buckets; /* buckets_num is a power of two */
-  uint8_t pad_[5];
+  uint8_t dual_bucket;  /* TableMode::kMemory: a key lives in one of two buckets */
+  uint8_t pad_[4];
 } hkv_table_view;
 
 /* BaseAllocator (include/merlin/allocator.cuh:27-58) as a table of callbacks.

@@ -20,8 +20,11 @@
  *   exceptions, checks ... merlin/debug.hpp:27-72
  *   GB / MB / KB ......... merlin/utils.cuh:338-342
  *
- * Not provided: TableMode::kMemory (dual bucket; init throws), S = uint32_t
- * (static_assert).
+ * TableMode::kMemory (dual bucket) runs insert_or_assign, find, clear, size and
+ * the export family, as in the reference; the calls the reference guards throw
+ * the same way, and assign, find*, lock_keys / unlock_keys / find_and_update
+ * (unguarded but single-bucket in the reference) throw too.
+ * Not provided: S = uint32_t (static_assert).
  */
 #ifndef MERLIN_HASHTABLE_HPP_
 #define MERLIN_HASHTABLE_HPP_
@@ -212,7 +215,7 @@ struct EvictStrategy {
 
 enum class TableMode {
   kThroughput = 0,  ///< Default: single-bucket, max throughput.
-  kMemory = 1,      ///< Dual-bucket, higher load factor (not supported here).
+  kMemory = 1,      ///< Dual-bucket, higher load factor.
 };
 
 /* memory_pool.cuh:139-143; kept so option structs copy over unchanged.  The

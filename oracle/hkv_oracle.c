@@ -23,6 +23,12 @@
  *   bucket count ........ include/merlin/core_kernels.cuh:349-357
  *   argument checks ..... include/merlin_hashtable.cuh:1016-1048, 3832-3861
  *   hybrid refusal rule . include/merlin/core_kernels/upsert.cuh:1524
+ *   dual-bucket mode .... include/merlin/core_kernels/dual_bucket_utils.cuh:36-101
+ *                         (addressing, digest), dual_bucket_upsert.cuh:139-600
+ *                         (insert_or_assign), dual_bucket_lookup.cuh:25-140
+ *                         (find: first bucket, then second),
+ *                         include/merlin_hashtable.cuh:992-1014 (init checks) and
+ *                         the `!is_memory_mode()` guards of the other calls
  *
  * The reference itself cannot be built or run here (CUDA only), and its tests
  * hold no golden vectors (inputs are unseeded).  What pins this file instead
@@ -40,7 +46,14 @@
  *     tests/test_util.cuh:371-376;
  *   - accum_or_assign: tests/accum_or_assign_test.cc.cu:2818-2845;
  *   - export_batch_if / size_if: tests/export_batch_if_test.cc.cu:268-296;
- *   - erase / clear counts: tests/merlin_hashtable_test.cc.cu:336-344.
+ *   - erase / clear counts: tests/merlin_hashtable_test.cc.cu:336-344;
+ *   - dual-bucket mode: closed form of the two bucket indices, the
+ *     b1 == b2 case of tests/dual_bucket_test.cc.cu:663-742, first eviction
+ *     above load factor 0.98 (:399-465), eviction quality >= 0.995 (:1406-1520),
+ *     the guards and init checks (:471-515, 941-1107), clear and re-insert
+ *     (:1841-1900).  In this mode a batch is not order-independent (where a
+ *     key lands depends on the bucket sizes at that moment); the oracle applies
+ *     the batch in input order.
  * Parity unpinned (only an execution of the reference could pin them, and none
  * is observable under the tests' preconditions): victim choice among equal
  * scores, which EMPTY slot an insert takes, and real LRU clock values.
@@ -80,6 +93,7 @@ struct hkvo_table {
   int clock_mode;
   uint64_t clock_base;
   int reach_max_capacity; /* merlin_hashtable.cuh:1064 */
+  int dual;               /* TableMode::kMemory, merlin_hashtable.cuh:93-98 */
 };
 
 static __thread char g_err[512];
@@ -141,8 +155,36 @@ void hkvo_locate(uint64_t key, uint64_t buckets_num, uint64_t* bkt,
   *digest = (uint8_t)(h >> 32);
 }
 
+/* get_dual_bucket_indices, dual_bucket_utils.cuh:36-50; start positions as
+ * dual_bucket_upsert.cuh:86-101 (the low and the high hash word, each modulo
+ * the capacity, then modulo 128 and rounded down to 4); digest = hash bits
+ * 56..63, dual_bucket_utils.cuh:70-74 */
+void hkvo_locate_dual(uint64_t key, uint64_t buckets_num, uint64_t bkt[2],
+                      uint32_t start[2], uint8_t* digest) {
+  uint64_t h = hkvo_murmur3_fmix64(key);
+  uint32_t lo = (uint32_t)h, hi = (uint32_t)(h >> 32);
+  bkt[0] = lo % buckets_num;
+  bkt[1] = hi % buckets_num;
+  if (bkt[1] == bkt[0]) bkt[1] = (bkt[1] + 1) % buckets_num;
+  uint32_t s0 = (uint32_t)((lo % (buckets_num * BUCKET)) % BUCKET);
+  uint32_t s1 = (uint32_t)((hi % (buckets_num * BUCKET)) % BUCKET);
+  start[0] = s0 - (s0 % 4);
+  start[1] = s1 - (s1 % 4);
+  *digest = (uint8_t)(h >> 56);
+}
+
 static inline int is_reserved(const hkvo_table* t, uint64_t k) {
   return (k & t->rmask1) == t->rmask2;
+}
+
+/* the calls that refuse a dual-bucket table, merlin_hashtable.cuh:1362, 1597,
+ * 1705, 1891, 2233, 2304, 2860, 2905, 3505 (MERLIN_CHECK(!is_memory_mode())).
+ * The calls the reference leaves unguarded although they probe one bucket
+ * only (assign, find*, lock_keys, find_and_update) are refused here as well. */
+static int refuse_dual(const hkvo_table* t, const char* what, int guarded) {
+  if (!t->dual) return HKV_SUCCESS;
+  return fail(guarded ? HKV_ERROR_CHECK : HKV_ERROR_UNSUPPORTED,
+              "[MEMORY_MODE] %s is not supported in dual-bucket mode.", what);
 }
 
 int hkvo_online_cores(void) {
@@ -179,9 +221,30 @@ int hkvo_create(const hkv_options* o, int hybrid_refusal, hkvo_table** out) {
   if (o->dim == 0 || o->value_size == 0)
     return fail(HKV_ERROR_ARGUMENT, "dim and value_size must be positive");
 
+  if (o->table_mode != 0 && o->table_mode != 1)
+    return fail(HKV_ERROR_ARGUMENT, "bad table_mode");
+  if (o->table_mode == 1) {
+    /* merlin_hashtable.cuh:992-1014 */
+    if (o->init_capacity != o->max_capacity)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] init_capacity must equal max_capacity. "
+                  "Auto-rehash is not supported in dual-bucket mode.");
+    if (o->max_hbm_for_vectors != 0)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] Only pure HBM (fast mode) is supported. "
+                  "Set max_hbm_for_vectors = 0.");
+    if (o->dim * o->value_size > 224 * 4)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] dim * sizeof(V) must not exceed 896 bytes");
+    if (o->init_capacity / o->max_bucket_size < 2)
+      return fail(HKV_ERROR_CHECK,
+                  "[MEMORY_MODE] capacity must provide at least 2 buckets");
+  }
+
   hkvo_table* t = (hkvo_table*)calloc(1, sizeof *t);
   if (!t) return fail(HKV_ERROR_RUNTIME, "out of memory");
   t->opts = *o;
+  t->dual = o->table_mode == 1;
   t->strategy = o->evict_strategy;
   t->hybrid_refusal = hybrid_refusal;
   /* core_kernels.cuh:343-357 */
@@ -206,8 +269,13 @@ int hkvo_create(const hkv_options* o, int hybrid_refusal, hkvo_table** out) {
   t->vmask2 = rk[6];
   t->empty_digest = (uint8_t)(hkvo_murmur3_fmix64(t->empty_key) >> 32);
   t->reclaim_digest = (uint8_t)(hkvo_murmur3_fmix64(t->reclaim_key) >> 32);
+  if (t->dual) {
+    /* dual_bucket_empty_digest, dual_bucket_utils.cuh:86-90; core_kernels.cuh:67-71 */
+    t->empty_digest = (uint8_t)(hkvo_murmur3_fmix64(t->empty_key) >> 56);
+    t->reclaim_digest = (uint8_t)(hkvo_murmur3_fmix64(t->reclaim_key) >> 56);
+  }
   t->epoch = IGNORED_EPOCH;
-  t->reach_max_capacity = o->init_capacity * 2 > o->max_capacity;
+  t->reach_max_capacity = t->dual || o->init_capacity * 2 > o->max_capacity;
   t->digests = (uint8_t*)malloc(t->capacity);
   t->keys = (uint64_t*)malloc(t->capacity * 8);
   t->scores = (uint64_t*)calloc(t->capacity, 8);
@@ -384,6 +452,19 @@ static inline int64_t lookup_slot(const hkvo_table* t, uint64_t key) {
   uint64_t bkt;
   uint32_t start;
   uint8_t dg;
+  if (t->dual) {
+    /* dual_bucket_lookup.cuh:25-140: the first bucket, then the second */
+    uint64_t b[2];
+    uint32_t st[2];
+    hkvo_locate_dual(key, t->buckets_num, b, st, &dg);
+    for (int w = 0; w < 2; w++) {
+      const uint8_t* d = t->digests + b[w] * BUCKET;
+      const uint64_t* k = t->keys + b[w] * BUCKET;
+      for (uint32_t p = 0; p < BUCKET; p++)
+        if (d[p] == dg && k[p] == key) return (int64_t)(b[w] * BUCKET + p);
+    }
+    return -1;
+  }
   hkvo_locate(key, t->buckets_num, &bkt, &start, &dg);
   const uint8_t* d = t->digests + bkt * BUCKET;
   const uint64_t* k = t->keys + bkt * BUCKET;
@@ -481,6 +562,75 @@ static void decide(const hkvo_table* t, int strategy, uint64_t key,
   r->result = (r->victim == t->reclaim_key) ? OCC_RECLAIMED : OCC_EVICT;
 }
 
+/*
+ * The same decision in dual-bucket mode, dual_bucket_upsert.cuh:139-600:
+ *   0. the key is looked for in both buckets (first b1, then b2);
+ *   1. otherwise the bucket with fewer keys is tried first (b1 on a tie), then
+ *      the other: in a bucket that is not full the first EMPTY slot in
+ *      circular order from the bucket's own start position is taken;
+ *   2. otherwise the minimum score over both buckets decides: refuse when
+ *      desired < min; the victim is the minimum of b1 when min1 <= min2, else
+ *      of b2 (lowest slot on ties; the reference's choice among equal scores
+ *      depends on its lane layout and is not reproduced).
+ */
+static void decide_dual(const hkvo_table* t, int strategy, uint64_t key,
+                        const uint64_t* in_scores, uint64_t i, occupy_t* r) {
+  uint64_t b[2];
+  uint32_t st[2];
+  hkvo_locate_dual(key, t->buckets_num, b, st, &r->digest);
+  r->desired = desired_when_missed(t, strategy, in_scores, i);
+  for (int w = 0; w < 2; w++) {
+    const uint8_t* d = t->digests + b[w] * BUCKET;
+    const uint64_t* k = t->keys + b[w] * BUCKET;
+    for (uint32_t p = 0; p < BUCKET; p++)
+      if (d[p] == r->digest && k[p] == key) {
+        r->result = OCC_DUPLICATE;
+        r->bkt = b[w];
+        r->pos = p;
+        return;
+      }
+  }
+  const int first = t->sizes[b[0]] <= t->sizes[b[1]] ? 0 : 1;
+  for (int turn = 0; turn < 2; turn++) {
+    const int w = turn == 0 ? first : 1 - first;
+    if (t->sizes[b[w]] >= (int32_t)BUCKET) continue;
+    const uint8_t* d = t->digests + b[w] * BUCKET;
+    const uint64_t* k = t->keys + b[w] * BUCKET;
+    for (uint32_t off = 0; off < BUCKET; off++) {
+      uint32_t p = (st[w] + off) & (BUCKET - 1);
+      if (d[p] == t->empty_digest && k[p] == t->empty_key) {
+        r->result = OCC_EMPTY;
+        r->bkt = b[w];
+        r->pos = p;
+        return;
+      }
+    }
+  }
+  uint64_t mins[2] = {MAX_SCORE, MAX_SCORE};
+  int pos[2] = {-1, -1};
+  for (int w = 0; w < 2; w++) {
+    const uint64_t* k = t->keys + b[w] * BUCKET;
+    const uint64_t* s = t->scores + b[w] * BUCKET;
+    for (uint32_t p = 0; p < BUCKET; p++) {
+      if (k[p] == t->locked_key || k[p] == t->empty_key) continue;
+      if (s[p] < mins[w]) {
+        mins[w] = s[p];
+        pos[w] = (int)p;
+      }
+    }
+  }
+  const int w = mins[0] <= mins[1] ? 0 : 1;
+  r->min_score = mins[w];
+  if (r->desired < mins[w] || pos[w] < 0) {
+    r->result = OCC_REFUSED;
+    return;
+  }
+  r->bkt = b[w];
+  r->pos = (uint32_t)pos[w];
+  r->victim = t->keys[b[w] * BUCKET + (uint32_t)pos[w]];
+  r->result = (r->victim == t->reclaim_key) ? OCC_RECLAIMED : OCC_EVICT;
+}
+
 /* digest + score + bucket size for an accepted key (update_with_digest and
  * the atomicAdd on buckets_size, upsert.cuh:112-146, 203-215) */
 static void commit_meta(hkvo_table* t, int strategy, const occupy_t* r,
@@ -560,6 +710,10 @@ static int double_capacity(hkvo_table* t) {
 }
 
 int hkvo_reserve(hkvo_table* t, uint64_t new_capacity) {
+  {
+    int drc = refuse_dual(t, "reserve()", 1);
+    if (drc) return drc;
+  }
   if (t->reach_max_capacity || new_capacity > t->opts.max_capacity) {
     t->reach_max_capacity = t->capacity * 2 > t->opts.max_capacity;
     return HKV_SUCCESS;
@@ -613,13 +767,17 @@ static void upsert_one(hkvo_table* t, int strategy, uint64_t i,
   uint64_t key = keys[i];
   if (is_reserved(t, key)) return;
   occupy_t r;
-  decide(t, strategy, key, scores, i, 0, &r);
+  if (t->dual)
+    decide_dual(t, strategy, key, scores, i, &r);
+  else
+    decide(t, strategy, key, scores, i, 0, &r);
   if (r.result == OCC_REFUSED) return;
   commit_meta(t, strategy, &r, scores, i);
   uint64_t slot = r.bkt * BUCKET + r.pos;
   memcpy(t->values + slot * t->vb, values + i * t->vb, t->vb);
   t->keys[slot] = key;
 }
+
 
 /*
  * Hybrid mode (values partly in host memory) runs two kernels per call
@@ -693,6 +851,10 @@ int hkvo_insert_and_evict(hkvo_table* t, uint64_t n, const uint64_t* keys,
                           const void* values_, const uint64_t* scores,
                           uint64_t* ek, void* ev_, uint64_t* es,
                           uint64_t* counter, int ignore) {
+  {
+    int drc = refuse_dual(t, "insert_and_evict()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   {
     int grc = grow_for(t, n);
@@ -737,6 +899,10 @@ int hkvo_insert_and_evict(hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_find_or_insert(hkvo_table* t, uint64_t n, const uint64_t* keys,
                         void* values_, const uint64_t* scores, int ignore) {
+  {
+    int drc = refuse_dual(t, "find_or_insert()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   {
     int grc = grow_for(t, n);
@@ -775,6 +941,10 @@ int hkvo_find_or_insert(hkvo_table* t, uint64_t n, const uint64_t* keys,
 int hkvo_find_or_insert_slot(hkvo_table* t, uint64_t n, const uint64_t* keys,
                              uint64_t* slots, uint8_t* founds,
                              const uint64_t* scores, int ignore) {
+  {
+    int drc = refuse_dual(t, "find_or_insert()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   {
     int grc = grow_for(t, n);
@@ -838,6 +1008,10 @@ static void add_row(int kind, uint8_t* dst, const uint8_t* delta, uint64_t dim) 
 int hkvo_accum_or_assign(hkvo_table* t, uint64_t n, const uint64_t* keys,
                          const void* vd_, const uint8_t* flags,
                          const uint64_t* scores, int ignore) {
+  {
+    int drc = refuse_dual(t, "accum_or_assign()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   {
     int grc = grow_for(t, n);
@@ -895,6 +1069,10 @@ static int assign_impl(hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_assign(hkvo_table* t, uint64_t n, const uint64_t* keys,
                 const void* values, const uint64_t* scores) {
+  {
+    int drc = refuse_dual(t, "assign()", 0);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   int rc = check_scores_arg(t, t->strategy, scores);
   if (rc) return rc;
@@ -903,6 +1081,10 @@ int hkvo_assign(hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_assign_scores(hkvo_table* t, uint64_t n, const uint64_t* keys,
                        const uint64_t* scores) {
+  {
+    int drc = refuse_dual(t, "assign_scores()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   int rc = check_scores_arg(t, t->strategy, scores);
   if (rc) return rc;
@@ -911,6 +1093,10 @@ int hkvo_assign_scores(hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_assign_values(hkvo_table* t, uint64_t n, const uint64_t* keys,
                        const void* values) {
+  {
+    int drc = refuse_dual(t, "assign_values()", 1);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   return assign_impl(t, n, keys, (const uint8_t*)values, NULL, 0);
 }
@@ -938,6 +1124,10 @@ int hkvo_find(const hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_find_slot(const hkvo_table* t, uint64_t n, const uint64_t* keys,
                    uint64_t* slots, uint8_t* founds, uint64_t* scores) {
+  {
+    int drc = refuse_dual(t, "find() by pointer", 0);
+    if (drc) return drc;
+  }
   for (uint64_t i = 0; i < n; i++) {
     int64_t slot = is_reserved(t, keys[i]) ? -1 : lookup_slot(t, keys[i]);
     founds[i] = slot >= 0;
@@ -964,6 +1154,10 @@ static void touch_score(hkvo_table* t, uint64_t slot, const uint64_t* in, uint64
  * through a null pointer when a strategy needs scores that were not given. */
 int hkvo_lock_keys(hkvo_table* t, uint64_t n, const uint64_t* keys, uint64_t* slots,
                    uint8_t* success, const uint64_t* scores) {
+  {
+    int drc = refuse_dual(t, "lock_keys()", 0);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   int rc = check_scores_arg(t, t->strategy, scores);
   if (rc) return rc;
@@ -983,6 +1177,10 @@ int hkvo_lock_keys(hkvo_table* t, uint64_t n, const uint64_t* keys, uint64_t* sl
  * core_kernels.cuh:1180-1204) */
 int hkvo_unlock_keys(hkvo_table* t, uint64_t n, const uint64_t* slots,
                      const uint64_t* keys, uint8_t* success) {
+  {
+    int drc = refuse_dual(t, "unlock_keys()", 0);
+    if (drc) return drc;
+  }
   for (uint64_t i = 0; i < n; i++) {
     int ok = slots[i] != UINT64_MAX && t->keys[slots[i]] == t->locked_key;
     if (ok) t->keys[slots[i]] = keys[i];
@@ -997,6 +1195,10 @@ int hkvo_unlock_keys(hkvo_table* t, uint64_t n, const uint64_t* slots,
  * finds; scores[i] returns the score after the touch. */
 int hkvo_find_and_update(hkvo_table* t, uint64_t n, const uint64_t* keys,
                          uint64_t* slots, uint8_t* founds, uint64_t* scores) {
+  {
+    int drc = refuse_dual(t, "find_and_update()", 0);
+    if (drc) return drc;
+  }
   if (n == 0) return HKV_SUCCESS;
   int rc = check_scores_arg(t, t->strategy, scores);
   if (rc) return rc;
@@ -1014,6 +1216,10 @@ int hkvo_find_and_update(hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 int hkvo_contains(const hkvo_table* t, uint64_t n, const uint64_t* keys,
                   uint8_t* founds) {
+  {
+    int drc = refuse_dual(t, "contains()", 1);
+    if (drc) return drc;
+  }
   for (uint64_t i = 0; i < n; i++)
     founds[i] = !is_reserved(t, keys[i]) && lookup_slot(t, keys[i]) >= 0;
   return HKV_SUCCESS;
@@ -1021,6 +1227,10 @@ int hkvo_contains(const hkvo_table* t, uint64_t n, const uint64_t* keys,
 
 /* remove_kernel, core_kernels.cuh:679-741 */
 int hkvo_erase(hkvo_table* t, uint64_t n, const uint64_t* keys) {
+  {
+    int drc = refuse_dual(t, "erase()", 1);
+    if (drc) return drc;
+  }
   for (uint64_t i = 0; i < n; i++) {
     if (is_reserved(t, keys[i])) continue;
     int64_t slot = lookup_slot(t, keys[i]);
@@ -1178,6 +1388,8 @@ int hkvo_insert_or_assign_mt(hkvo_table* t, uint64_t n, const uint64_t* keys,
                              const void* values, const uint64_t* scores,
                              int ignore, int threads) {
   if (n == 0) return HKV_SUCCESS;
+  /* a key of a dual-bucket table has two buckets: no disjoint bucket ranges */
+  if (t->dual) return hkvo_insert_or_assign(t, n, keys, values, scores, ignore);
   {
     int grc = grow_for(t, n);
     if (grc) return grc;

@@ -39,6 +39,12 @@ int hkvo_reserved_keys(int start_bit, uint64_t out[7]);
 void hkvo_locate(uint64_t key, uint64_t buckets_num, uint64_t* bkt,
                  uint32_t* start, uint8_t* digest);
 
+/* dual-bucket mode (TableMode::kMemory): both candidate buckets, their start
+ * positions and the digest (hash bits 56..63), dual_bucket_utils.cuh:36-74,
+ * dual_bucket_upsert.cuh:86-101 */
+void hkvo_locate_dual(uint64_t key, uint64_t buckets_num, uint64_t bkt[2],
+                      uint32_t start[2], uint8_t* digest);
+
 /* create_table (core_kernels.cuh:327-381) + argument checks of
  * HashTable::init (merlin_hashtable.cuh:1016-1048).  `hybrid_refusal` selects
  * the `score <= min` refusal rule of the hybrid kernels (upsert.cuh:1524)

@@ -707,6 +707,76 @@ static void test_functor_forms() {
   run_functor_forms<3>();   // one thread per slot
 }
 
+
+// TableMode::kMemory through the header: init checks, insert_or_assign + find, guards
+// (tests/dual_bucket_test.cc.cu:74-158, 471-515, 641-661, 1051-1107)
+static void test_dual_bucket_mode() {
+  constexpr size_t DIM = 16, CAP = 128 * 128, N = 8000;
+  using Table = HashTable<K, V, S, EvictStrategy::kCustomized>;
+  auto make = [&](size_t init, size_t max, size_t hbm, size_t dim) {
+    HashTableOptions o;
+    o.init_capacity = init;
+    o.max_capacity = max;
+    o.max_hbm_for_vectors = hbm;
+    o.dim = dim;
+    o.table_mode = TableMode::kMemory;
+    return o;
+  };
+  auto rejects = [&](const HashTableOptions& o) {
+    Table t;
+    try {
+      t.init(o);
+    } catch (const std::exception&) {
+      return true;
+    }
+    return false;
+  };
+  CHECK(rejects(make(CAP, 2 * CAP, 0, DIM)));
+  CHECK(rejects(make(CAP, CAP, GB(1), DIM)));
+  CHECK(rejects(make(CAP, CAP, 0, 225)));
+  CHECK(rejects(make(128, 128, 0, DIM)));
+  Table table;
+  table.init(make(CAP, CAP, 0, DIM));
+  auto keys = random_keys(N, 99);
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  for (size_t i = 0; i < N; i++) scores[i] = 10 + i;
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM), dout(N * DIM);
+  DevBuf<S> ds(N), dso(N);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p);
+  CHECK(table.size() == N);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  auto f = df.down(N);
+  CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  CHECK(dout.down(N * DIM) == vals);
+  CHECK(dso.down(N) == scores);
+  int threw = 0;
+  auto expect_throw = [&](auto&& call) {
+    try {
+      call();
+    } catch (const std::exception&) {
+      threw++;
+    }
+  };
+  expect_throw([&] { table.erase(N, dk.p); });
+  expect_throw([&] { table.contains(N, dk.p, df.p); });
+  expect_throw([&] { table.reserve(2 * CAP); });
+  expect_throw([&] { table.find_or_insert(N, dk.p, dout.p, ds.p); });
+  expect_throw([&] { table.assign_scores(N, dk.p, ds.p); });
+  expect_throw([&] { table.assign_values(N, dk.p, dv.p); });
+  expect_throw([&] { table.insert_or_assign(N, dk.p, dv.p, ds.p, 0, false); });
+  CHECK(threw == 7);
+  CHECK(table.size() == N);
+  table.clear();
+  CHECK(table.size() == 0);
+}
+
 int main() {
   try {
     test_basic();
@@ -716,6 +786,7 @@ int main() {
     test_option_checks();
     test_growth_and_key_locks();
     test_functor_forms();
+    test_dual_bucket_mode();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;

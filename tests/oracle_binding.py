@@ -26,6 +26,7 @@ _SIG = {
     "hkvo_murmur3_fmix64": (_u64, [_u64]),
     "hkvo_reserved_keys": (_i, [_i, C.POINTER(_u64)]),
     "hkvo_locate": (None, [_u64, _u64, C.POINTER(_u64), C.POINTER(C.c_uint32), C.POINTER(C.c_uint8)]),
+    "hkvo_locate_dual": (None, [_u64, _u64, C.POINTER(_u64), C.POINTER(C.c_uint32), C.POINTER(C.c_uint8)]),
     "hkvo_create": (_i, [C.POINTER(Options), _i, C.POINTER(_p)]),
     "hkvo_destroy": (None, [_p]),
     "hkvo_last_error": (C.c_char_p, []),
@@ -101,6 +102,15 @@ def locate(key, buckets_num):
     d = C.c_uint8()
     _lib.hkvo_locate(key, buckets_num, C.byref(b), C.byref(s), C.byref(d))
     return b.value, s.value, d.value
+
+
+def locate_dual(key, buckets_num):
+    """((b1, b2), (start1, start2), digest) of a key in dual-bucket mode."""
+    b = (_u64 * 2)()
+    s = (C.c_uint32 * 2)()
+    d = C.c_uint8()
+    _lib.hkvo_locate_dual(key, buckets_num, b, s, C.byref(d))
+    return (b[0], b[1]), (s[0], s[1]), d.value
 
 
 def online_cores():

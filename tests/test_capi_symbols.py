@@ -47,8 +47,15 @@ def test_option_checks_need_no_gpu():
         t = HashTable()
         with pytest.raises(MerlinException):
             t.init(default_options(init_capacity=1024, max_capacity=1024, **bad))
+    # dual-bucket mode has checks of its own (merlin_hashtable.cuh:992-1014)
+    for bad in (dict(init_capacity=1024, max_capacity=2048), dict(max_hbm_for_vectors=1 << 30),
+                dict(dim=225), dict(init_capacity=128, max_capacity=128)):
+        kw = dict(init_capacity=1024, max_capacity=1024, max_hbm_for_vectors=0, dim=4, table_mode=1)
+        kw.update(bad)
+        with pytest.raises(MerlinException):
+            HashTable().init(default_options(**kw))
     t = HashTable()
-    with pytest.raises(NotImplementedError):
-        t.init(default_options(init_capacity=1024, max_capacity=1024, table_mode=1))
+    with pytest.raises(ValueError):
+        t.init(default_options(init_capacity=1024, max_capacity=1024, table_mode=2))
     with pytest.raises(NotImplementedError):
         t.init(default_options(init_capacity=1024, max_capacity=1024, score_size=4))

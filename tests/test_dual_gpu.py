@@ -1,0 +1,288 @@
+"""GPU tests of dual-bucket mode (TableMode::kMemory): insert_or_assign and find.
+
+Where a key lands depends on the sizes of its two buckets at that moment, so a
+batch applied concurrently is order-dependent in general.  Bit-exact parity
+with the oracle is therefore checked on batches whose keys have pairwise
+disjoint candidate buckets (then every key sees the table as it was before the
+batch, on the GPU as in the oracle's input order), bucket by bucket; ordinary
+batches are checked through the scenarios and bounds of the reference's own
+tests (tests/dual_bucket_test.cc.cu) and through invariants.
+"""
+import numpy as np
+import pytest
+import torch
+
+import workloads as w
+from gpu_util import DEV, dev, export_table, host_u64, sort_by_key
+from hierarchicalkv_amd import EvictStrategy, HashTable, MerlinException, default_options
+
+pytestmark = pytest.mark.gpu
+
+
+def dual_options(capacity, dim, strategy=EvictStrategy.kCustomized, **kw):
+    # create_memory_mode_table, tests/dual_bucket_test.cc.cu:42-52
+    return default_options(init_capacity=capacity, max_capacity=capacity, max_hbm_for_vectors=0,
+                           dim=dim, table_mode=1, evict_strategy=strategy, **kw)
+
+
+def bytes_of(vals):
+    return np.ascontiguousarray(vals).view(np.uint8).reshape(len(vals), -1)
+
+
+def gpu_find(t, keys, dim, dtype=torch.float32):
+    n = len(keys)
+    out = torch.zeros(n, dim, dtype=dtype, device=DEV)
+    f = torch.zeros(n, dtype=torch.bool, device=DEV)
+    s = torch.zeros(n, dtype=torch.int64, device=DEV)
+    t.find(n, dev(keys), out, f, s)
+    torch.cuda.synchronize()
+    return bytes_of(out.cpu().numpy()), f.cpu().numpy(), host_u64(s)
+
+
+def buckets_of(table, vb, nb):
+    """Per bucket: sorted (key, score, value bytes) of what the GPU table holds there."""
+    out = []
+    dk = torch.zeros(128, dtype=torch.int64, device=DEV)
+    dv = torch.zeros(128 * vb, dtype=torch.uint8, device=DEV)
+    ds = torch.zeros(128, dtype=torch.int64, device=DEV)
+    dc = torch.zeros(1, dtype=torch.int64, device=DEV)
+    for b in range(nb):
+        table.export_batch(128, 128 * b, dc, dk, dv, ds)
+        torch.cuda.synchronize()
+        c = int(dc.item())
+        out.append(sort_by_key(host_u64(dk[:c]).copy(), dv[:c * vb].cpu().numpy().reshape(c, vb).copy(),
+                               host_u64(ds[:c]).copy()))
+    return out
+
+
+def disjoint_batches(oracle, keys, nb, limit):
+    """Split keys into batches in which no two keys share a candidate bucket."""
+    batches, cur, used = [], [], set()
+    for k in keys.tolist():
+        (b1, b2), _, _ = oracle.locate_dual(k, nb)
+        if b1 in used or b2 in used or len(cur) >= limit:
+            batches.append(np.array(cur, dtype=np.uint64))
+            cur, used = [], set()
+        cur.append(k)
+        used.update((b1, b2))
+    if cur:
+        batches.append(np.array(cur, dtype=np.uint64))
+    return batches
+
+
+@pytest.mark.parametrize("strategy,dim,dtype", [
+    (EvictStrategy.kCustomized, 8, np.float32),
+    (EvictStrategy.kLru, 5, np.float32),
+    (EvictStrategy.kLfu, 3, np.int8),
+])
+def test_parity_on_bucket_disjoint_batches(oracle, strategy, dim, dtype):
+    nb = 64
+    cap = nb * 128
+    kw = {}
+    if dtype == np.int8:
+        kw = dict(value_kind=0, value_size=1)
+    o = dual_options(cap, dim, strategy, **kw)
+    t = HashTable()
+    t.init(o)
+    ot = oracle.OracleTable(o)
+    if strategy == EvictStrategy.kLru:
+        t.set_clock(1, 1 << 50)
+        ot.set_clock(1, 1 << 50)
+    vb = dim * np.dtype(dtype).itemsize
+    rng = np.random.default_rng(1234 + dim)
+    universe = w.unique_keys(900 + dim, 0, int(cap * 1.6))
+    # 2.2 x capacity upserts: fresh keys, then a mix of old (updates) and fresh ones
+    seq = np.concatenate([universe[:cap], rng.permutation(universe)[:int(cap * 1.2)]])
+    batches = disjoint_batches(oracle, seq, nb, 24)
+    assert np.mean([len(b) for b in batches]) > 4
+    perm = rng.permutation(len(seq)).astype(np.uint64) + np.uint64(1)  # distinct, in no order
+    counter = 0
+    checks = {len(batches) // 3, 2 * len(batches) // 3, len(batches) - 1}
+    for bi, keys in enumerate(batches):
+        n = len(keys)
+        if dtype == np.int8:
+            vals = rng.integers(-128, 127, (n, dim), dtype=np.int8)
+        else:
+            vals = rng.random((n, dim), dtype=np.float32)
+        sc = None
+        if strategy == EvictStrategy.kCustomized:
+            sc = perm[counter:counter + n].copy()  # refusals, evictions and re-scores downwards
+        elif strategy == EvictStrategy.kLfu:
+            sc = rng.integers(1, 1 << 40, n, dtype=np.uint64)
+        counter += n
+        t.insert_or_assign(n, dev(keys), dev(vals), dev(sc))
+        ot.insert_or_assign(keys, bytes_of(vals), sc)
+        if bi in checks:
+            assert t.size() == ot.size()
+            got = buckets_of(t, vb, nb)
+            for b in range(nb):
+                ek, ev, es = sort_by_key(*ot.export_batch_if(n=128, offset=128 * b))
+                gk, gv, gs = got[b]
+                assert np.array_equal(gk, ek), (bi, b)
+                assert np.array_equal(gs, es), (bi, b)
+                assert np.array_equal(gv, ev), (bi, b)
+    assert ot.size() > 0.97 * cap  # the table did fill up and evict
+    # find agrees for residents, evicted and never-seen keys
+    q = np.concatenate([universe, w.unique_keys(5, 0, 1000)])
+    tdtype = torch.int8 if dtype == np.int8 else torch.float32
+    gv, gf, gs = gpu_find(t, q, dim, tdtype)
+    ov, of, os_ = ot.find(q)
+    assert np.array_equal(gf, of)
+    assert np.array_equal(gs[of], os_[of]) and np.array_equal(gv[of], ov[of])
+    t.close()
+    ot.close()
+
+
+def test_b1_equals_b2_update_and_clear(oracle):
+    # tests/dual_bucket_test.cc.cu:74-237, 663-742, 1841-1900
+    o = dual_options(4 * 128, 16)
+    t = HashTable()
+    t.init(o)
+    keys = np.arange(1, 257, dtype=np.uint64)
+    vals = np.repeat(keys.astype(np.float32)[:, None], 16, axis=1)
+    t.insert_or_assign(256, dev(keys), dev(vals), dev(keys.copy()))
+    assert t.size() == 256
+    gv, gf, gs = gpu_find(t, keys, 16)
+    assert gf.all() and np.array_equal(gv, bytes_of(vals)) and np.array_equal(gs, keys)
+    t.insert_or_assign(256, dev(keys), dev(vals * 2), dev(keys + 1000))
+    assert t.size() == 256
+    gv, gf, gs = gpu_find(t, keys, 16)
+    assert gf.all() and np.array_equal(gv, bytes_of(vals * 2)) and np.array_equal(gs, keys + 1000)
+    ek, _, _ = export_table(t, 64)
+    assert sorted(ek.tolist()) == keys.tolist()
+    # absent and reserved keys
+    q = np.array([1000, 2000, (1 << 64) - 1, (1 << 64) - 2, (1 << 64) - 3, (1 << 64) - 4], dtype=np.uint64)
+    _, gf, _ = gpu_find(t, q, 16)
+    assert not gf.any()
+    t.insert_or_assign(len(q), dev(q), dev(np.zeros((len(q), 16), np.float32)), dev(q.copy()))
+    assert t.size() == 258  # the four reserved keys were skipped
+    t.clear()
+    assert t.size() == 0
+    _, gf, _ = gpu_find(t, keys, 16)
+    assert not gf.any()
+    t.insert_or_assign(256, dev(keys), dev(vals), dev(keys.copy()))
+    gv, gf, _ = gpu_find(t, keys, 16)
+    assert gf.all() and np.array_equal(gv, bytes_of(vals)) and t.size() == 256
+    # empty batch
+    t.insert_or_assign(0, None, None, None)
+    t.close()
+
+
+def test_init_checks_and_guards():
+    # tests/dual_bucket_test.cc.cu:471-515, 641-661, 941-1107, 1187-1196
+    for bad in (dict(init_capacity=1024, max_capacity=2048), dict(max_hbm_for_vectors=1 << 30),
+                dict(dim=225), dict(init_capacity=128, max_capacity=128)):
+        kw = dict(init_capacity=1024, max_capacity=1024, max_hbm_for_vectors=0, dim=4, table_mode=1,
+                  evict_strategy=EvictStrategy.kCustomized)
+        kw.update(bad)
+        with pytest.raises(MerlinException):
+            HashTable().init(default_options(**kw))
+    big = HashTable()
+    big.init(dual_options(256, 224))
+    big.close()
+    t = HashTable()
+    t.init(dual_options(1024, 4))
+    assert t.is_pure_hbm()
+    n = 8
+    keys = dev(np.arange(1, n + 1, dtype=np.uint64))
+    vals = torch.ones(n, 4, dtype=torch.float32, device=DEV)
+    sc = dev(np.arange(1, n + 1, dtype=np.uint64))
+    flags = torch.ones(n, dtype=torch.bool, device=DEV)
+    ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    cnt = torch.zeros(1, dtype=torch.int64, device=DEV)
+    t.insert_or_assign(n, keys, vals, sc)
+    with pytest.raises(MerlinException):
+        t.insert_or_assign(n, keys, vals, sc, unique_key=False)
+    calls = [
+        lambda: t.erase(n, keys),
+        lambda: t.contains(n, keys, flags),
+        lambda: t.reserve(2048),
+        lambda: t.find_or_insert(n, keys, vals, sc),
+        lambda: t.find_or_insert_ptr(n, keys, ptrs, flags, sc),
+        lambda: t.insert_and_evict(n, keys, vals, sc, keys.clone(), vals.clone(), sc.clone(), cnt),
+        lambda: t.accum_or_assign(n, keys, vals, flags, sc),
+        lambda: t.assign_scores(n, keys, sc),
+        lambda: t.assign_values(n, keys, vals),
+        lambda: t.assign(n, keys, vals, sc),
+        lambda: t.find_ptr(n, keys, ptrs, flags),
+        lambda: t.lock_keys(n, keys, ptrs, flags),
+        lambda: t.find_and_update(n, keys, ptrs, flags),
+    ]
+    for call in calls:
+        with pytest.raises(Exception) as e:
+            call()
+        assert "MEMORY_MODE" in str(e.value)
+    assert t.size() == n
+    t.close()
+
+
+def test_no_loss_before_the_first_eviction_and_load_factor(oracle):
+    # tests/dual_bucket_test.cc.cu:399-465 (batches of 128, score = key): nothing is evicted
+    # below load factor 0.98.  Up to 0.9 big batches are used here, then the reference's 128.
+    cap = 1 << 20
+    dim = 4
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    nxt, inserted, first = 1, 0, None
+    while inserted < cap:
+        n = 1 << 16 if inserted + (1 << 16) <= int(cap * 0.9) else 128
+        keys = np.arange(nxt, nxt + n, dtype=np.uint64)
+        vals = w.values_from_keys(keys, dim)
+        t.insert_or_assign(n, dev(keys), dev(vals), dev(keys.copy()))
+        nxt += n
+        inserted += n
+        size = t.size()
+        if size < inserted:
+            first = size / cap
+            break
+        if n > 128 and inserted >= int(cap * 0.9) - (1 << 16):
+            # every key so far is there, with its row and score
+            allk = np.arange(1, nxt, dtype=np.uint64)
+            gv, gf, gs = gpu_find(t, allk, dim)
+            assert gf.all() and np.array_equal(gs, allk)
+            assert np.array_equal(gv, bytes_of(w.values_from_keys(allk, dim)))
+    assert first is not None and first > 0.980, first
+    print(f"dual-bucket first eviction at load factor {first:.4f} (capacity 2^20)")
+    t.close()
+
+
+def test_eviction_quality_and_consistency_at_full_load(oracle):
+    # tests/dual_bucket_test.cc.cu:1406-1520 (quality >= 0.995) and :239-330 (score eviction)
+    cap = 128 * 1024
+    dim = 8
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    total = 5 * cap
+    rng = np.random.default_rng(42)
+    keys = np.arange(1, total + 1, dtype=np.uint64)
+    scores = (rng.integers(0, 1 << 63, total, dtype=np.uint64) >> np.uint64(1)) | np.uint64(1)
+    for lo in range(0, total, cap):
+        k = keys[lo:lo + cap]
+        t.insert_or_assign(cap, dev(k), dev(w.values_from_keys(k, dim)), dev(scores[lo:lo + cap]))
+    ek, ev, es = export_table(t, dim * 4)
+    assert len(ek) == t.size() and len(ek) > 0.99 * cap
+    assert len(np.unique(ek)) == len(ek), "a key sits in both of its buckets"
+    ideal = set(keys[np.argsort(scores)[::-1][:len(ek)]].tolist())
+    quality = sum(1 for k in ek.tolist() if k in ideal) / len(ek)
+    print(f"dual-bucket eviction quality {quality:.4f}, load factor {len(ek) / cap:.4f}")
+    assert quality >= 0.995
+    # residents carry their own score and row, and find sees exactly the exported set
+    assert np.array_equal(es, scores[ek.astype(np.int64) - 1])
+    assert np.array_equal(ev, bytes_of(w.values_from_keys(ek, dim)))
+    gv, gf, gs = gpu_find(t, keys, dim)
+    assert int(gf.sum()) == len(ek) and set(keys[gf].tolist()) == set(ek.tolist())
+    assert np.array_equal(gs[gf], scores[gf])
+    # every resident key is in one of its two candidate buckets: a find could not see it otherwise,
+    # and the bucket sizes add up
+    assert t.size() == len(ek)
+    # high scores go in, low scores are refused
+    newk = np.arange(total + 1, total + 1025, dtype=np.uint64)
+    hi = np.full(1024, 1 << 63, dtype=np.uint64) + np.arange(1024, dtype=np.uint64)
+    t.insert_or_assign(1024, dev(newk), dev(w.values_from_keys(newk, dim)), dev(hi))
+    _, gf, _ = gpu_find(t, newk, dim)
+    assert gf.sum() > 0.8 * 1024  # tests/dual_bucket_test.cc.cu:318-320
+    lowk = np.arange(total + 5000, total + 5100, dtype=np.uint64)
+    t.insert_or_assign(100, dev(lowk), dev(w.values_from_keys(lowk, dim)), dev(np.zeros(100, np.uint64)))
+    _, gf, _ = gpu_find(t, lowk, dim)
+    assert not gf.any()
+    t.close()
