@@ -183,6 +183,11 @@ __device__ __forceinline__ bool cas_lock(uint64_t* p, uint64_t& expected,
                                               __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                               __HIP_MEMORY_SCOPE_AGENT);
 }
+/* Slot lock without knowing what the slot holds: the key word becomes LOCKED and its
+ * previous content comes back. */
+__device__ __forceinline__ uint64_t swap_lock(uint64_t* p, uint64_t locked) {
+  return __hip_atomic_exchange(p, locked, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 /* Every store this wavefront has issued is complete (written through) and the
  * compiler moves no memory access across this point. */
 __device__ __forceinline__ void wait_stores() {

@@ -622,9 +622,13 @@ upsert_kernel(View v, UpsertArgs a) {
         got = kStRefused;
       } else {
         uint64_t* kp = v.keys + bslot + bpos;
-        const uint64_t vk = ld_u64(kp);
-        uint64_t seen = vk;
-        if (vk != v.locked_key && vk != v.empty_key && cas_lock(kp, seen, v.locked_key)) {
+        /* one exchange instead of a load and a CAS: whatever key the slot held is the
+         * victim and the slot is locked.  LOCKED coming back means somebody else holds
+         * the slot (nothing changed); EMPTY is put back at once. */
+        const uint64_t vk = swap_lock(kp, v.locked_key);
+        const bool mine = vk != v.locked_key && vk != v.empty_key;
+        if (vk == v.empty_key) st_unlock(kp, vk);
+        if (mine) {
           /* somebody may have raised the score since the scan */
           if (ld_u64(v.scores + bslot + bpos) <= best) {
             victim = vk;
