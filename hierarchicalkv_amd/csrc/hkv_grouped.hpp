@@ -293,7 +293,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
     const bool needs_old = a.strategy == HKV_LFU || a.strategy == HKV_EPOCH_LFU;
     const uint64_t old = needs_old ? v.scores[slot] : 0;
     uint64_t snew;
-    if (final_score(a, false, desired, in_score, old, snew)) v.scores[slot] = snew;
+    if (final_score(a, false, desired, in_score, old, snew) && !HKV_EXP_FLAG(256)) v.scores[slot] = snew;
   }
   if (OP == kOpAccumOrAssign) {
     /* rows move for the keys that stay "present" only */
@@ -313,6 +313,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
   uint8_t* usr_base = (OP == kOpFindOrInsert ? a.values_io : const_cast<uint8_t*>(a.values_in)) +
                       base * v.value_bytes;
   for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
+    if (HKV_EXP_FLAG(1024)) break;
     T buf[kBatch];
     T tab[OP == kOpAccumOrAssign ? kBatch : 1];
 #pragma unroll
@@ -328,7 +329,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
           if (OP == kOpFindOrInsert) {
             buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
           } else {
-            buf[b] = reinterpret_cast<const T*>(usr_base + (uint64_t)kk * v.value_bytes)[c];
+            buf[b] = ld_unit<VEC, false>(usr_base + (uint64_t)kk * v.value_bytes, c);
             if (OP == kOpAccumOrAssign)
               tab[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
           }
@@ -344,11 +345,11 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
         const int64_t sl = s_slot[kk];
         if (sl >= 0) {
           if (OP == kOpFindOrInsert) {
-            reinterpret_cast<T*>(usr_base + (uint64_t)kk * v.value_bytes)[c] = buf[b];
+            st_unit<VEC, false>(usr_base + (uint64_t)kk * v.value_bytes, c, buf[b]);
           } else if (OP == kOpAccumOrAssign) {
             st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, add_unit(tab[b], buf[b], a.value_kind));
           } else {
-            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
+            if (!HKV_EXP_FLAG(512)) st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
           }
         }
       }

@@ -283,7 +283,16 @@ lookup_kernel(View v, FindArgs a) {
         const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
         const uint32_t c = idx - kk * units;
         if (s_slot[kk] >= 0) {
-          reinterpret_cast<T*>(a.out_values + (base + kk) * v.value_bytes)[c] = buf[b];
+          T* dst = reinterpret_cast<T*>(a.out_values + (base + kk) * v.value_bytes) + c;
+          if constexpr (VEC == 16) {
+            /* streaming store: the output is not read again here, and rows left dirty
+             * in the caches would be written back at the expense of the next call
+             * (measured: find itself 2 % slower, a following upsert 6 % faster) */
+            const u32x4_t t = {buf[b].x, buf[b].y, buf[b].z, buf[b].w};
+            __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(dst));
+          } else {
+            *dst = buf[b];
+          }
         }
       }
     }

@@ -157,7 +157,14 @@ template <int VEC, bool TABLE>
 __device__ __forceinline__ typename VecType<VEC>::type ld_unit(const uint8_t* row, uint32_t u) {
   using T = typename VecType<VEC>::type;
   if constexpr (!TABLE) {
-    return reinterpret_cast<const T*>(row)[u];
+    if constexpr (VEC == 16) {
+      /* a caller's row is read once: streaming load, so that it does not push table
+       * lines out of the caches */
+      const u32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(row) + u);
+      return make_uint4(t.x, t.y, t.z, t.w);
+    } else {
+      return reinterpret_cast<const T*>(row)[u];
+    }
   } else if constexpr (VEC == 16) {
     const uint64_t* p = reinterpret_cast<const uint64_t*>(row) + 2 * u;
     const uint64_t lo = ld_u64(p), hi = ld_u64(p + 1);
@@ -172,7 +179,13 @@ template <int VEC, bool TABLE>
 __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecType<VEC>::type x) {
   using T = typename VecType<VEC>::type;
   if constexpr (!TABLE) {
-    reinterpret_cast<T*>(row)[u] = x;
+    if constexpr (VEC == 16) {
+      /* written once, not read again by this kernel: streaming store */
+      const u32x4_t t = {x.x, x.y, x.z, x.w};
+      __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(row) + u);
+    } else {
+      reinterpret_cast<T*>(row)[u] = x;
+    }
   } else if constexpr (VEC == 16) {
 #ifdef HKV_EXP_PLAIN_ROW_STORES
     reinterpret_cast<T*>(row)[u] = x;
