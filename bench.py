@@ -63,6 +63,13 @@ def main():
                     help="also run one plain 1 GiB device copy (reference point for "
                          "FETCH_SIZE / WRITE_SIZE when profiling)")
     ap.add_argument("--cpu-capacity-log2", type=int, default=24)
+    ap.add_argument("--matrix", action="store_true",
+                    help="instead of the one-line benchmark: the reference's own benchmark table "
+                         "(README.md:245-317, benchmark/merlin_hashtable_benchmark.cc.cu), every API "
+                         "at load factor 0.50 / 0.75 / 1.00 for dim 8, 32 and 64, printed as markdown")
+    ap.add_argument("--matrix-hybrid", action="store_true",
+                    help="with --matrix: the hybrid table of README.md:289-303 (dim 64, capacity "
+                         "128M, 16 GB of the rows in HBM, the rest in pinned host memory)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path "
@@ -78,6 +85,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.matrix:
+        run_matrix(args, np, torch, dev)
+        return
     cap = 1 << args.capacity_log2
     dim = args.dim
     n = 1 << args.batch_log2
@@ -233,6 +243,104 @@ def main():
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args, np, w)
     print(json.dumps(result))
+
+
+def run_matrix(args, np, torch, dev):
+    """The reference's benchmark protocol (benchmark/merlin_hashtable_benchmark.cc.cu:75-420):
+    LRU table, consecutive integer keys up to the load factor, then ONE timed call of 2^20 keys
+    per API, 60 % of them from the last inserted batch and 40 % never seen
+    (benchmark_util.cuh:135-177), wall clock from the call to the end of the stream, best of two,
+    in units of 2^30 KV/s.  One table per (dim, load factor) serves all APIs here, read-only ones
+    first (the reference builds a fresh table per API; an insert of 0.4 M new keys moves the load
+    factor of a 64 M table by 0.6 %)."""
+    from hierarchicalkv_amd import EvictStrategy, HashTable, default_options, Predicate
+
+    n = 1 << 20
+    M = 1 << 20
+    if args.matrix_hybrid:
+        configs = [(64, 128 * M, 16 << 30)]
+    else:
+        configs = [(8, 128 * M, 4 << 30), (32, 128 * M, 16 << 30), (64, 64 * M, 16 << 30)]
+    apis = ["insert_or_assign", "find", "find_or_insert", "assign", "find*", "find_or_insert*",
+            "insert_and_evict", "export_batch", "export_batch_if", "contains"]
+    order = ["find", "find*", "contains", "export_batch", "export_batch_if", "assign",
+             "find_or_insert", "find_or_insert*", "insert_or_assign", "insert_and_evict"]
+
+    def d64(a):
+        return torch.from_numpy(a.view(np.int64)).to(dev)
+
+    print("| dim | capacity | HBM for rows | load factor | " + " | ".join(apis) + " |")
+    print("|---|---|---|---|" + "---|" * len(apis))
+    for dim, cap, hbm in configs:
+        for lf in (0.50, 0.75, 1.00):
+            table = HashTable()
+            table.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=hbm,
+                                       dim=dim, evict_strategy=EvictStrategy.kLru))
+            vals = torch.ones(n, dim, dtype=torch.float32, device=dev)
+            defv = torch.full((n, dim), 2.0, dtype=torch.float32, device=dev)
+            ptrs = torch.zeros(n, dtype=torch.int64, device=dev)
+            founds = torch.zeros(n, dtype=torch.bool, device=dev)
+            scores = torch.zeros(n, dtype=torch.int64, device=dev)
+            ek = torch.zeros(n, dtype=torch.int64, device=dev)
+            es = torch.zeros(n, dtype=torch.int64, device=dev)
+            cnt = torch.zeros(1, dtype=torch.int64, device=dev)
+            # step 1 and 2 of the reference: consecutive keys, then top up to the load factor
+            start = 0
+            target = int(cap * lf)
+            while start < target:
+                m = min(n, target - start)
+                table.insert_or_assign(m, d64(np.arange(start, start + m, dtype=np.uint64)), vals)
+                start += m
+            while True:
+                short = target - table.size()
+                if short <= cap * 1e-3 or start > 3 * cap:
+                    break
+                m = min(n, short)
+                table.insert_or_assign(m, d64(np.arange(start, start + m, dtype=np.uint64)), vals)
+                start += m
+            threshold = 0  # the reference's threshold is the device clock before the prefill: keeps all
+            res = {}
+            fresh = (1 << 64) - 5  # never-seen keys count down from the top, below the reserved ones
+            for api in order:
+                best = float("inf")
+                for rep in range(2):
+                    hit = np.arange(start - n, start - n + int(n * 0.6), dtype=np.uint64)
+                    m_new = n - len(hit)
+                    new = np.arange(fresh - m_new + 1, fresh + 1, dtype=np.uint64)[::-1]
+                    fresh -= m_new
+                    keys = d64(np.concatenate([hit, new]))
+                    cnt.zero_()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    if api == "find":
+                        table.find(n, keys, vals, founds)  # LRU: no scores asked for (:108)
+                    elif api == "find*":
+                        table.find_ptr(n, keys, ptrs, founds)
+                    elif api == "contains":
+                        table.contains(n, keys, founds)
+                    elif api == "export_batch":
+                        table.export_batch(int(n / lf * 0.995), 0, cnt, keys, vals)
+                    elif api == "export_batch_if":
+                        table.export_batch_if(Predicate.kScoreGt, 0, threshold, int(n / lf * 0.995), 0,
+                                              cnt, keys, vals)
+                    elif api == "assign":
+                        table.assign(n, keys, defv)
+                    elif api == "find_or_insert":
+                        table.find_or_insert(n, keys, vals)
+                    elif api == "find_or_insert*":
+                        table.find_or_insert_ptr(n, keys, ptrs, founds)
+                    elif api == "insert_or_assign":
+                        table.insert_or_assign(n, keys, vals)
+                    elif api == "insert_and_evict":
+                        table.insert_and_evict(n, keys, vals, None, ek, defv, es, cnt)
+                    torch.cuda.synchronize()
+                    best = min(best, time.perf_counter() - t0)
+                res[api] = n / best / float(1 << 30)
+            print("| %d | %dM | %d GB | %.2f | " % (dim, cap // M, hbm >> 30, table.size() / cap)
+                  + " | ".join("%.3f" % res[a] for a in apis) + " |", flush=True)
+            table.close()
+            del table, vals, defv
+            torch.cuda.empty_cache()
 
 
 def cpu_baseline(args, np, w):

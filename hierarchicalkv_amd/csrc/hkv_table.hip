@@ -633,9 +633,8 @@ template <class Pred>
 void launch_export(const hkv_table* t, uint64_t pattern, uint64_t threshold,
                    uint64_t n, uint64_t offset, uint64_t* d_counter,
                    uint64_t* keys, void* values, uint64_t* scores, hipStream_t s) {
-  const uint64_t waves = (n + kWave - 1) / kWave;
-  const unsigned blocks = (unsigned)std::min<uint64_t>((waves + 3) / 4, 16384);
-  hipLaunchKernelGGL((export_if_kernel<Pred>), dim3(blocks), dim3(256), 0, s,
+  const unsigned blocks = export_grid(n, kExportThreads);
+  hipLaunchKernelGGL((export_if_kernel<Pred>), dim3(blocks), dim3(kExportThreads), 0, s,
                      t->view, Pred(), pattern, threshold, offset, n,
                      (unsigned long long*)d_counter, keys, (uint8_t*)values, scores);
 }
@@ -643,8 +642,7 @@ void launch_export(const hkv_table* t, uint64_t pattern, uint64_t threshold,
 template <class Pred>
 void launch_size_if(const hkv_table* t, uint64_t pattern, uint64_t threshold,
                     unsigned long long* d_out, hipStream_t s) {
-  const unsigned blocks =
-      (unsigned)std::min<uint64_t>((t->view.capacity + 255) / 256, 8192);
+  const unsigned blocks = scan_grid(t->view.capacity, 256);
   hipLaunchKernelGGL((size_if_kernel<Pred>), dim3(blocks), dim3(256), 0, s,
                      t->view, Pred(), pattern, threshold, d_out);
 }

@@ -74,63 +74,156 @@ __device__ __forceinline__ void wave_copy_row(uint8_t* dst, const uint8_t* src,
   }
 }
 
-/*
- * export_batch_if: scan slots [offset, offset + n) in slot order, append every
- * entry whose key is not reserved and for which pred(key, score, pattern,
- * threshold) holds.  Output is compact and unordered across wavefronts
- * (same contract as dump_kernel_v2, core_kernels.cuh:983-1041).
+/* ---- compaction shared by the export kernels ---------------------------------------------
  *
- * One slot per lane for the key / score scan; a 64-bit ballot gives the
- * wavefront's match set, one atomic per wavefront reserves the output range,
- * and the wavefront then copies the matched rows cooperatively.
- * `values` and `scores` may be null.
+ * A workgroup scans a chunk of slots, every thread keeping up to kExportPerThread
+ * matches in registers.  The matches of the chunk get consecutive output positions from
+ * ONE atomic on the caller's counter per chunk (atomics on one word serialise on this
+ * memory system, about 15 ns each: one per wavefront made the counter the bottleneck of
+ * the whole export), and the rows are then copied by the whole workgroup from a list of
+ * matched slots in LDS, with streaming loads and stores.  Output order is unspecified,
+ * as with dump_kernel_v2 (core_kernels.cuh:983-1041).
  */
+constexpr int kExportPerThread = 8;
+
+/* exclusive position of this thread's `cnt` matches inside the workgroup's chunk, and the
+ * chunk's total; all threads of the workgroup call it (two barriers) */
+template <int THREADS>
+__device__ __forceinline__ uint32_t block_offsets(uint32_t cnt, uint32_t* s_wave, uint32_t& total) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  uint32_t inc = cnt;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const uint32_t t = __shfl_up(inc, off);
+    if (lane >= off) inc += t;
+  }
+  __syncthreads(); /* s_wave of the previous chunk has been read by everybody */
+  if (lane == kWave - 1) s_wave[wave] = inc;
+  __syncthreads();
+  uint32_t before = 0;
+  total = 0;
+#pragma unroll
+  for (int w = 0; w < THREADS / kWave; w++) {
+    const uint32_t t = s_wave[w];
+    if (w < wave) before += t;
+    total += t;
+  }
+  return before + inc - cnt;
+}
+
+/* rows of the chunk's matches: s_src[r] is the slot (relative to `first_slot`) of match r,
+ * which goes to output row `base + r`; UNIT bytes per thread and trip, 4 trips in flight */
+template <int THREADS, class T>
+__device__ __forceinline__ void export_rows(const hkv_table_view& v, uint64_t first_slot,
+                                            const uint16_t* s_src, uint32_t total,
+                                            unsigned long long base, uint8_t* out_values) {
+  const uint32_t units = v.value_bytes / sizeof(T);
+  const uint32_t tu = total * units;
+  constexpr int kBatch = 4;
+  for (uint32_t idx0 = threadIdx.x; idx0 < tu; idx0 += THREADS * kBatch) {
+    T buf[kBatch];
+    uint32_t row[kBatch], cc[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * THREADS;
+      row[b] = idx / units;
+      cc[b] = idx - row[b] * units;
+      if (idx < tu)
+        buf[b] = __builtin_nontemporal_load(
+            reinterpret_cast<const T*>(value_row(v, first_slot + s_src[row[b]])) + cc[b]);
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; b++) {
+      const uint32_t idx = idx0 + b * THREADS;
+      if (idx < tu)
+        __builtin_nontemporal_store(
+            buf[b], reinterpret_cast<T*>(out_values + (base + row[b]) * v.value_bytes) + cc[b]);
+    }
+  }
+}
+template <int THREADS>
+__device__ __forceinline__ void export_rows_any(const hkv_table_view& v, uint64_t first_slot,
+                                                const uint16_t* s_src, uint32_t total,
+                                                unsigned long long base, uint8_t* out_values) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  const uintptr_t mis = (uintptr_t)out_values | v.value_bytes;
+  if ((mis & 15) == 0)
+    export_rows<THREADS, u32x4_t>(v, first_slot, s_src, total, base, out_values);
+  else if ((mis & 3) == 0)
+    export_rows<THREADS, uint32_t>(v, first_slot, s_src, total, base, out_values);
+  else
+    export_rows<THREADS, uint8_t>(v, first_slot, s_src, total, base, out_values);
+}
+
+/*
+ * export_batch_if: scan slots [offset, offset + n), append every entry whose key is not
+ * reserved and for which pred(key, score, pattern, threshold) holds.  `values` and
+ * `scores` may be null.
+ */
+constexpr int kExportThreads = 256;
 template <class Pred>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kExportThreads)
 export_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern,
                  uint64_t threshold, uint64_t offset, uint64_t n,
                  unsigned long long* counter, uint64_t* out_keys,
                  uint8_t* out_values, uint64_t* out_scores) {
-  const int lane = lane_id();
-  const uint64_t wave_global =
-      ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
-  const uint64_t waves_total = ((uint64_t)gridDim.x * blockDim.x) / kWave;
-  const uint64_t chunks = (n + kWave - 1) / kWave;
-  for (uint64_t c = wave_global; c < chunks; c += waves_total) {
-    const uint64_t i = c * kWave + lane;
-    uint64_t slot = offset + i;
-    uint64_t key = v.empty_key;
-    uint64_t score = 0;
-    bool match = false;
-    if (i < n) {
-      key = v.keys[slot];
-      score = v.scores[slot];
-      match = !is_reserved_key(v, key) && pred(key, score, pattern, threshold);
-    }
-    const unsigned long long vote = __ballot(match);
-    if (vote == 0) continue;
-    const int cnt = __popcll(vote);
-    unsigned long long base = 0;
-    if (lane == 0) base = atomicAdd(counter, (unsigned long long)cnt);
-    base = __shfl(base, 0);
-    const int rank = __popcll(vote & ((1ull << lane) - 1));
-    if (match) {
-      out_keys[base + rank] = key;
-      if (out_scores) out_scores[base + rank] = score;
-    }
-    if (out_values) {
-      unsigned long long rest = vote;
-      int r = 0;
-      while (rest) {
-        const int src_lane = __ffsll(rest) - 1;
-        rest &= rest - 1;
-        const uint64_t s = offset + c * kWave + src_lane;
-        wave_copy_row(out_values + (base + r) * v.value_bytes, value_row(v, s),
-                      v.value_bytes, lane);
-        r++;
+  constexpr int kChunk = kExportThreads * kExportPerThread;
+  __shared__ uint16_t s_src[kChunk];
+  __shared__ uint32_t s_wave[kExportThreads / kWave];
+  __shared__ unsigned long long s_base;
+  const int tid = threadIdx.x;
+  const uint64_t chunks = (n + kChunk - 1) / kChunk;
+  for (uint64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    const uint64_t cbase = c * kChunk;
+    uint64_t key[kExportPerThread], score[kExportPerThread];
+#pragma unroll
+    for (int r = 0; r < kExportPerThread; r++) {
+      const uint64_t i = cbase + (uint64_t)r * kExportThreads + tid;
+      key[r] = v.empty_key;
+      score[r] = 0;
+      if (i < n) {
+        key[r] = v.keys[offset + i];
+        score[r] = v.scores[offset + i];
       }
     }
+    uint32_t mask = 0;
+#pragma unroll
+    for (int r = 0; r < kExportPerThread; r++)
+      if (!is_reserved_key(v, key[r]) && pred(key[r], score[r], pattern, threshold)) mask |= 1u << r;
+    uint32_t total;
+    uint32_t at = block_offsets<kExportThreads>((uint32_t)__popc(mask), s_wave, total);
+    if (total == 0) continue; /* the same for the whole workgroup */
+    if (tid == 0) s_base = atomicAdd(counter, (unsigned long long)total);
+    {
+      uint32_t a = at;
+#pragma unroll
+      for (int r = 0; r < kExportPerThread; r++)
+        if (mask & (1u << r)) s_src[a++] = (uint16_t)(r * kExportThreads + tid);
+    }
+    __syncthreads();
+    const unsigned long long base = s_base;
+#pragma unroll
+    for (int r = 0; r < kExportPerThread; r++) {
+      if (mask & (1u << r)) {
+        out_keys[base + at] = key[r];
+        if (out_scores) out_scores[base + at] = score[r];
+        at++;
+      }
+    }
+    if (out_values) export_rows_any<kExportThreads>(v, offset + cbase, s_src, total, base, out_values);
+    __syncthreads(); /* s_src and s_base are reused by the next chunk */
   }
+}
+
+/* sum of `local` over the workgroup, one atomic per workgroup */
+__device__ __forceinline__ void block_count(uint64_t local, unsigned long long* counter) {
+  __shared__ unsigned long long s_sum;
+  if (threadIdx.x == 0) s_sum = 0;
+  __syncthreads();
+  for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
+  if (lane_id() == 0 && local) atomicAdd(&s_sum, (unsigned long long)local);
+  __syncthreads();
+  if (threadIdx.x == 0 && s_sum) atomicAdd(counter, s_sum);
 }
 
 /* size_if: number of entries satisfying the predicate (size_if_kernel,
@@ -139,7 +232,6 @@ template <class Pred>
 __global__ void __launch_bounds__(256)
 size_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern,
                uint64_t threshold, unsigned long long* counter) {
-  const int lane = lane_id();
   uint64_t local = 0;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t s = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -148,8 +240,7 @@ size_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern,
     uint64_t score = v.scores[s];
     if (!is_reserved_key(v, key) && pred(key, score, pattern, threshold)) local++;
   }
-  for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
-  if (lane == 0 && local) atomicAdd(counter, (unsigned long long)local);
+  block_count(local, counter);
 }
 
 /* erase_if: tombstone every entry the predicate selects (the predicate form of
@@ -159,7 +250,6 @@ template <class Pred>
 __global__ void __launch_bounds__(256)
 erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshold,
                 unsigned long long* counter) {
-  const int lane = lane_id();
   uint64_t local = 0;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t s = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -174,8 +264,7 @@ erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshol
       local++;
     }
   }
-  for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
-  if (lane == 0 && local) atomicAdd(counter, (unsigned long long)local);
+  block_count(local, counter);
 }
 
 /*
@@ -254,38 +343,63 @@ traverse_kernel(hkv_table_view v, uint64_t n, uint64_t offset, Func f) {
 }
 
 /* dump_kernel with a functor, core_kernels.cuh:1043-1112 (export_batch_if_v2):
- * the functor alone decides, reserved keys included */
+ * the functor alone decides, reserved keys included.  The tiles evaluate the functor slot
+ * by slot; the matches of a chunk are then compacted as in export_if_kernel. */
+constexpr int kExportV2Threads = 128;
 template <class K, class V, class S, class Pred, unsigned GroupSize>
-__global__ void __launch_bounds__(128)
+__global__ void __launch_bounds__(kExportV2Threads)
 export_if_v2_kernel(hkv_table_view v, uint64_t n, uint64_t offset, Pred pred,
                     unsigned long long* counter, K* out_keys, V* out_values, S* out_scores) {
+  constexpr int kChunk = kExportV2Threads * kExportPerThread;
+  __shared__ uint16_t s_src[kChunk];
+  __shared__ uint32_t s_wave[kExportV2Threads / kWave];
+  __shared__ unsigned long long s_base;
   coop::thread_block_tile<GroupSize> g(coop::tiled_partition<GroupSize>(coop::this_thread_block()));
-  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  const uint32_t dim = v.value_bytes / sizeof(V);
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-    const uint64_t slot = i + offset;
-    const K key = static_cast<K>(v.keys[slot]);
-    const S score = static_cast<S>(v.scores[slot]);
-    const V* value = reinterpret_cast<const V*>(value_row(v, slot));
-    const bool match = pred.template operator()<GroupSize>(key, value, score, g);
-    const unsigned long long vote = g.ballot(match);
-    const int cnt = __popcll(vote);
-    unsigned long long base = 0;
-    if (g.thread_rank() == 0 && cnt) base = atomicAdd(counter, (unsigned long long)cnt);
-    base = g.shfl(base, 0);
-    const int before = __popcll(vote & ((1ull << g.thread_rank()) - 1));
-    if (match) {
-      out_keys[base + before] = key;
-      if (out_scores) out_scores[base + before] = score;
+  const int tid = threadIdx.x;
+  const uint64_t chunks = (n + kChunk - 1) / kChunk;
+  for (uint64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    const uint64_t cbase = c * kChunk;
+    uint64_t key[kExportPerThread], score[kExportPerThread];
+    uint32_t mask = 0;
+#pragma unroll
+    for (int r = 0; r < kExportPerThread; r++) {
+      const uint64_t i = cbase + (uint64_t)r * kExportV2Threads + tid;
+      key[r] = 0;
+      score[r] = 0;
+      /* the caller picks GroupSize so that n is a multiple of it: a tile is inside or outside */
+      if (i < n) {
+        const uint64_t slot = offset + i;
+        key[r] = v.keys[slot];
+        score[r] = v.scores[slot];
+        const V* value = reinterpret_cast<const V*>(value_row(v, slot));
+        if (pred.template operator()<GroupSize>(static_cast<K>(key[r]), value,
+                                                static_cast<S>(score[r]), g))
+          mask |= 1u << r;
+      }
     }
-    for (unsigned r = 0; r < GroupSize; r++) {
-      if (!((vote >> r) & 1ull)) continue;
-      const int bias = __popcll(vote & ((1ull << r) - 1));
-      const uint64_t cur = (i / GroupSize) * GroupSize + r + offset;
-      const V* src = reinterpret_cast<const V*>(value_row(v, cur));
-      for (uint32_t d = g.thread_rank(); d < dim; d += GroupSize)
-        out_values[(base + bias) * dim + d] = src[d];
+    uint32_t total;
+    uint32_t at = block_offsets<kExportV2Threads>((uint32_t)__popc(mask), s_wave, total);
+    if (total == 0) continue;
+    if (tid == 0) s_base = atomicAdd(counter, (unsigned long long)total);
+    {
+      uint32_t a = at;
+#pragma unroll
+      for (int r = 0; r < kExportPerThread; r++)
+        if (mask & (1u << r)) s_src[a++] = (uint16_t)(r * kExportV2Threads + tid);
     }
+    __syncthreads();
+    const unsigned long long base = s_base;
+#pragma unroll
+    for (int r = 0; r < kExportPerThread; r++) {
+      if (mask & (1u << r)) {
+        out_keys[base + at] = static_cast<K>(key[r]);
+        if (out_scores) out_scores[base + at] = static_cast<S>(score[r]);
+        at++;
+      }
+    }
+    export_rows_any<kExportV2Threads>(v, offset + cbase, s_src, total, base,
+                                      reinterpret_cast<uint8_t*>(out_values));
+    __syncthreads();
   }
 }
 
@@ -295,6 +409,7 @@ __global__ void __launch_bounds__(128)
 erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* counter) {
   coop::thread_block_tile<GroupSize> g(coop::tiled_partition<GroupSize>(coop::this_thread_block()));
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  uint64_t local = 0;
   for (uint64_t slot = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; slot < n; slot += stride) {
     const uint64_t raw = v.keys[slot];
     const K key = static_cast<K>(raw);
@@ -302,19 +417,25 @@ erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* 
     const V* value = reinterpret_cast<const V*>(value_row(v, slot));
     bool match = pred.template operator()<GroupSize>(key, value, score, g);
     if (is_reserved_key(v, raw)) match = false;
-    const unsigned long long vote = g.ballot(match);
-    const int cnt = __popcll(vote);
-    /* GroupSize divides 128, so the slots of a tile share a bucket */
-    if (g.thread_rank() == 0 && cnt) {
-      atomicAdd(counter, (unsigned long long)cnt);
-      atomicSub(v.sizes + (slot >> 7), cnt);
-    }
     if (match) {
       v.digests[slot] = v.reclaim_digest;
       v.keys[slot] = v.reclaim_key;
       v.scores[slot] = 0;
+      atomicSub(v.sizes + (slot >> 7), 1);
+      local++;
     }
   }
+  block_count(local, counter);
+}
+
+/* launch shapes of the scans above */
+inline unsigned export_grid(uint64_t n, int threads) {
+  const uint64_t chunks = (n + (uint64_t)threads * kExportPerThread - 1) / ((uint64_t)threads * kExportPerThread);
+  return (unsigned)(chunks < 4096 ? (chunks ? chunks : 1) : 4096);
+}
+inline unsigned scan_grid(uint64_t slots, int threads) {
+  const uint64_t blocks = (slots + threads - 1) / threads;
+  return (unsigned)(blocks < 2048 ? (blocks ? blocks : 1) : 2048);
 }
 
 /* One-word clear as a kernel: callers may be capturing a graph, where memset

@@ -605,8 +605,7 @@ class HashTable : public HashTableBase<K, V, S> {
                        d_count);
     {
       detail::RoleGuard g(table_, 2, stream);
-      const unsigned blocks =
-          static_cast<unsigned>(std::min<uint64_t>((v.capacity + 255) / 256, 16384));
+      const unsigned blocks = hkv::scan_grid(v.capacity, 256);
       hipLaunchKernelGGL((hkv::erase_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
                          dim3(blocks), dim3(256), 0, stream, v,
                          detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
@@ -633,7 +632,7 @@ class HashTable : public HashTableBase<K, V, S> {
     {
       detail::RoleGuard g(table_, 2, stream);
       const uint64_t n = v.capacity;
-      const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
+      const unsigned blocks = hkv::scan_grid(n, 128);
       const uint64_t dim = options_.dim;
       if (dim >= 32 && n % 32 == 0)
         hipLaunchKernelGGL((hkv::erase_if_v2_kernel<K, V, S, PredFunctor, 32>), dim3(blocks),
@@ -668,7 +667,7 @@ class HashTable : public HashTableBase<K, V, S> {
     if (offset >= v.capacity) return;
     n = std::min<size_type>(v.capacity - offset, n);
     if (n == 0) return;
-    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
+    const unsigned blocks = hkv::export_grid(n, hkv::kExportV2Threads);
     const uint64_t dim = options_.dim;
     auto* cnt = reinterpret_cast<unsigned long long*>(d_counter);
     if (dim >= 32 && n % 32 == 0)
@@ -749,8 +748,7 @@ class HashTable : public HashTableBase<K, V, S> {
     if (offset >= v.capacity) return;
     n = std::min<size_type>(v.capacity - offset, n);
     if (n == 0) return;
-    const uint64_t waves = (n + hkv::kWave - 1) / hkv::kWave;
-    const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((waves + 3) / 4, 16384));
+    const unsigned blocks = hkv::export_grid(n, hkv::kExportThreads);
     hipLaunchKernelGGL((hkv::export_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
                        dim3(blocks), dim3(256), 0, stream, v,
                        detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
@@ -772,8 +770,7 @@ class HashTable : public HashTableBase<K, V, S> {
                        d_count);
     {
       detail::RoleGuard g(table_, 0, stream);
-      const unsigned blocks =
-          static_cast<unsigned>(std::min<uint64_t>((v.capacity + 255) / 256, 8192));
+      const unsigned blocks = hkv::scan_grid(v.capacity, 256);
       hipLaunchKernelGGL((hkv::size_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
                          dim3(blocks), dim3(256), 0, stream, v,
                          detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
