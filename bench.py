@@ -265,6 +265,10 @@ def run_matrix(args, np, torch, dev):
             "insert_and_evict", "export_batch", "export_batch_if", "contains"]
     order = ["find", "find*", "contains", "export_batch", "export_batch_if", "assign",
              "find_or_insert", "find_or_insert*", "insert_or_assign", "insert_and_evict"]
+    if args.matrix_hybrid:
+        # insert_and_evict needs a pure-HBM table, as in the reference (merlin_hashtable.cuh:1373-1375)
+        apis.remove("insert_and_evict")
+        order.remove("insert_and_evict")
 
     def d64(a):
         return torch.from_numpy(a.view(np.int64)).to(dev)
