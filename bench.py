@@ -67,6 +67,10 @@ def main():
                     help="instead of the one-line benchmark: the reference's own benchmark table "
                          "(README.md:245-317, benchmark/merlin_hashtable_benchmark.cc.cu), every API "
                          "at load factor 0.50 / 0.75 / 1.00 for dim 8, 32 and 64, printed as markdown")
+    ap.add_argument("--ops", action="store_true",
+                    help="instead of the one-line benchmark: every entry point at the metric shape "
+                         "(capacity 2^26, dim 64, batch 2^20, load factor 1.0), kernel time by HIP "
+                         "events and algorithmic GB/s against the 8 TB/s peak, printed as markdown")
     ap.add_argument("--matrix-hybrid", action="store_true",
                     help="with --matrix: the hybrid table of README.md:289-303 (dim 64, capacity "
                          "128M, 16 GB of the rows in HBM, the rest in pinned host memory)")
@@ -87,6 +91,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.matrix:
         run_matrix(args, np, torch, dev)
+        return
+    if args.ops:
+        run_ops(args, np, torch, dev, w)
         return
     cap = 1 << args.capacity_log2
     dim = args.dim
@@ -345,6 +352,106 @@ def run_matrix(args, np, torch, dev):
             table.close()
             del table, vals, defv
             torch.cuda.empty_cache()
+
+
+def run_ops(args, np, torch, dev, w):
+    """Every entry point at the metric shape, one row each: average HIP-event time of 6 calls
+    after 2 warm-up calls, 10^9 KV/s, algorithmic bytes per key and their rate against the
+    8 TB/s peak.  Bytes per key, VB = 256: find hit 145 + 2 VB; find* hit 153; contains hit 145;
+    upsert hit 161 + 2 VB, upsert into a full bucket 1185 + 2 VB; find_or_insert hit 169 + 2 VB;
+    insert_and_evict evicting 1201 + 4 VB; accum hit 161 + 3 VB; assign hit 161 + 2 VB;
+    export 16 per scanned slot + (2 VB + 16) per match; erase hit 165."""
+    from hierarchicalkv_amd import EvictStrategy, HashTable, default_options, Predicate
+
+    cap, dim, n = 1 << args.capacity_log2, args.dim, 1 << args.batch_log2
+    vb = dim * 4
+    seed = 0x484B5600
+    table = HashTable()
+    table.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb,
+                               dim=dim, evict_strategy=EvictStrategy.kLru))
+
+    def d64(a):
+        return torch.from_numpy(a.view(np.int64)).to(dev)
+
+    vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
+    pos, starts, size = 0, [], 0
+    while size < 0.999 * cap and pos < 3 * cap:
+        for _ in range(max(1, (cap // n) // 8)):
+            table.insert_or_assign(n, d64(w.unique_keys(seed, pos, n)), vals)
+            starts.append(pos)
+            pos += n
+        size = table.size()
+    nb = len(starts)
+    out = torch.empty(n, dim, dtype=torch.float32, device=dev)
+    ev_vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
+    founds = torch.empty(n, dtype=torch.bool, device=dev)
+    flags = torch.empty(n, dtype=torch.bool, device=dev)
+    ptrs = torch.zeros(n, dtype=torch.int64, device=dev)
+    ek = torch.zeros(n, dtype=torch.int64, device=dev)
+    es = torch.zeros(n, dtype=torch.int64, device=dev)
+    cnt = torch.zeros(1, dtype=torch.int64, device=dev)
+    state = {"old": 0, "pos": pos}
+
+    def resident():
+        # an old pre-fill batch that is still resident and cold in the caches: the batches 8 to 31
+        # from the end take turns (the table holds the newest ~64, and every upsert row below
+        # pushes out half a batch)
+        state["old"] += 1
+        return w.unique_keys(seed, starts[nb - 8 - state["old"] % 24], n)
+
+    def mixed(new_fraction=0.5):
+        m = int(n * new_fraction)
+        fresh = w.unique_keys(seed, state["pos"], m)
+        state["pos"] += m
+        return np.concatenate([resident()[: n - m], fresh])
+
+    hit, full = 161 + 2 * vb, 1185 + 2 * vb
+    rows = [
+        ("find (100 % hit)", lambda k: table.find(n, k, out, founds), resident, 145 + 2 * vb),
+        ("find* (100 % hit)", lambda k: table.find_ptr(n, k, ptrs, founds), resident, 153),
+        ("contains (100 % hit)", lambda k: table.contains(n, k, founds), resident, 145),
+        ("assign (100 % hit)", lambda k: table.assign(n, k, vals), resident, hit),
+        ("insert_or_assign (50 % new)", lambda k: table.insert_or_assign(n, k, vals), mixed,
+         0.5 * hit + 0.5 * full),
+        ("find_or_insert (50 % new)", lambda k: table.find_or_insert(n, k, out), mixed,
+         0.5 * (169 + 2 * vb) + 0.5 * full),
+        ("find_or_insert* (50 % new)", lambda k: table.find_or_insert_ptr(n, k, ptrs, founds), mixed,
+         0.5 * 177 + 0.5 * (1185 + 16)),
+        ("insert_and_evict (50 % new)",
+         lambda k: (cnt.zero_(), table.insert_and_evict(n, k, vals, None, ek, ev_vals, es, cnt)), mixed,
+         0.5 * hit + 0.5 * (1201 + 4 * vb)),
+        ("accum_or_assign (50 % new, flags from find)", None, mixed, 0.5 * (161 + 3 * vb) + 0.5 * (full + 1)),
+        ("export_batch_if (2^20 slots, all match)",
+         lambda k: table.export_batch_if(Predicate.kAlways, 0, 0, n, (state["old"] % 32) * n, cnt, ek, out, es),
+         resident, 16 + 2 * vb + 16),
+        ("erase (100 % hit)", lambda k: table.erase(n, k), resident, 165),
+    ]
+    print("| call | ms per 2^20 keys | 10^9 KV/s | algorithmic bytes per key | algorithmic GB/s | fraction of 8 TB/s |")
+    print("|---|---|---|---|---|---|")
+    for name, fn, gen, bpk in rows:
+        times = []
+        for rep in range(8):
+            k = d64(gen())
+            if fn is None:  # accum_or_assign: the flags say which keys are there (as config 5 does)
+                table.find(n, k, out, flags)
+                torch.cuda.synchronize()
+                call = lambda: table.accum_or_assign(n, k, vals, flags)
+            else:
+                call = lambda: fn(k)
+            torch.cuda.synchronize()
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            call()
+            b.record()
+            torch.cuda.synchronize()
+            if rep >= 2:
+                times.append(a.elapsed_time(b))
+        ms = sum(times) / len(times)
+        gbs = bpk * n / (ms * 1e-3) / 1e9
+        print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f |" % (name, ms, n / ms / 1e6, bpk, gbs, gbs / HBM_PEAK_GBS),
+              flush=True)
+    table.close()
 
 
 def cpu_baseline(args, np, w):
