@@ -438,6 +438,16 @@ inline unsigned scan_grid(uint64_t slots, int threads) {
   return (unsigned)(blocks < 2048 ? (blocks ? blocks : 1) : 2048);
 }
 
+/* 32-bit score arrays of the caller <-> the table's 64-bit scores (zero-extended) */
+__global__ void widen_scores_kernel(const uint32_t* in, uint64_t* out, uint64_t n) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = in[i];
+}
+__global__ void narrow_scores_kernel(const uint64_t* in, uint32_t* out, uint64_t n) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = (uint32_t)in[i];
+}
+
 /* One-word clear as a kernel: callers may be capturing a graph, where memset
  * nodes are best avoided. */
 template <class T>

@@ -24,7 +24,9 @@
  * the export family, as in the reference; the calls the reference guards throw
  * the same way, and assign, find*, lock_keys / unlock_keys / find_and_update
  * (unguarded but single-bucket in the reference) throw too.
- * Not provided: S = uint32_t (static_assert).
+ * S = uint32_t (Customized strategy only, as in the reference) is served by widening and
+ * narrowing the caller's score arrays around each call: the table keeps 64-bit scores, and
+ * such calls allocate a temporary buffer on the stream.
  */
 #ifndef MERLIN_HASHTABLE_HPP_
 #define MERLIN_HASHTABLE_HPP_
@@ -350,6 +352,66 @@ constexpr int value_kind_of() {
   return HKV_VALUE_BYTES;
 }
 
+/* Score arrays at the boundary.  The C ABI speaks 64-bit scores; for S = uint64_t these
+ * wrappers are the caller's pointer, for S = uint32_t a temporary 64-bit array on the
+ * stream that is filled from / written back to the caller's 32-bit array. */
+template <class S>
+struct ScoresIn {
+  const uint64_t* p;
+  ScoresIn(const S* s, size_t, hipStream_t) : p(s) {}
+  const uint64_t* get() const { return p; }
+};
+template <>
+struct ScoresIn<uint32_t> {
+  uint64_t* tmp = nullptr;
+  hipStream_t st;
+  ScoresIn(const uint32_t* s, size_t n, hipStream_t stream) : st(stream) {
+    if (s == nullptr || n == 0) return;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&tmp), n * sizeof(uint64_t), st));
+    hipLaunchKernelGGL(hkv::widen_scores_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
+                       dim3(256), 0, st, s, tmp, static_cast<uint64_t>(n));
+  }
+  ~ScoresIn() {
+    if (tmp) (void)hipFreeAsync(tmp, st);
+  }
+  ScoresIn(const ScoresIn&) = delete;
+  ScoresIn& operator=(const ScoresIn&) = delete;
+  const uint64_t* get() const { return tmp; }
+};
+template <class S>
+struct ScoresOut {
+  uint64_t* p;
+  ScoresOut(S* s, size_t, hipStream_t) : p(s) {}
+  uint64_t* get() const { return p; }
+  void finish() {}
+};
+template <>
+struct ScoresOut<uint32_t> {
+  uint32_t* dst;
+  uint64_t* tmp = nullptr;
+  size_t n;
+  hipStream_t st;
+  /* starts from the caller's contents: entries a call leaves untouched (keys not found)
+   * come back unchanged */
+  ScoresOut(uint32_t* s, size_t n_, hipStream_t stream) : dst(s), n(n_), st(stream) {
+    if (s == nullptr || n == 0) return;
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&tmp), n * sizeof(uint64_t), st));
+    hipLaunchKernelGGL(hkv::widen_scores_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
+                       dim3(256), 0, st, s, tmp, static_cast<uint64_t>(n));
+  }
+  ~ScoresOut() {
+    if (tmp) (void)hipFreeAsync(tmp, st);
+  }
+  ScoresOut(const ScoresOut&) = delete;
+  ScoresOut& operator=(const ScoresOut&) = delete;
+  uint64_t* get() const { return tmp; }
+  void finish() {
+    if (tmp)
+      hipLaunchKernelGGL(hkv::narrow_scores_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
+                         dim3(256), 0, st, tmp, dst, static_cast<uint64_t>(n));
+  }
+};
+
 /* the caller's functor sees K and S; the kernel works on the 64-bit patterns */
 template <class K, class S, template <typename, typename> class PredFunctor>
 struct PredAdapter {
@@ -409,8 +471,11 @@ class HashTable : public HashTableBase<K, V, S> {
 
   static_assert(std::is_same<K, int64_t>::value || std::is_same<K, uint64_t>::value,
                 "The key_type must be int64_t or uint64_t.");
-  static_assert(std::is_same<S, uint64_t>::value,
-                "The score_type must be uint64_t (uint32_t scores are not supported).");
+  static_assert(std::is_same<S, uint64_t>::value || std::is_same<S, uint32_t>::value,
+                "The score_type must be uint64_t or uint32_t.");
+  /* merlin_hashtable.cuh:944-949 */
+  static_assert(std::is_same<S, uint64_t>::value || Strategy == EvictStrategy::kCustomized,
+                "The uint32_t score_type is only supported with EvictStrategy::kCustomized.");
   static_assert(std::is_trivially_copyable<V>::value, "value_type must be trivially copyable");
   static_assert(sizeof(size_type) == sizeof(uint64_t), "size_type must be 64 bits wide");
 
@@ -454,7 +519,7 @@ class HashTable : public HashTableBase<K, V, S> {
     o.evict_strategy = Strategy;
     o.value_kind = detail::value_kind_of<V>();
     o.value_size = sizeof(V);
-    o.score_size = sizeof(S);
+    o.score_size = sizeof(uint64_t); /* the table's own width; 32-bit scores are widened at the calls */
     default_allocator_ = (allocator == nullptr);
     allocator_ = default_allocator_ ? nullptr : allocator;
     if (allocator_ != nullptr) {
@@ -470,7 +535,8 @@ class HashTable : public HashTableBase<K, V, S> {
   void insert_or_assign(const size_type n, const key_type* keys, const value_type* values,
                         const score_type* scores = nullptr, hipStream_t stream = 0,
                         bool unique_key = true, bool ignore_evict_strategy = false) override {
-    throw_on_error_(hkv_insert_or_assign(table_, n, u64(keys), values, scores, stream, unique_key,
+    detail::ScoresIn<S> sc(scores, n, stream);
+    throw_on_error_(hkv_insert_or_assign(table_, n, u64(keys), values, sc.get(), stream, unique_key,
                                          ignore_evict_strategy));
   }
 
@@ -479,10 +545,13 @@ class HashTable : public HashTableBase<K, V, S> {
                         value_type* evicted_values, score_type* evicted_scores,
                         size_type* d_evicted_counter, hipStream_t stream = 0,
                         bool unique_key = true, bool ignore_evict_strategy = false) override {
-    throw_on_error_(hkv_insert_and_evict(table_, n, u64(keys), values, scores, u64(evicted_keys),
-                                         evicted_values, evicted_scores,
+    detail::ScoresIn<S> sc(scores, n, stream);
+    detail::ScoresOut<S> es(evicted_scores, n, stream);
+    throw_on_error_(hkv_insert_and_evict(table_, n, u64(keys), values, sc.get(), u64(evicted_keys),
+                                         evicted_values, es.get(),
                                          reinterpret_cast<uint64_t*>(d_evicted_counter), stream,
                                          unique_key, ignore_evict_strategy));
+    es.finish();
   }
 
   size_type insert_and_evict(const size_type n, const key_type* keys, const value_type* values,
@@ -491,24 +560,30 @@ class HashTable : public HashTableBase<K, V, S> {
                              hipStream_t stream = 0, bool unique_key = true,
                              bool ignore_evict_strategy = false) override {
     uint64_t cnt = 0;
-    throw_on_error_(hkv_insert_and_evict_count(table_, n, u64(keys), values, scores,
-                                               u64(evicted_keys), evicted_values, evicted_scores,
+    detail::ScoresIn<S> sc(scores, n, stream);
+    detail::ScoresOut<S> es(evicted_scores, n, stream);
+    throw_on_error_(hkv_insert_and_evict_count(table_, n, u64(keys), values, sc.get(),
+                                               u64(evicted_keys), evicted_values, es.get(),
                                                stream, unique_key, ignore_evict_strategy, &cnt));
+    es.finish();
+    if (!std::is_same<S, uint64_t>::value) HKV_HIP_CHECK(hipStreamSynchronize(stream));
     return static_cast<size_type>(cnt);
   }
 
   void accum_or_assign(const size_type n, const key_type* keys, const value_type* value_or_deltas,
                        const bool* accum_or_assigns, const score_type* scores = nullptr,
                        hipStream_t stream = 0, bool ignore_evict_strategy = false) override {
+    detail::ScoresIn<S> sc(scores, n, stream);
     throw_on_error_(hkv_accum_or_assign(table_, n, u64(keys), value_or_deltas,
-                                        reinterpret_cast<const uint8_t*>(accum_or_assigns), scores,
+                                        reinterpret_cast<const uint8_t*>(accum_or_assigns), sc.get(),
                                         stream, ignore_evict_strategy));
   }
 
   void find_or_insert(const size_type n, const key_type* keys, value_type* values,
                       score_type* scores = nullptr, hipStream_t stream = 0,
                       bool unique_key = true, bool ignore_evict_strategy = false) override {
-    throw_on_error_(hkv_find_or_insert(table_, n, u64(keys), values, scores, stream, unique_key,
+    detail::ScoresIn<S> sc(scores, n, stream);
+    throw_on_error_(hkv_find_or_insert(table_, n, u64(keys), values, sc.get(), stream, unique_key,
                                        ignore_evict_strategy));
   }
 
@@ -518,8 +593,9 @@ class HashTable : public HashTableBase<K, V, S> {
                       key_type** locked_key_ptrs = nullptr) override {
     if (locked_key_ptrs != nullptr)
       throw std::runtime_error("find_or_insert with locked_key_ptrs is not supported");
+    detail::ScoresIn<S> sc(scores, n, stream);
     throw_on_error_(hkv_find_or_insert_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
-                                           reinterpret_cast<uint8_t*>(founds), scores, stream,
+                                           reinterpret_cast<uint8_t*>(founds), sc.get(), stream,
                                            unique_key, ignore_evict_strategy));
   }
 
@@ -527,9 +603,10 @@ class HashTable : public HashTableBase<K, V, S> {
   void lock_keys(const size_type n, key_type const* keys, key_type** locked_key_ptrs,
                  bool* succeededs = nullptr, hipStream_t stream = 0,
                  score_type const* scores = nullptr) override {
+    detail::ScoresIn<S> sc(scores, n, stream);
     throw_on_error_(hkv_lock_keys(table_, n, u64(keys),
                                   reinterpret_cast<uint64_t**>(locked_key_ptrs),
-                                  reinterpret_cast<uint8_t*>(succeededs), scores, stream));
+                                  reinterpret_cast<uint8_t*>(succeededs), sc.get(), stream));
   }
   /* merlin_hashtable.cuh:2026-2044 */
   void unlock_keys(const size_type n, key_type** locked_key_ptrs, const key_type* keys,
@@ -541,11 +618,13 @@ class HashTable : public HashTableBase<K, V, S> {
   void assign(const size_type n, const key_type* keys, const value_type* values,
               const score_type* scores = nullptr, hipStream_t stream = 0,
               bool unique_key = true) override {
-    throw_on_error_(hkv_assign(table_, n, u64(keys), values, scores, stream, unique_key));
+    detail::ScoresIn<S> sc(scores, n, stream);
+    throw_on_error_(hkv_assign(table_, n, u64(keys), values, sc.get(), stream, unique_key));
   }
   void assign_scores(const size_type n, const key_type* keys, const score_type* scores = nullptr,
                      hipStream_t stream = 0, bool unique_key = true) override {
-    throw_on_error_(hkv_assign_scores(table_, n, u64(keys), scores, stream, unique_key));
+    detail::ScoresIn<S> sc(scores, n, stream);
+    throw_on_error_(hkv_assign_scores(table_, n, u64(keys), sc.get(), stream, unique_key));
   }
   /* alias of assign_scores (merlin_hashtable.cuh:2285-2290) */
   void assign(const size_type n, const key_type* keys, const score_type* scores = nullptr,
@@ -559,20 +638,26 @@ class HashTable : public HashTableBase<K, V, S> {
 
   void find(const size_type n, const key_type* keys, value_type* values, bool* founds,
             score_type* scores = nullptr, hipStream_t stream = 0) const override {
+    detail::ScoresOut<S> so(scores, n, stream);
     throw_on_error_(hkv_find(table_, n, u64(keys), values, reinterpret_cast<uint8_t*>(founds),
-                             scores, stream));
+                             so.get(), stream));
+    so.finish();
   }
   void find(const size_type n, const key_type* keys, value_type* values, key_type* missed_keys,
             int* missed_indices, int* missed_size, score_type* scores = nullptr,
             hipStream_t stream = 0) const override {
+    detail::ScoresOut<S> so(scores, n, stream);
     throw_on_error_(hkv_find_missed(table_, n, u64(keys), values, u64(missed_keys), missed_indices,
-                                    missed_size, scores, stream));
+                                    missed_size, so.get(), stream));
+    so.finish();
   }
   void find(const size_type n, const key_type* keys, value_type** values, bool* founds,
             score_type* scores = nullptr, hipStream_t stream = 0,
             bool unique_key = true) const override {
+    detail::ScoresOut<S> so(scores, n, stream);
     throw_on_error_(hkv_find_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
-                                 reinterpret_cast<uint8_t*>(founds), scores, stream, unique_key));
+                                 reinterpret_cast<uint8_t*>(founds), so.get(), stream, unique_key));
+    so.finish();
   }
   /* merlin_hashtable.cuh:2811-2843 */
   void find_and_update(const size_type n, const key_type* keys, value_type** values, bool* founds,
@@ -581,8 +666,10 @@ class HashTable : public HashTableBase<K, V, S> {
     if (!unique_key)
       throw std::runtime_error(
           "Not support update score when keys are not unique or bucket capacity is small.");
+    detail::ScoresIn<S> sc(scores, n, stream);
     throw_on_error_(hkv_find_and_update(table_, n, u64(keys), reinterpret_cast<void**>(values),
-                                        reinterpret_cast<uint8_t*>(founds), scores, stream));
+                                        reinterpret_cast<uint8_t*>(founds),
+                                        const_cast<uint64_t*>(sc.get()), stream));
   }
   void contains(const size_type n, const key_type* keys, bool* founds,
                 hipStream_t stream = 0) const override {
@@ -717,8 +804,10 @@ class HashTable : public HashTableBase<K, V, S> {
   void export_batch(size_type n, const size_type offset, size_type* d_counter, key_type* keys,
                     value_type* values, score_type* scores = nullptr,
                     hipStream_t stream = 0) const override {
+    detail::ScoresOut<S> so(scores, n, stream);
     throw_on_error_(hkv_export_batch(table_, n, offset, reinterpret_cast<uint64_t*>(d_counter),
-                                     u64(keys), values, scores, stream));
+                                     u64(keys), values, so.get(), stream));
+    so.finish();
   }
 
   size_type export_batch(const size_type n, const size_type offset, key_type* keys,
@@ -748,14 +837,16 @@ class HashTable : public HashTableBase<K, V, S> {
     if (offset >= v.capacity) return;
     n = std::min<size_type>(v.capacity - offset, n);
     if (n == 0) return;
+    detail::ScoresOut<S> so(scores, n, stream);
     const unsigned blocks = hkv::export_grid(n, hkv::kExportThreads);
     hipLaunchKernelGGL((hkv::export_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
                        dim3(blocks), dim3(256), 0, stream, v,
                        detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
                        static_cast<uint64_t>(threshold), static_cast<uint64_t>(offset),
                        static_cast<uint64_t>(n), reinterpret_cast<unsigned long long*>(d_counter),
-                       u64(keys), reinterpret_cast<uint8_t*>(values), scores);
+                       u64(keys), reinterpret_cast<uint8_t*>(values), so.get());
     HKV_HIP_CHECK(hipGetLastError());
+    so.finish();
   }
 
   /* merlin_hashtable.cuh:3460-3476.  Synchronises `stream`. */

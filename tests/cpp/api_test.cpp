@@ -777,6 +777,103 @@ static void test_dual_bucket_mode() {
   CHECK(table.size() == 0);
 }
 
+
+// S = uint32_t (tests/uint32_score_test.cc.cu:48-186): find_or_insert + find return the
+// 32-bit scores handed in, missing keys leave the caller's score entries alone,
+// assign_scores + export_batch round-trip, insert_and_evict hands back 32-bit scores.
+static void test_uint32_scores() {
+  using S32 = uint32_t;
+  using Table = HashTable<K, V, S32, EvictStrategy::kCustomized>;
+  constexpr size_t DIM = 16, CAP = 1 << 15, N = 4096;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  Table table;
+  table.init(o);
+  auto keys = random_keys(N, 321);
+  auto vals = values_of(keys, DIM);
+  std::vector<S32> scores(N);
+  for (size_t i = 0; i < N; i++) scores[i] = 1000u + static_cast<S32>(i) * 3u;
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM), dout(N * DIM);
+  DevBuf<S32> ds(N), dso(N);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  table.find_or_insert(N, dk.p, dv.p, ds.p);
+  CHECK(table.size() == N);
+  table.find(N, dk.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  auto f = df.down(N);
+  CHECK(std::all_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  CHECK(dso.down(N) == scores);
+  CHECK(dout.down(N * DIM) == vals);
+  // missing keys: founds false, the score entries keep the caller's sentinel
+  auto missing = random_keys(N, 654);
+  DevBuf<K> dm(N);
+  dm.up(missing);
+  std::vector<S32> sentinel(N, 0xDEADBEEFu);
+  dso.up(sentinel);
+  table.find(N, dm.p, dout.p, df.p, dso.p);
+  HIP(hipDeviceSynchronize());
+  f = df.down(N);
+  CHECK(std::none_of(f.begin(), f.end(), [](uint8_t b) { return b != 0; }));
+  CHECK(dso.down(N) == sentinel);
+  // assign_scores, then export everything
+  for (size_t i = 0; i < N; i++) scores[i] = 500000u + static_cast<S32>(N - i);
+  ds.up(scores);
+  table.assign_scores(N, dk.p, ds.p);
+  DevBuf<K> xk(CAP);
+  DevBuf<V> xv(CAP * DIM);
+  DevBuf<S32> xs(CAP);
+  const size_t dumped = table.export_batch(table.capacity(), 0, xk.p, xv.p, xs.p);
+  CHECK(dumped == N);
+  {
+    std::map<K, S32> want;
+    for (size_t i = 0; i < N; i++) want[keys[i]] = scores[i];
+    auto hk = xk.down(dumped);
+    auto hs = xs.down(dumped);
+    bool ok = true;
+    for (size_t i = 0; i < dumped; i++) {
+      auto it = want.find(hk[i]);
+      ok &= it != want.end() && it->second == hs[i];
+      if (it != want.end()) want.erase(it);
+    }
+    CHECK(ok && want.empty());
+  }
+  // fill one bucket's worth of pressure: insert_and_evict returns 32-bit scores of what left
+  constexpr size_t M = 1 << 15;
+  auto more = random_keys(M, 987);
+  auto mvals = values_of(more, DIM);
+  std::vector<S32> mscores(M);
+  for (size_t i = 0; i < M; i++) mscores[i] = 2000000u + static_cast<S32>(i);
+  DevBuf<K> mk(M), ek(M);
+  DevBuf<V> mv(M * DIM), ev(M * DIM);
+  DevBuf<S32> ms(M), es(M);
+  mk.up(more);
+  mv.up(mvals);
+  ms.up(mscores);
+  const size_t before = table.size();
+  const size_t c = table.insert_and_evict(M, mk.p, mv.p, ms.p, ek.p, ev.p, es.p);
+  CHECK(c + table.size() == before + M);
+  CHECK(c > 0);
+  {
+    std::map<K, S32> old;
+    for (size_t i = 0; i < N; i++) old[keys[i]] = scores[i];
+    for (size_t i = 0; i < M; i++) old[more[i]] = mscores[i];
+    auto hk = ek.down(c);
+    auto hs = es.down(c);
+    bool ok = true;
+    for (size_t i = 0; i < c; i++) ok &= old.count(hk[i]) == 1 && old[hk[i]] == hs[i];
+    CHECK(ok);
+  }
+  // a predicate over 32-bit scores
+  const size_t high = table.size_if<ExportIfPredFunctor>(0, static_cast<S32>(2000000u - 1));
+  CHECK(high > 0 && high <= M);
+}
+
 int main() {
   try {
     test_basic();
@@ -787,6 +884,7 @@ int main() {
     test_growth_and_key_locks();
     test_functor_forms();
     test_dual_bucket_mode();
+    test_uint32_scores();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
