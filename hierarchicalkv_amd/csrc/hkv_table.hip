@@ -23,6 +23,7 @@
 #include "hkv_c_api.h"
 #include "hkv_misc.hpp"
 #include "hkv_upsert.hpp"
+#include "hkv_dedup.hpp"
 #include "hkv_dual.hpp"
 #include "hkv_grouped.hpp"
 #include "hkv_keylocks.hpp"
@@ -598,6 +599,27 @@ int refuse_dual(const hkv_table* t, const char* what, bool guarded) {
               "[MEMORY_MODE] %s is not supported in dual-bucket mode.", what);
 }
 
+/* unique_key == false: the batch is reduced to one occurrence per key first; `keys` then
+ * points at the reduced copy, which lives until the guard goes out of scope (stream-ordered). */
+struct DedupGuard {
+  DedupPlan d;
+  bool on = false;
+  ~DedupGuard() {
+    if (on) dedup_free(d);
+  }
+};
+int maybe_dedup(const hkv_table* t, int unique_key, uint64_t n, const uint64_t*& keys,
+                hipStream_t s, DedupGuard& g) {
+  if (unique_key || n < 2) return HKV_SUCCESS;
+  if (n >= (UINT64_C(1) << 31))
+    return fail(HKV_ERROR_UNSUPPORTED, "unique_key = false needs a batch below 2^31 keys");
+  const hipError_t e = dedup_make(t->view, n, keys, s, g.d);
+  if (e != hipSuccess) return fail(HKV_ERROR_HIP, "duplicate-key pass: %s", hipGetErrorString(e));
+  g.on = true;
+  keys = g.d.keys;
+  return HKV_SUCCESS;
+}
+
 void launch_dual_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   const dim3 grid((unsigned)((a.n + kTilesPerWave - 1) / kTilesPerWave)), block(kWave);
   if (vec == 16)
@@ -868,6 +890,8 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
   if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  DedupGuard dg;
+  if (!t->dual) HKV_TRY(maybe_dedup(t, unique_key, n, keys, (hipStream_t)stream, dg));
   UpsertArgs a{};
   a.keys = keys;
   a.values_in = (const uint8_t*)values;
@@ -906,10 +930,10 @@ int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
   /* merlin_hashtable.cuh:1384-1386 */
   if (!t->pure_hbm)
     return fail(HKV_ERROR_RUNTIME, "Only support pure HBM mode for insert_and_evict.");
-  if (!unique_key)
-    return fail(HKV_ERROR_UNSUPPORTED, "insert_and_evict needs unique keys in a batch");
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
   if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  DedupGuard dg;
+  HKV_TRY(maybe_dedup(t, unique_key, n, keys, (hipStream_t)stream, dg));
   UpsertArgs a{};
   a.keys = keys;
   a.values_in = (const uint8_t*)values;
@@ -965,10 +989,11 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
                        void* values, const uint64_t* scores, hkv_stream_t stream,
                        int unique_key, int ignore) {
   HKV_TRY(refuse_dual(t, "find_or_insert()", true));
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
   if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  DedupGuard dg;
+  HKV_TRY(maybe_dedup(t, unique_key, n, keys, (hipStream_t)stream, dg));
   UpsertArgs a{};
   a.keys = keys;
   a.values_io = (uint8_t*)values;
@@ -976,17 +1001,26 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.n = n;
   a.strategy = strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
-  return run_upsert<kOpFindOrInsert>(t, a, vec, true, (hipStream_t)stream);
+  HKV_TRY(run_upsert<kOpFindOrInsert>(t, a, vec, true, (hipStream_t)stream));
+  if (dg.on) {
+    /* the other occurrences of a key get the row its representative ended up with (what it
+     * read, or what it inserted; a refused key keeps its own row, like its representative) */
+    hipLaunchKernelGGL(dedup_fix_rows_kernel, dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream,
+                       (const uint32_t*)dg.d.rep, n, (uint8_t*)values, t->view.value_bytes);
+    HKV_HIP(hipGetLastError());
+  }
+  return HKV_SUCCESS;
 }
 
 int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
                            void** values, uint8_t* founds, const uint64_t* scores,
                            hkv_stream_t stream, int unique_key, int ignore) {
   HKV_TRY(refuse_dual(t, "find_or_insert()", true));
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
   if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  DedupGuard dg;
+  HKV_TRY(maybe_dedup(t, unique_key, n, keys, (hipStream_t)stream, dg));
   UpsertArgs a{};
   a.keys = keys;
   a.out_ptrs = values;
@@ -994,7 +1028,13 @@ int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.scores = scores;
   a.n = n;
   a.strategy = strategy;
-  return run_upsert<kOpFindOrInsertPtr>(t, a, 16, true, (hipStream_t)stream);
+  HKV_TRY(run_upsert<kOpFindOrInsertPtr>(t, a, 16, true, (hipStream_t)stream));
+  if (dg.on) {
+    hipLaunchKernelGGL(dedup_fix_ptrs_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (const uint32_t*)dg.d.rep, n, values, founds);
+    HKV_HIP(hipGetLastError());
+  }
+  return HKV_SUCCESS;
 }
 
 static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,

@@ -151,7 +151,13 @@ int hkv_table_create_with_allocator(const hkv_options* opts,
 /* HashTable::~HashTable, merlin_hashtable.cuh:953-971.  Synchronous. */
 int hkv_table_destroy(hkv_table* t);
 
-/* HashTable::insert_or_assign, merlin_hashtable.cuh:1125-1305 */
+/* unique_key (here and below): 1 = the caller guarantees that no key occurs twice in the
+ * batch; 0 = keys may repeat: the batch is first reduced to one occurrence per key (device
+ * sort, temporary memory from the stream's pool), as the reference's kernels for such
+ * batches leave every key in the table once.  A dual-bucket table needs 1
+ * (merlin_hashtable.cuh:1167-1169).
+ *
+ * HashTable::insert_or_assign, merlin_hashtable.cuh:1125-1305 */
 int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
                          const void* values, const uint64_t* scores,
                          hkv_stream_t stream, int unique_key,

@@ -483,3 +483,89 @@ def test_lock_keys_unlock_keys_find_and_update(oracle):
         assert (row == vals[i].view(np.uint8)).all()
     assert_same_table(t, o, dim * 4)
     t.close()
+
+
+def test_batches_with_repeated_keys(oracle):
+    """unique_key = false: every key ends up in the table once, whatever the call
+    (tests/find_or_insert_ptr_test.cc.cu:3390-3475: 1024 copies of one key leave one entry);
+    which occurrence wins is unspecified, so values and scores are checked against the set of
+    the key's occurrences."""
+    cap, dim = 1 << 14, 8
+    o = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 30, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    rng = np.random.default_rng(314)
+    # the reference's scenario: one key, 1024 times, through the pointer overload
+    t = HashTable()
+    t.init(o)
+    n = 1024
+    same = np.full(n, 0x0101010101010101, dtype=np.uint64)
+    ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    founds = torch.ones(n, dtype=torch.bool, device=DEV)
+    sc = np.arange(1, n + 1, dtype=np.uint64)
+    t.find_or_insert_ptr(n, dev(same), ptrs, founds, dev(sc), unique_key=False)
+    torch.cuda.synchronize()
+    assert t.size() == 1
+    p = ptrs.cpu().numpy()
+    assert p[0] != 0 and (p == p[0]).all() and not founds.cpu().numpy().any()
+    t.find_or_insert_ptr(n, dev(same), ptrs, founds, dev(sc), unique_key=False)
+    torch.cuda.synchronize()
+    assert t.size() == 1 and (ptrs.cpu().numpy() == p[0]).all() and founds.cpu().numpy().all()
+    t.close()
+
+    # insert_or_assign: 4096 occurrences of 1000 keys
+    t = HashTable()
+    t.init(o)
+    uniq = w.unique_keys(61, 0, 1000)
+    n = 4096
+    pick = rng.integers(0, 1000, n)
+    pick[:1000] = np.arange(1000)  # every key at least once
+    keys = uniq[pick]
+    vals = rng.random((n, dim), dtype=np.float32)
+    sc = rng.permutation(n).astype(np.uint64) + np.uint64(10)
+    t.insert_or_assign(n, dev(keys), dev(vals), dev(sc), unique_key=False)
+    assert t.size() == 1000
+    ek, ev, es = sort_by_key(*export_table(t, dim * 4))
+    assert np.array_equal(ek, np.sort(uniq))
+    vb = bytes_of(vals)
+    for i in range(0, 1000, 37):
+        occ = np.flatnonzero(keys == ek[i])
+        hit = [j for j in occ if np.array_equal(vb[j], ev[i]) and sc[j] == es[i]]
+        assert hit, "the resident row and score must come from one occurrence of the key"
+    # find_or_insert with values: all occurrences of a key read the same row, the table's
+    q = np.concatenate([keys[:2000], w.unique_keys(62, 0, 500), w.unique_keys(62, 0, 500)])
+    m = len(q)
+    io = torch.from_numpy(rng.random((m, dim), dtype=np.float32)).to(DEV)
+    qs = rng.permutation(m).astype(np.uint64) + np.uint64(100000)
+    t.find_or_insert(m, dev(q), io, dev(qs), unique_key=False)
+    torch.cuda.synchronize()
+    assert t.size() == 1500
+    got = bytes_of(io.cpu().numpy())
+    out = torch.zeros(m, dim, dtype=torch.float32, device=DEV)
+    f = torch.zeros(m, dtype=torch.bool, device=DEV)
+    t.find(m, dev(q), out, f)
+    torch.cuda.synchronize()
+    assert f.cpu().numpy().all()
+    assert np.array_equal(got, bytes_of(out.cpu().numpy()))
+    t.close()
+
+    # insert_and_evict on a full table: what left + what stayed == what was there + new keys
+    t = HashTable()
+    t.init(o)
+    for b in range(5):
+        k = w.unique_keys(63, b * 4096, 4096)
+        t.insert_or_assign(4096, dev(k), dev(rng.random((4096, dim), dtype=np.float32)),
+                           dev(w.monotone_scores(b + 1, 4096)))
+    before = t.size()
+    fresh = w.unique_keys(64, 0, 1500)
+    keys = np.concatenate([fresh, fresh[:700], fresh[100:400]])
+    n = len(keys)
+    ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+    evv = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+    es = torch.zeros(n, dtype=torch.int64, device=DEV)
+    c = t.insert_and_evict(n, dev(keys), dev(rng.random((n, dim), dtype=np.float32)),
+                           dev(w.monotone_scores(9, n)), ek, evv, es, unique_key=False)
+    assert c + t.size() == before + 1500
+    assert len(np.unique(host_u64(ek)[:c])) == c
+    gk, _, _ = export_table(t, dim * 4)
+    assert len(np.unique(gk)) == len(gk)
+    t.close()
