@@ -89,6 +89,7 @@ SIGNATURES = {
     "hkv_accum_or_assign": (_i, [_T, _u64, _p, _p, _p, _p, _p, _i]),
     "hkv_find_or_insert": (_i, [_T, _u64, _p, _p, _p, _p, _i, _i]),
     "hkv_find_or_insert_ptr": (_i, [_T, _u64, _p, _p, _p, _p, _p, _i, _i]),
+    "hkv_find_or_insert_ptr_lock": (_i, [_T, _u64, _p, _p, _p, _p, _p, _p, _i]),
     "hkv_assign": (_i, [_T, _u64, _p, _p, _p, _p, _i]),
     "hkv_assign_scores": (_i, [_T, _u64, _p, _p, _p, _i]),
     "hkv_assign_values": (_i, [_T, _u64, _p, _p, _p, _i]),

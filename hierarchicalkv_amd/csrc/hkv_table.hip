@@ -1012,6 +1012,26 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
   return HKV_SUCCESS;
 }
 
+int hkv_find_or_insert_ptr_lock(hkv_table* t, uint64_t n, const uint64_t* keys, void** values,
+                                uint8_t* founds, const uint64_t* scores,
+                                uint64_t** locked_key_ptrs, hkv_stream_t stream, int ignore) {
+  HKV_TRY(refuse_dual(t, "find_or_insert()", true));
+  if (!locked_key_ptrs) return fail(HKV_ERROR_ARGUMENT, "locked_key_ptrs is null");
+  if (n == 0) return HKV_SUCCESS;
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.out_ptrs = values;
+  a.founds = founds;
+  a.scores = scores;
+  a.locked_key_ptrs = locked_key_ptrs;
+  a.n = n;
+  a.strategy = strategy;
+  t->keys_may_be_locked = true; /* LOCKED key words stay behind until unlock_keys */
+  return run_upsert<kOpFindOrInsertPtr>(t, a, 16, true, (hipStream_t)stream);
+}
+
 int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
                            void** values, uint8_t* founds, const uint64_t* scores,
                            hkv_stream_t stream, int unique_key, int ignore) {

@@ -55,6 +55,8 @@ struct UpsertArgs {
   uint64_t* evicted_scores;  /* may be null */
   unsigned long long* evicted_counter;
   void** out_ptrs;           /* find_or_insert pointer overload */
+  uint64_t** locked_key_ptrs; /* same overload: when given, the slots stay LOCKED and their key
+                                 addresses go here (find_ptr_or_insert.cuh:232-242) */
   uint8_t* founds;
   uint64_t n;
   uint64_t epoch;
@@ -694,6 +696,7 @@ upsert_kernel(View v, UpsertArgs a) {
     if (OP == kOpFindOrInsertPtr && (locked || refused_now)) {
       a.out_ptrs[i] = locked ? row : nullptr;
       a.founds[i] = got == kStDuplicate;
+      if (a.locked_key_ptrs) a.locked_key_ptrs[i] = locked ? v.keys + slot : nullptr;
     }
     if (commit && !HKV_EXP_FLAG(8)) {
       write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
@@ -724,7 +727,9 @@ upsert_kernel(View v, UpsertArgs a) {
     /* ---- step 5: everything written under the locks is out; release them --------------------------- */
     wait_stores();
     HKV_MARK(14); /* store drain */
-    if (locked) st_unlock(v.keys + slot, commit ? key : victim);
+    /* the pointer overload may be asked to leave its slots locked for unlock_keys */
+    const bool keep_locked = OP == kOpFindOrInsertPtr && a.locked_key_ptrs != nullptr;
+    if (locked && !keep_locked) st_unlock(v.keys + slot, commit ? key : victim);
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
     if (pend_mask) __builtin_amdgcn_s_sleep(1);

@@ -152,7 +152,14 @@ class HashTable:
                                       _stream(stream), int(unique_key), int(ignore_evict_strategy)))
 
     def find_or_insert_ptr(self, n, keys, value_ptrs, founds, scores=None, stream=None,
-                           unique_key=True, ignore_evict_strategy=False):
+                           unique_key=True, ignore_evict_strategy=False, locked_key_ptrs=None):
+        if locked_key_ptrs is not None:
+            if not unique_key:
+                raise ValueError("unique_key should be true and max_bucket_size should be larger.")
+            _check(lib.hkv_find_or_insert_ptr_lock(self._h, n, _ptr(keys), _ptr(value_ptrs),
+                                                   _ptr(founds), _ptr(scores), _ptr(locked_key_ptrs),
+                                                   _stream(stream), int(ignore_evict_strategy)))
+            return
         _check(lib.hkv_find_or_insert_ptr(self._h, n, _ptr(keys), _ptr(value_ptrs), _ptr(founds),
                                           _ptr(scores), _stream(stream), int(unique_key),
                                           int(ignore_evict_strategy)))

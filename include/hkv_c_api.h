@@ -200,6 +200,14 @@ int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
                            void** values, uint8_t* founds /* bool[n] */,
                            const uint64_t* scores, hkv_stream_t stream,
                            int unique_key, int ignore_evict_strategy);
+/* The same overload with locked_key_ptrs (merlin_hashtable.cuh:1878-1927,
+ * find_ptr_or_insert.cuh:27-245): the slots of the accepted keys stay LOCKED, their key
+ * addresses are returned, and the caller releases them with hkv_unlock_keys after writing
+ * the rows.  Keys of the batch must be unique. */
+int hkv_find_or_insert_ptr_lock(hkv_table* t, uint64_t n, const uint64_t* keys,
+                                void** values, uint8_t* founds, const uint64_t* scores,
+                                uint64_t** locked_key_ptrs, hkv_stream_t stream,
+                                int ignore_evict_strategy);
 
 /* HashTable::assign (values + scores), merlin_hashtable.cuh:2071-2213 */
 int hkv_assign(hkv_table* t, uint64_t n, const uint64_t* keys,

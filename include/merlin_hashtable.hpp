@@ -591,9 +591,16 @@ class HashTable : public HashTableBase<K, V, S> {
                       score_type* scores = nullptr, hipStream_t stream = 0,
                       bool unique_key = true, bool ignore_evict_strategy = false,
                       key_type** locked_key_ptrs = nullptr) override {
-    if (locked_key_ptrs != nullptr)
-      throw std::runtime_error("find_or_insert with locked_key_ptrs is not supported");
     detail::ScoresIn<S> sc(scores, n, stream);
+    if (locked_key_ptrs != nullptr) {
+      /* merlin_hashtable.cuh:1914-1918 */
+      if (!unique_key)
+        throw std::invalid_argument("unique_key should be true and max_bucket_size should be larger.");
+      throw_on_error_(hkv_find_or_insert_ptr_lock(
+          table_, n, u64(keys), reinterpret_cast<void**>(values), reinterpret_cast<uint8_t*>(founds),
+          sc.get(), reinterpret_cast<uint64_t**>(locked_key_ptrs), stream, ignore_evict_strategy));
+      return;
+    }
     throw_on_error_(hkv_find_or_insert_ptr(table_, n, u64(keys), reinterpret_cast<void**>(values),
                                            reinterpret_cast<uint8_t*>(founds), sc.get(), stream,
                                            unique_key, ignore_evict_strategy));

@@ -569,3 +569,69 @@ def test_batches_with_repeated_keys(oracle):
     gk, _, _ = export_table(t, dim * 4)
     assert len(np.unique(gk)) == len(gk)
     t.close()
+
+
+def test_find_or_insert_with_locked_key_pointers(oracle):
+    """find_or_insert(…, locked_key_ptrs): the accepted keys stay LOCKED (invisible to lookups)
+    until unlock_keys, and the table then equals what the plain pointer overload leaves
+    (merlin_hashtable.cuh:1878-1927, find_ptr_or_insert.cuh:27-245)."""
+    cap, dim, bs = 1 << 13, 8, 7000
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    keys = w.unique_keys(95, 0, bs)
+    vals = w.values_from_keys(keys, dim)
+    sc = w.monotone_scores(1, bs)
+    t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
+    o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1), sc)
+    n = 3000
+    batch = np.concatenate([keys[:1000], w.unique_keys(96, 0, n - 1000),
+                            np.array([M64, M64 - 1], np.uint64)])
+    n = len(batch)
+    bsc = w.monotone_scores(2, n)
+    vptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    kptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+    founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.find_or_insert_ptr(n, dev(batch), vptrs, founds, dev(bsc), locked_key_ptrs=kptrs)
+    torch.cuda.synchronize()
+    oslots, of = o.find_or_insert_slot(batch, bsc)
+    accepted = (of != 2) & (oslots != np.uint64(M64))  # reserved keys are not looked at at all
+    assert np.array_equal(founds.cpu().numpy()[accepted], of[accepted].astype(bool))
+    vp, kp = vptrs.cpu().numpy(), kptrs.cpu().numpy()
+    assert np.array_equal(vp != 0, accepted) and np.array_equal(kp != 0, accepted)
+    assert accepted[:n - 2].sum() > 2000 and not accepted[-2:].any()
+    assert t.size() == o.size()
+    # every accepted key is invisible while locked, the rest of the table is not
+    c = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.contains(n, dev(batch), c)
+    torch.cuda.synchronize()
+    assert not c.cpu().numpy().any()
+    c2 = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.contains(bs, dev(keys), c2)
+    untouched = o.contains(keys)
+    untouched[:1000] = False
+    assert np.array_equal(c2.cpu().numpy(), untouched)
+    # rows are written through the value pointers, then the keys are released
+    newrows = w.values_from_keys(batch, dim) + np.float32(0.5)
+    import ctypes as C
+    from gpu_util import hip
+    for i in np.flatnonzero(accepted)[::41]:
+        row = np.ascontiguousarray(newrows[i])
+        assert hip().hipMemcpy(C.c_void_p(int(vp[i])), row.ctypes.data, dim * 4, 1) == 0
+    ok = torch.zeros(n, dtype=torch.bool, device=DEV)
+    t.unlock_keys(n, kptrs, dev(batch), ok)
+    torch.cuda.synchronize()
+    assert np.array_equal(ok.cpu().numpy(), accepted)
+    out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+    f = torch.zeros(n, dtype=torch.bool, device=DEV)
+    s = torch.zeros(n, dtype=torch.int64, device=DEV)
+    t.find(n, dev(batch), out, f, s)
+    torch.cuda.synchronize()
+    assert np.array_equal(f.cpu().numpy(), accepted)
+    outn = out.cpu().numpy()
+    for i in np.flatnonzero(accepted)[::41]:
+        assert np.array_equal(outn[i], newrows[i])
+    # keys and scores equal the oracle's table (rows of new keys are the caller's business)
+    gk, _, gs = sort_by_key(*export_table(t, dim * 4))
+    ok_, _, os_ = sort_by_key(*o.export_all())
+    assert np.array_equal(gk, ok_) and np.array_equal(gs, os_)
+    t.close()
