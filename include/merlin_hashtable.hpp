@@ -856,25 +856,30 @@ class HashTable : public HashTableBase<K, V, S> {
     so.finish();
   }
 
-  /* merlin_hashtable.cuh:3460-3476.  Synchronises `stream`. */
+  /* merlin_hashtable.cuh:3460-3476: the count goes to a device word, asynchronously */
+  template <template <typename, typename> class PredFunctor>
+  void size_if(const key_type& pattern, const score_type& threshold, size_type* d_counter,
+               hipStream_t stream = 0) const {
+    hkv_table_view v;
+    throw_on_error_(hkv_table_get_view(table_, &v));
+    detail::RoleGuard g(table_, 0, stream);
+    hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
+    const unsigned blocks = hkv::scan_grid(v.capacity, 256);
+    hipLaunchKernelGGL((hkv::size_if_kernel<detail::PredAdapter<K, S, PredFunctor>>), dim3(blocks),
+                       dim3(256), 0, stream, v, detail::PredAdapter<K, S, PredFunctor>(),
+                       static_cast<uint64_t>(pattern), static_cast<uint64_t>(threshold),
+                       reinterpret_cast<unsigned long long*>(d_counter));
+    HKV_HIP_CHECK(hipGetLastError());
+  }
+
+  /* convenience form without a counter argument (not in the reference): returns the count and
+   * synchronises `stream` */
   template <template <typename, typename> class PredFunctor>
   size_type size_if(const key_type& pattern, const score_type& threshold,
                     hipStream_t stream = 0) const {
-    hkv_table_view v;
-    throw_on_error_(hkv_table_get_view(table_, &v));
     unsigned long long* d_count = nullptr;
     HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
-    hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
-                       d_count);
-    {
-      detail::RoleGuard g(table_, 0, stream);
-      const unsigned blocks = hkv::scan_grid(v.capacity, 256);
-      hipLaunchKernelGGL((hkv::size_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
-                         dim3(blocks), dim3(256), 0, stream, v,
-                         detail::PredAdapter<K, S, PredFunctor>(), static_cast<uint64_t>(pattern),
-                         static_cast<uint64_t>(threshold), d_count);
-      HKV_HIP_CHECK(hipGetLastError());
-    }
+    size_if<PredFunctor>(pattern, threshold, reinterpret_cast<size_type*>(d_count), stream);
     unsigned long long h = 0;
     HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
     HKV_HIP_CHECK(hipStreamSynchronize(stream));

@@ -386,6 +386,10 @@ static void test_insert_and_evict_and_predicates() {
   CHECK(erased == odd_high);
   CHECK(table.size() == before - erased);
   CHECK(table.size_if<EraseIfPredFunctor>(0, threshold) == 0);
+  // the reference's form of size_if: device counter, asynchronous (merlin_hashtable.cuh:3460-3476)
+  table.size_if<ExportIfPredFunctor>(0, threshold, dc.p);
+  HIP(hipDeviceSynchronize());
+  CHECK(dc.down(1)[0] == table.size_if<ExportIfPredFunctor>(0, threshold));
 }
 
 struct CountingAllocator : public DefaultAllocator {
