@@ -19,14 +19,27 @@ def bytes_of(a):
     return np.ascontiguousarray(a).view(np.uint8).reshape(len(a), -1)
 
 
-@pytest.mark.parametrize("seed,dim,cap", [(1, 4, 1 << 13), (2, 16, 1 << 13), (3, 5, 12345 // 128 * 128 + 128),
-                                          (4, 64, 1 << 12)])
-def test_random_call_sequences(oracle, seed, dim, cap):
+@pytest.mark.parametrize("seed,dim,cap,strategy", [
+    (1, 4, 1 << 13, EvictStrategy.kCustomized),
+    (2, 16, 1 << 13, EvictStrategy.kCustomized),
+    (3, 5, 12345 // 128 * 128 + 128, EvictStrategy.kCustomized),
+    (4, 64, 1 << 12, EvictStrategy.kCustomized),
+    (5, 8, 1 << 13, EvictStrategy.kLru),       # scores from the deterministic clock
+    (6, 32, 1 << 12, EvictStrategy.kEpochLru),
+])
+def test_random_call_sequences(oracle, seed, dim, cap, strategy):
     o = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 30, dim=dim,
-                        evict_strategy=EvictStrategy.kCustomized)
+                        evict_strategy=strategy)
     t = HashTable()
     t.init(o)
     ot = oracle.OracleTable(o)
+    clocked = strategy != EvictStrategy.kCustomized
+    if clocked:
+        t.set_clock(1, 1 << 44)
+        ot.set_clock(1, 1 << 44)
+    if strategy == EvictStrategy.kEpochLru:
+        t.set_global_epoch(1)
+        ot.set_global_epoch(1)
     rng = np.random.default_rng(1000 + seed)
     universe = w.unique_keys(500 + seed, 0, 3 * cap)
     vb = dim * 4
@@ -39,7 +52,10 @@ def test_random_call_sequences(oracle, seed, dim, cap):
             keys[rng.integers(0, n)] = np.uint64((1 << 64) - 1 - int(rng.integers(0, 4)))
         vals = rng.random((n, dim), dtype=np.float32)
         seq += 1
-        sc = w.monotone_scores(seq, n, seed=seed)
+        sc = None if clocked else w.monotone_scores(seq, n, seed=seed)
+        if strategy == EvictStrategy.kEpochLru and step % 16 == 15:
+            t.set_global_epoch(1 + step // 16)
+            ot.set_global_epoch(1 + step // 16)
         op = rng.choice(["insert_or_assign", "find", "find_or_insert", "insert_and_evict", "assign",
                          "accum_or_assign", "erase", "contains", "export_if"],
                         p=[0.25, 0.12, 0.12, 0.15, 0.08, 0.1, 0.08, 0.05, 0.05])
@@ -52,7 +68,8 @@ def test_random_call_sequences(oracle, seed, dim, cap):
             keep = present if (rng.random() < 0.5 and present.sum() > 0) else ~present
             if keep.sum() == 0:
                 keep = ~keep
-            keys, vals, sc = keys[keep], vals[keep], sc[keep]
+            keys, vals = keys[keep], vals[keep]
+            sc = None if sc is None else sc[keep]
             n = len(keys)
         dk, dv, ds = dev(keys), dev(vals), dev(sc)
         if op == "insert_or_assign":
@@ -108,6 +125,9 @@ def test_random_call_sequences(oracle, seed, dim, cap):
             assert np.array_equal(f.cpu().numpy(), ot.contains(keys)), (step, op)
         elif op == "export_if":
             thr = int(w.monotone_scores(max(1, seq - 5), 1, seed=seed)[0])
+            if clocked:  # somewhere inside the range of scores the clock has handed out
+                _, _, alls = ot.export_all()
+                thr = int(np.median(alls)) if len(alls) else 0
             got = sort_by_key(*export_table(t, vb, Predicate.kScoreGe, 0, thr, chunk=1000))
             want = sort_by_key(*ot.export_batch_if(int(Predicate.kScoreGe), 0, thr))
             assert all(np.array_equal(x, y) for x, y in zip(got, want)), (step, op)
