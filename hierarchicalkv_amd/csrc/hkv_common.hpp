@@ -163,6 +163,17 @@ __device__ __forceinline__ void st_u32(uint32_t* p, uint32_t x) {
 __device__ __forceinline__ void st_u8(uint8_t* p, uint8_t x) {
   __hip_atomic_store(p, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+/* 16-byte agent-coherent load at byte `offset` of an array of `bytes` bytes (below 4 GiB),
+ * as one instruction.  The compiler offers 128-bit agent-scope loads only through a buffer
+ * resource; the array's base and size are the same for the whole wavefront, the offset is
+ * per lane.  Offsets past the end read zero. */
+__device__ __forceinline__ uint4 ld_u128_at(const void* base, uint64_t bytes, uint64_t offset) {
+  const __amdgpu_buffer_rsrc_t rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (uint32_t)bytes, 0x00020000);
+  const u32x4_t x = __builtin_amdgcn_raw_buffer_load_b128(rs, (uint32_t)offset, 0, 16 /* sc1 */);
+  return make_uint4(x.x, x.y, x.z, x.w);
+}
 /* 16-byte write-through store, marked non-temporal: what is written this way (value
  * rows, a whole digest line) is not read again soon, and keeping it out of the caches
  * leaves them to the digest and key lines the next call probes (measured: the next find
@@ -172,7 +183,6 @@ __device__ __forceinline__ void st_u8(uint8_t* p, uint8_t x) {
  * issued from inline assembly: the wavefront's store counter still covers it
  * (wait_stores), and the s_nop keeps the next instruction from overwriting
  * the data registers while the store reads them. */
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void st_u128(void* p, const uint4& x) {
   u32x4_t d = {x.x, x.y, x.z, x.w};
   asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" : : "v"(p), "v"(d) : "memory");

@@ -30,18 +30,6 @@
 
 namespace hkv {
 
-/* the 16 digest bytes of lane j, read past the caches */
-__device__ __forceinline__ uint4 ld_digests16(const View& v, uint32_t bkt, int j) {
-  const uint32_t* dp =
-      reinterpret_cast<const uint32_t*>(v.digests + (uint64_t)bkt * kBucketSize + j * 16);
-  uint4 d;
-  d.x = ld_u32(dp + 0);
-  d.y = ld_u32(dp + 1);
-  d.z = ld_u32(dp + 2);
-  d.w = ld_u32(dp + 3);
-  return d;
-}
-
 /* how often phase 2 looks again before the key is given up as refused (every
  * repeat means another tile changed one of the two buckets in between) */
 constexpr int kDualMaxTries = 1024;

@@ -116,6 +116,19 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
   }
 }
 
+/* the 16 digest bytes of lane j of a tile, read past the caches */
+__device__ __forceinline__ uint4 ld_digests16(const View& v, uint32_t bkt, int j) {
+  const uint64_t off = (uint64_t)bkt * kBucketSize + j * 16;
+  if (v.capacity < (UINT64_C(1) << 32)) return ld_u128_at(v.digests, v.capacity, off);
+  const uint32_t* dp = reinterpret_cast<const uint32_t*>(v.digests + off);
+  uint4 d;
+  d.x = ld_u32(dp + 0);
+  d.y = ld_u32(dp + 1);
+  d.z = ld_u32(dp + 2);
+  d.w = ld_u32(dp + 3);
+  return d;
+}
+
 /*
  * Second opinion for a writer, by the 8-lane tile that owns the key, with
  * coherent loads: returns the slot of the key, -1 when the key is not in the
@@ -125,13 +138,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
 __device__ __forceinline__ int64_t tile_reprobe(const View& v, uint64_t key,
                                                 uint32_t bkt, uint32_t digest,
                                                 int tile, int j, uint32_t& em) {
-  const uint32_t* dp =
-      reinterpret_cast<const uint32_t*>(v.digests + (uint64_t)bkt * kBucketSize + j * 16);
-  uint4 d;
-  d.x = __hip_atomic_load(dp + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  d.y = __hip_atomic_load(dp + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  d.z = __hip_atomic_load(dp + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  d.w = __hip_atomic_load(dp + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint4 d = ld_digests16(v, bkt, j);
   em = match16_natural(d, v.empty_digest * 0x01010101u);
   uint32_t m = match16(d, digest * 0x01010101u);
   const uint64_t slot0 = (uint64_t)bkt * kBucketSize + j * 16;

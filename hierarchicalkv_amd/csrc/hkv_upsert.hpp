@@ -284,6 +284,25 @@ __device__ __forceinline__ uint32_t first_from(uint64_t lo, uint64_t hi, uint32_
 template <bool LOCKED_RULE>
 __device__ __forceinline__ void scan_load(const View& v, uint64_t bslot, int j, uint64_t* sc,
                                           uint64_t* kc) {
+  if (v.capacity < (UINT64_C(1) << 29)) {
+    /* one 16-byte coherent load per line and lane (ld_u128_at): half the load instructions
+     * of the 8-byte form, measured 6 % on a whole insert_or_assign batch */
+#pragma unroll
+    for (int it = 0; it < kTile; it++) {
+      const uint4 x = ld_u128_at(v.scores, v.capacity * 8, (bslot + it * 16 + j * 2) * 8);
+      sc[2 * it] = x.x | ((uint64_t)x.y << 32);
+      sc[2 * it + 1] = x.z | ((uint64_t)x.w << 32);
+    }
+    if (LOCKED_RULE) {
+#pragma unroll
+      for (int it = 0; it < kTile; it++) {
+        const uint4 x = ld_u128_at(v.keys, v.capacity * 8, (bslot + it * 16 + j * 2) * 8);
+        kc[2 * it] = x.x | ((uint64_t)x.y << 32);
+        kc[2 * it + 1] = x.z | ((uint64_t)x.w << 32);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int it = 0; it < kTile; it++) {
     const uint64_t* sp = v.scores + bslot + it * 16 + j * 2;
