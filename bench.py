@@ -45,7 +45,7 @@ def upsert_bytes(vb, new_fraction):
 # 1 GiB device-to-device copy: 2.000 and 1.000).  Counters cannot be read from inside
 # this process, so the figures of the committed profile summary are reported; they
 # apply to the default workload and the default (slot-lock) upsert path only.
-MEASURED_TRAFFIC = {"upsert_kernel": 1541.4e6, "lookup_kernel": 868.2e6}
+MEASURED_TRAFFIC = {"upsert_kernel": 1553.3e6, "lookup_kernel": 868.2e6}
 
 
 def main():
