@@ -18,6 +18,7 @@
 #include <mutex>
 #include <new>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "hkv_c_api.h"
@@ -165,6 +166,10 @@ struct hkv_table {
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
   bool keys_may_be_locked; /* lock_keys has been called: LOCKED key words may sit in the table */
   bool dual;               /* TableMode::kMemory: two candidate buckets per key */
+  bool io_by_cpu;          /* value rows of the writers are moved by host threads */
+  std::mutex io_mutex;     /* one CPU-IO call at a time uses the staging area */
+  void* io_stage;          /* pinned staging area of the CPU-IO calls, grown on demand */
+  uint64_t io_stage_bytes;
 };
 
 namespace {
@@ -588,6 +593,138 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   return HKV_SUCCESS;
 }
 
+/* ---- io_by_cpu: host threads move the value rows of the writers -----------------
+ * merlin_hashtable.cuh:1275-1292 (insert_or_assign), 1820-1841 (find_or_insert),
+ * 2175-2192 (assign), 2414-2431 (assign_values); write_by_cpu upsert.cuh:1711-1747,
+ * read_or_write_by_cpu find_or_insert.cuh:1814-1855.  All rows of such a table are in
+ * pinned host memory (max_hbm_for_vectors must be 0).  A kernel settles keys, scores and
+ * digests and reports the row address of every accepted key; addresses and the caller's
+ * rows are copied to the host, the stream is synchronised and up to 16 host threads copy
+ * the rows; the role of the group lock is held until they are done.  The upserts follow
+ * the plain kernels' rule (refuse when score < min), as the reference's do with this
+ * option. */
+struct CpuIoStage {
+  uint8_t** ptrs;   /* n row addresses (device view of the pinned rows) */
+  uint8_t* founds;  /* n flags */
+  uint8_t* rows;    /* n caller rows */
+};
+
+int cpu_io_stage(hkv_table* t, uint64_t n, CpuIoStage& st) {
+  const uint64_t vb = t->view.value_bytes;
+  const uint64_t off_founds = n * 8, off_rows = (off_founds + n + 255) & ~UINT64_C(255);
+  const uint64_t need = off_rows + n * vb;
+  if (need > t->io_stage_bytes) {
+    if (t->io_stage) (void)hipHostFree(t->io_stage);
+    t->io_stage = nullptr;
+    t->io_stage_bytes = 0;
+    HKV_HIP(hipHostMalloc(&t->io_stage, need, hipHostMallocDefault));
+    t->io_stage_bytes = need;
+  }
+  uint8_t* base = (uint8_t*)t->io_stage;
+  st.ptrs = (uint8_t**)base;
+  st.founds = base + off_founds;
+  st.rows = base + off_rows;
+  return HKV_SUCCESS;
+}
+
+/* an address the kernels reported -> the host's address of the same row */
+inline uint8_t* cpu_io_host_row(const hkv_table* t, const uint8_t* p) {
+  return (uint8_t*)t->h_values + (p - t->view.host_values);
+}
+
+/* direction per key: 0 skip, 1 caller row -> table, 2 table -> caller row */
+template <class Dir>
+void cpu_io_copy(const hkv_table* t, uint64_t n, const CpuIoStage& st, Dir dir) {
+  const uint64_t vb = t->view.value_bytes;
+  const unsigned workers = (unsigned)std::min<uint64_t>(16, (n + 4095) / 4096);
+  auto work = [&](uint64_t lo, uint64_t hi) {
+    for (uint64_t i = lo; i < hi; i++) {
+      if (!st.ptrs[i]) continue;
+      uint8_t* row = cpu_io_host_row(t, st.ptrs[i]);
+      const int d = dir(i);
+      if (d == 1)
+        memcpy(row, st.rows + i * vb, vb);
+      else if (d == 2)
+        memcpy(st.rows + i * vb, row, vb);
+    }
+  };
+  if (workers <= 1) {
+    work(0, n);
+    return;
+  }
+  std::vector<std::thread> th;
+  const uint64_t per = (n + workers - 1) / workers;
+  for (unsigned w = 0; w < workers; w++) {
+    const uint64_t lo = std::min<uint64_t>(n, w * per), hi = std::min<uint64_t>(n, lo + per);
+    if (lo < hi) th.emplace_back(work, lo, hi);
+  }
+  for (auto& x : th) x.join();
+}
+
+/* A key that took a slot may lose it to a later key of the same batch (evicted again);
+ * its address is dropped, so the row is written by the key that owns the slot at the end.
+ * Keys that only read their row (`readers`: the hits of find_or_insert) keep theirs. */
+__global__ void cpu_io_owner_kernel(View v, const uint64_t* keys, uint8_t** ptrs,
+                                    const uint8_t* readers, uint64_t n) {
+  const uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const uint8_t* p = ptrs[i];
+  if (!p || (readers && readers[i])) return;
+  const uint64_t slot = v.hbm_slots + (uint64_t)(p - v.host_values) / v.value_bytes;
+  if (ld_u64(v.keys + slot) != keys[i]) ptrs[i] = nullptr;
+}
+
+/* insert_or_assign (reads == false) and find_or_insert (reads == true) */
+int cpu_io_upsert(hkv_table* t, UpsertArgs a, void* values, bool reads, hipStream_t s) {
+  HKV_TRY(grow_for(t, a.n, s));
+  const uint64_t n = a.n, vb = t->view.value_bytes;
+  std::lock_guard<std::mutex> host_lock(t->io_mutex);
+  CpuIoStage st{};
+  HKV_TRY(cpu_io_stage(t, n, st));
+  void* d_tmp = nullptr;
+  HKV_HIP(hipMallocAsync(&d_tmp, n * 9, s));
+  a.out_ptrs = (void**)d_tmp;
+  a.founds = (uint8_t*)d_tmp + n * 8;
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.value_kind = t->opts.value_kind;
+  a.refuse_equal = 0;
+  hipError_t e = hipSuccess;
+  {
+    LockGuard g(t, StreamGroupLock::kInserter, s);
+    e = g.acquire();
+    if (e == hipSuccess) e = hipMemsetAsync(d_tmp, 0, n * 9, s); /* reserved / refused keys: no address */
+    if (e == hipSuccess) {
+      launch_upsert<kOpFindOrInsertPtr, true>(16, t->view, a, s);
+      hipLaunchKernelGGL(cpu_io_owner_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
+                         t->view, a.keys, (uint8_t**)d_tmp,
+                         reads ? (const uint8_t*)d_tmp + n * 8 : nullptr, n);
+      e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(st.ptrs, d_tmp, n * 8, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(st.founds, (uint8_t*)d_tmp + n * 8, n, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(st.rows, values, n * vb, hipMemcpyDefault, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e == hipSuccess) {
+      if (reads) {
+        /* every read before any write: a row that is read by one key and taken over by
+         * another key of the batch still holds what it held before the call */
+        cpu_io_copy(t, n, st, [&](uint64_t i) { return st.founds[i] ? 2 : 0; });
+        cpu_io_copy(t, n, st, [&](uint64_t i) { return st.founds[i] ? 0 : 1; });
+        e = hipMemcpyAsync(values, st.rows, n * vb, hipMemcpyDefault, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+      } else {
+        cpu_io_copy(t, n, st, [](uint64_t) { return 1; });
+      }
+    }
+  }
+  (void)hipFreeAsync(d_tmp, s);
+  HKV_HIP(e);
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
+}
+
+
 /* The calls that refuse a dual-bucket table with a MERLIN_CHECK
  * (merlin_hashtable.cuh:1362, 1597, 1705, 1891, 2233, 2304, 2860, 2905, 3505) report
  * HKV_ERROR_CHECK.  The calls the reference leaves unguarded although they probe one bucket
@@ -709,8 +846,8 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
     return fail(HKV_ERROR_CHECK,
                 "[HierarchicalKV] `io_by_cpu` should not be true when "
                 "`max_hbm_for_vectors` is not 0!");
-  if (o->io_by_cpu)
-    return fail(HKV_ERROR_UNSUPPORTED, "io_by_cpu is not supported");
+  if (o->io_by_cpu && o->table_mode == 1)
+    return fail(HKV_ERROR_UNSUPPORTED, "io_by_cpu is not supported in dual-bucket mode");
   if (o->evict_strategy < 0 || o->evict_strategy > 4)
     return fail(HKV_ERROR_ARGUMENT, "bad evict_strategy %d", o->evict_strategy);
   if (o->score_size != 8)
@@ -737,6 +874,9 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->scratch_bytes = 0;
   t->keys_may_be_locked = false;
   t->dual = o->table_mode == 1;
+  t->io_by_cpu = o->io_by_cpu != 0;
+  t->io_stage = nullptr;
+  t->io_stage_bytes = 0;
   /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default while the
    * two-phase path is being tuned), "auto" = two-phase for large batches,
    * "grouped" = two-phase whenever it is possible (tests) */
@@ -880,6 +1020,7 @@ int hkv_table_destroy(hkv_table* t) {
   table_free(t, 0, t->d_scratch);
   table_free(t, 0, t->d_values);
   table_free(t, 1, t->h_values);
+  if (t->io_stage) (void)hipHostFree(t->io_stage);
   delete t;
   return HKV_SUCCESS;
 }
@@ -917,7 +1058,10 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
     if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
     return HKV_SUCCESS;
   }
-  return run_upsert<kOpInsertOrAssign>(t, a, vec, true, (hipStream_t)stream);
+  if (t->io_by_cpu) return cpu_io_upsert(t, a, const_cast<void*>(values), false, (hipStream_t)stream);
+  /* with unique_key == false the reference leaves its lock-key kernels for the plain one
+   * (merlin_hashtable.cuh:1235-1258), whose rule is "refuse when score < min" */
+  return run_upsert<kOpInsertOrAssign>(t, a, vec, unique_key != 0, (hipStream_t)stream);
 }
 
 int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
@@ -1001,7 +1145,10 @@ int hkv_find_or_insert(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.n = n;
   a.strategy = strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
-  HKV_TRY(run_upsert<kOpFindOrInsert>(t, a, vec, true, (hipStream_t)stream));
+  if (t->io_by_cpu)
+    HKV_TRY(cpu_io_upsert(t, a, values, true, (hipStream_t)stream));
+  else /* merlin_hashtable.cuh:1779-1803: lock-key kernels only with unique keys */
+    HKV_TRY(run_upsert<kOpFindOrInsert>(t, a, vec, unique_key != 0, (hipStream_t)stream));
   if (dg.on) {
     /* the other occurrences of a key get the row its representative ended up with (what it
      * read, or what it inserted; a refused key keeps its own row, like its representative) */
@@ -1070,6 +1217,43 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.touch_scores = touch_scores;
   a.strategy = t->opts.evict_strategy;
   const int vec = pick_vec(t->view.value_bytes, {values});
+  if (t->io_by_cpu && values) {
+    /* scores by the kernel, row addresses by a lookup, rows by host threads */
+    const uint64_t vb = t->view.value_bytes;
+    std::lock_guard<std::mutex> host_lock(t->io_mutex);
+    CpuIoStage st{};
+    HKV_TRY(cpu_io_stage(t, n, st));
+    void* d_tmp = nullptr;
+    HKV_HIP(hipMallocAsync(&d_tmp, n * 9, s));
+    hipError_t e = hipSuccess;
+    {
+      LockGuard g(t, StreamGroupLock::kUpdater, s);
+      e = g.acquire();
+      if (e == hipSuccess && touch_scores) {
+        a.values = nullptr;
+        hipLaunchKernelGGL((assign_kernel<16, 1>), dim3(grid_for(n)), dim3(kWave), 0, s, t->view, a);
+        e = hipGetLastError();
+      }
+      if (e == hipSuccess) e = hipMemsetAsync(d_tmp, 0, n * 9, s); /* reserved keys: no address */
+      if (e == hipSuccess) {
+        FindArgs f{};
+        f.keys = keys;
+        f.out_ptrs = (void**)d_tmp;
+        f.founds = (uint8_t*)d_tmp + n * 8;
+        f.n = n;
+        launch_lookup<kLookupPtr>(16, t->view, f, s);
+        e = hipGetLastError();
+      }
+      if (e == hipSuccess) e = hipMemcpyAsync(st.ptrs, d_tmp, n * 8, hipMemcpyDeviceToHost, s);
+      if (e == hipSuccess) e = hipMemcpyAsync(st.rows, values, n * vb, hipMemcpyDefault, s);
+      if (e == hipSuccess) e = hipStreamSynchronize(s);
+      if (e == hipSuccess) cpu_io_copy(t, n, st, [](uint64_t) { return 1; });
+    }
+    (void)hipFreeAsync(d_tmp, s);
+    HKV_HIP(e);
+    if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+    return HKV_SUCCESS;
+  }
   {
     LockGuard g(t, StreamGroupLock::kUpdater, s);
     HKV_HIP(g.acquire());

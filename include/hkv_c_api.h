@@ -87,7 +87,8 @@ typedef struct hkv_options {
   int32_t block_size;
   int32_t io_block_size;
   int32_t device_id; /* -1: current device */
-  int32_t io_by_cpu;
+  int32_t io_by_cpu; /* host threads move the rows of insert_or_assign, find_or_insert, assign and
+                        assign_values (needs max_hbm_for_vectors == 0; these calls then synchronise) */
   int32_t use_constant_memory;
   int32_t reserved_key_start_bit;
   uint64_t num_of_buckets_per_alloc;

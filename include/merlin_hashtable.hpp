@@ -237,7 +237,7 @@ struct HashTableOptions {
   int block_size = 128;            ///< Kept for source compatibility; unused.
   int io_block_size = 1024;        ///< Kept for source compatibility; unused.
   int device_id = -1;              ///< The ID of device.
-  bool io_by_cpu = false;          ///< Not supported (must stay false).
+  bool io_by_cpu = false;          ///< Host threads move the rows of the writers (needs max_hbm_for_vectors == 0).
   bool use_constant_memory = false;  ///< reserved
   int reserved_key_start_bit = 0;       ///< The binary index of reserved key.
   size_t num_of_buckets_per_alloc = 1;  ///< Checked as in the reference; the

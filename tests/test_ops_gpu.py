@@ -323,6 +323,66 @@ def test_hybrid_mode(oracle):
     t.close()
 
 
+def test_io_by_cpu(oracle):
+    """io_by_cpu (merlin_hashtable.cuh:1275-1292, 1820-1841, 2175-2192, 2414-2431): all rows in
+    pinned host memory, host threads move the rows of insert_or_assign, find_or_insert, assign
+    and assign_values; the upserts follow the plain kernels' rule (refuse when score < min)."""
+    cap, dim, bs = 1 << 15, 16, 1 << 12
+    with pytest.raises(MerlinException):  # merlin_hashtable.cuh:1071-1073
+        HashTable().init(default_options(init_capacity=cap, max_capacity=cap, dim=dim,
+                                         max_hbm_for_vectors=1 << 20, io_by_cpu=1))
+    t, o, _ = make_pair(oracle, hybrid=False, init_capacity=cap, max_capacity=cap, dim=dim,
+                        max_hbm_for_vectors=0, io_by_cpu=1, evict_strategy=EvictStrategy.kCustomized)
+    assert not t.is_pure_hbm() and t.view().hbm_slots == 0
+
+    def distinct(b, n):
+        return (np.uint64(b + 1) << np.uint64(24)) + np.random.Generator(np.random.PCG64(300 + b)).permutation(n).astype(np.uint64)
+    nb = (cap + 3 * bs) // bs  # past load factor 1.0: the last batches evict
+    fill(t, o, 131, nb, bs, dim, distinct)
+    assert t.size() == o.size()
+    assert_same_table(t, o, dim * 4)
+    recent = w.unique_keys(131, (nb - 2) * bs, bs)
+    # insert_or_assign, half hits; a refusal at score == min would show (plain rule: accepted)
+    keys = np.concatenate([recent[: bs // 2], w.unique_keys(132, 0, bs // 2),
+                           np.array([M64, M64 - 2], np.uint64)])
+    n = len(keys)
+    vals = w.uniform_values(133, 0, n, dim)
+    sc = distinct(nb + 2, n)
+    t.insert_or_assign(n, dev(keys), dev(vals), dev(sc))
+    o.insert_or_assign(keys, bytes_of(vals), sc)
+    assert_same_table(t, o, dim * 4)
+    # find_or_insert: hits read, new keys write
+    keys = np.concatenate([recent[bs // 2:], w.unique_keys(134, 0, bs // 2)])
+    io = w.uniform_values(135, 0, bs, dim)
+    d_io = dev(io)
+    sc = distinct(nb + 3, bs)
+    t.find_or_insert(bs, dev(keys), d_io, dev(sc))
+    oio = bytes_of(io).copy()
+    o.find_or_insert(keys, oio, sc)
+    torch.cuda.synchronize()
+    assert (host_bytes(d_io, bs, dim * 4) == oio).all()
+    assert_same_table(t, o, dim * 4)
+    # assign (rows + scores) and assign_values (rows only), 50 % present
+    keys = np.concatenate([recent[: bs // 2], w.unique_keys(136, 0, bs // 2)])
+    vals = w.uniform_values(137, 0, bs, dim)
+    sc = distinct(nb + 4, bs)
+    t.assign(bs, dev(keys), dev(vals), dev(sc))
+    o.assign(keys, bytes_of(vals), sc)
+    assert_same_table(t, o, dim * 4)
+    vals = w.uniform_values(138, 0, bs, dim)
+    t.assign_values(bs, dev(keys), dev(vals))
+    o.assign_values(keys, bytes_of(vals))
+    assert_same_table(t, o, dim * 4)
+    # the reading calls are the ordinary ones
+    out = torch.zeros(bs, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.find(bs, dev(keys), out, founds, None)
+    torch.cuda.synchronize()
+    ov, of, _ = o.find(keys)
+    assert (founds.cpu().numpy() == of).all() and (bytes_of(out.cpu().numpy())[of] == ov[of]).all()
+    t.close()
+
+
 def test_calls_on_two_streams_are_ordered_by_role(oracle):
     """Writers and readers on different streams: the group lock orders them the
     way the calls were issued (group_lock.cuh:43-56), without host syncs."""
