@@ -131,8 +131,12 @@ class StreamGroupLock {
     hipEvent_t ev;
     bool dirty;
   };
+  /* Updaters on different streams are ordered among themselves as well (the reference
+   * lets them overlap and pays a slot lock per key for it): an updater that is alone on
+   * the table needs no slot locks. */
   static bool conflicts(Role a, Role b) {
     if (a == kInserter || b == kInserter) return true;
+    if (a == kUpdater && b == kUpdater) return true;
     return a != b;
   }
   std::mutex mu_;
@@ -788,6 +792,23 @@ void launch_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((lookup_kernel<MODE, 1>), grid, block, 0, s, v, a);
 }
 
+template <bool LOCKFREE>
+void launch_assign(int vec, const View& v, const AssignArgs& a, hipStream_t s) {
+  const dim3 grid(grid_for(a.n)), block(kWave);
+  if (vec == 16) {
+    switch (pick_upl(v.value_bytes, 16)) {
+      case 1: hipLaunchKernelGGL((assign_kernel<16, 1, LOCKFREE>), grid, block, 0, s, v, a); break;
+      case 2: hipLaunchKernelGGL((assign_kernel<16, 2, LOCKFREE>), grid, block, 0, s, v, a); break;
+      case 4: hipLaunchKernelGGL((assign_kernel<16, 4, LOCKFREE>), grid, block, 0, s, v, a); break;
+      default: hipLaunchKernelGGL((assign_kernel<16, 8, LOCKFREE>), grid, block, 0, s, v, a); break;
+    }
+  } else if (vec == 4) {
+    hipLaunchKernelGGL((assign_kernel<4, 8, LOCKFREE>), grid, block, 0, s, v, a);
+  } else {
+    hipLaunchKernelGGL((assign_kernel<1, 8, LOCKFREE>), grid, block, 0, s, v, a);
+  }
+}
+
 template <class Pred>
 void launch_export(const hkv_table* t, uint64_t pattern, uint64_t threshold,
                    uint64_t n, uint64_t offset, uint64_t* d_counter,
@@ -1204,9 +1225,14 @@ int hkv_find_or_insert_ptr(hkv_table* t, uint64_t n, const uint64_t* keys,
   return HKV_SUCCESS;
 }
 
+/* The group lock keeps every other writer off the table while an updater runs; with unique
+ * keys the kernel then needs no slot locks.  Without the group lock (api_lock == false) other
+ * streams may carry updaters the library knows nothing of, and a repeated key has two tiles
+ * on one slot: both keep the slot locks. */
 static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
                          const void* values, const uint64_t* scores,
-                         int touch_scores, hipStream_t s) {
+                         int touch_scores, int unique_key, hipStream_t s) {
+  const bool lockfree = t->opts.api_lock && unique_key;
   AssignArgs a{};
   a.keys = keys;
   a.values = (const uint8_t*)values;
@@ -1231,7 +1257,7 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
       e = g.acquire();
       if (e == hipSuccess && touch_scores) {
         a.values = nullptr;
-        hipLaunchKernelGGL((assign_kernel<16, 1>), dim3(grid_for(n)), dim3(kWave), 0, s, t->view, a);
+        launch_assign<false>(16, t->view, a, s);
         e = hipGetLastError();
       }
       if (e == hipSuccess) e = hipMemsetAsync(d_tmp, 0, n * 9, s); /* reserved keys: no address */
@@ -1257,19 +1283,10 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
   {
     LockGuard g(t, StreamGroupLock::kUpdater, s);
     HKV_HIP(g.acquire());
-    const dim3 grid(grid_for(n)), block(kWave);
-    if (vec == 16) {
-      switch (pick_upl(t->view.value_bytes, 16)) {
-        case 1: hipLaunchKernelGGL((assign_kernel<16, 1>), grid, block, 0, s, t->view, a); break;
-        case 2: hipLaunchKernelGGL((assign_kernel<16, 2>), grid, block, 0, s, t->view, a); break;
-        case 4: hipLaunchKernelGGL((assign_kernel<16, 4>), grid, block, 0, s, t->view, a); break;
-        default: hipLaunchKernelGGL((assign_kernel<16, 8>), grid, block, 0, s, t->view, a); break;
-      }
-    } else if (vec == 4) {
-      hipLaunchKernelGGL((assign_kernel<4, 8>), grid, block, 0, s, t->view, a);
-    } else {
-      hipLaunchKernelGGL((assign_kernel<1, 8>), grid, block, 0, s, t->view, a);
-    }
+    if (lockfree)
+      launch_assign<true>(vec, t->view, a, s);
+    else
+      launch_assign<false>(vec, t->view, a, s);
     HKV_HIP(hipGetLastError());
   }
   if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
@@ -1279,27 +1296,24 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
 int hkv_assign(hkv_table* t, uint64_t n, const uint64_t* keys, const void* values,
                const uint64_t* scores, hkv_stream_t stream, int unique_key) {
   HKV_TRY(refuse_dual(t, "assign()", false));
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
-  return assign_common(t, n, keys, values, scores, 1, (hipStream_t)stream);
+  return assign_common(t, n, keys, values, scores, 1, unique_key, (hipStream_t)stream);
 }
 
 int hkv_assign_scores(hkv_table* t, uint64_t n, const uint64_t* keys,
                       const uint64_t* scores, hkv_stream_t stream, int unique_key) {
   HKV_TRY(refuse_dual(t, "assign_scores()", true));
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
   HKV_TRY(check_scores_arg(t, t->opts.evict_strategy, scores));
-  return assign_common(t, n, keys, nullptr, scores, 1, (hipStream_t)stream);
+  return assign_common(t, n, keys, nullptr, scores, 1, unique_key, (hipStream_t)stream);
 }
 
 int hkv_assign_values(hkv_table* t, uint64_t n, const uint64_t* keys,
                       const void* values, hkv_stream_t stream, int unique_key) {
   HKV_TRY(refuse_dual(t, "assign_values()", true));
-  (void)unique_key;
   if (n == 0) return HKV_SUCCESS;
-  return assign_common(t, n, keys, values, nullptr, 0, (hipStream_t)stream);
+  return assign_common(t, n, keys, values, nullptr, 0, unique_key, (hipStream_t)stream);
 }
 
 int hkv_find(const hkv_table* t, uint64_t n, const uint64_t* keys, void* values,

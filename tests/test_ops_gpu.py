@@ -415,6 +415,52 @@ def test_calls_on_two_streams_are_ordered_by_role(oracle):
     t.close()
 
 
+def test_assign_family_on_two_streams_and_with_repeated_keys(oracle):
+    """Updaters issued on different streams take effect in the order of the calls (each is
+    alone on the table, which is what lets the assign kernels run without slot locks);
+    unique_key=False keeps the slot locks: a repeated key gets one of its rows, whole."""
+    cap, dim, bs = 1 << 15, 64, 1 << 13
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    fill(t, o, 141, 3, bs, dim, lambda b, n: w.monotone_scores(b + 1, n))
+    keys = np.concatenate([w.unique_keys(141, bs, bs // 2), w.unique_keys(142, 0, bs // 2)])
+    dk = dev(keys)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    keep = []
+    torch.cuda.synchronize()
+    for r in range(6):
+        vals = w.uniform_values(143 + r, 0, bs, dim)
+        sc = w.monotone_scores(10 + r, bs)
+        dv, ds = dev(vals), dev(sc)
+        keep.append((dv, ds))
+        torch.cuda.synchronize()
+        if r % 3 == 0:
+            t.assign(bs, dk, dv, ds, stream=(s1, s2)[r % 2])
+            o.assign(keys, bytes_of(vals), sc)
+        elif r % 3 == 1:
+            t.assign_values(bs, dk, dv, stream=(s1, s2)[r % 2])
+            o.assign_values(keys, bytes_of(vals))
+        else:
+            t.assign_scores(bs, dk, ds, stream=(s1, s2)[r % 2])
+            o.assign_scores(keys, sc)
+    torch.cuda.synchronize()
+    assert_same_table(t, o, dim * 4)
+    # repeated keys: 64 copies of each of 128 resident keys, every copy with its own row
+    base = w.unique_keys(141, 2 * bs, 128)
+    rep = np.repeat(base, 64)
+    rows = np.arange(len(rep), dtype=np.float32)[:, None] + np.zeros((1, dim), np.float32)
+    t.assign_values(len(rep), dev(rep), dev(rows), unique_key=False)
+    out = torch.zeros(128, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(128, dtype=torch.bool, device=DEV)
+    t.find(128, dev(base), out, founds, None)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert founds.cpu().numpy().all()
+    assert (got == got[:, :1]).all()  # one writer's row, not a mixture
+    assert ((got[:, 0] // 64).astype(np.int64) == np.arange(128)).all()
+    t.close()
+
+
 def test_error_classes(oracle):
     t = HashTable()
     t.init(default_options(init_capacity=1024, max_capacity=1024, max_hbm_for_vectors=1 << 30, dim=4,
