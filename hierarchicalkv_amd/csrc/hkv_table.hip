@@ -586,7 +586,11 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
     if (plan.feasible) {
       if constexpr (OP != kOpFindOrInsertPtr)
         HKV_TRY(run_grouped<OP>(t, a, vec, refuse_equal, plan, s));
-    } else if (refuse_equal || t->keys_may_be_locked) {
+    } else if (t->keys_may_be_locked) {
+      /* slots that lock_keys (or the pointer overload with locked_key_ptrs) left LOCKED must
+       * be hidden from the victim scan, which then reads the key words beside the scores; with
+       * no such slot the plain scan finds the same victims (a slot locked by another key of
+       * the batch is retried instead of skipped) */
       launch_upsert<OP, true>(vec, t->view, a, s);
     } else {
       launch_upsert<OP, false>(vec, t->view, a, s);
