@@ -379,9 +379,12 @@ __device__ __forceinline__ void bulk_rows(int move, uint8_t* tab, uint8_t* usr,
           x[q][w] = T{};
           if (u < units) {
             if (mv == kMoveInToTable) x[q][w] = ld_unit<VEC, false>(us, u);
-            if (CAN_READ_TABLE && mv == kMoveTableToIo) x[q][w] = ld_unit<VEC, true>(tb, u);
+            /* the row of a key that was found was last written before this launch (keys are
+             * unique, so no other key of the batch has touched it): an ordinary streaming
+             * load, one 16-byte access instead of the two 8-byte coherent ones */
+            if (CAN_READ_TABLE && mv == kMoveTableToIo) x[q][w] = ld_unit<VEC, false>(tb, u);
             if (CAN_ACCUM && mv == kMoveAccum) {
-              x[q][w] = ld_unit<VEC, true>(tb, u);
+              x[q][w] = ld_unit<VEC, false>(tb, u);
               y[q][w] = ld_unit<VEC, false>(us, u);
             }
           }
@@ -699,15 +702,17 @@ upsert_kernel(View v, UpsertArgs a) {
       if (votes) {
         const int leader = (int)__ffsll(votes) - 1;
         unsigned long long base_idx = 0;
-        if (lane == leader)
+        if (HKV_EXP_FLAG(128))
+          base_idx = (unsigned long long)blockIdx.x * 32;
+        else if (lane == leader)
           base_idx = atomicAdd(a.evicted_counter, (unsigned long long)__popcll(votes));
         base_idx = __shfl(base_idx, leader);
         const unsigned long long idx = base_idx + __popcll(votes & ((1ull << lane) - 1));
-        if (emit) {
+        if (emit && !HKV_EXP_FLAG(64)) {
           a.evicted_keys[idx] = refused_now ? key : victim;
           if (a.evicted_scores) a.evicted_scores[idx] = refused_now ? desired : best;
         }
-        bulk_evicted<VEC, UPL>(emit ? (refused_now ? 1 : 2) : 0,
+        bulk_evicted<VEC, UPL>(emit && !HKV_EXP_FLAG(32) ? (refused_now ? 1 : 2) : 0,
                                refused_now ? a.values_in + i * v.value_bytes : row,
                                a.evicted_values + idx * v.value_bytes, units, lane);
       }
