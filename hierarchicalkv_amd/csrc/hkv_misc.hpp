@@ -55,11 +55,18 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
 /* Sum of the per-bucket sizes (SumOp over buckets_size, core_kernels.cuh:1395-1423) */
 __global__ void __launch_bounds__(256)
 size_kernel(View v, unsigned long long* out) {
+  /* the array starts on a 256-byte boundary: four counters per load, the tail one by one;
+   * few blocks, because the one word they all add to takes one update at a time */
   uint64_t local = 0;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t b = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-       b < v.buckets_num; b += stride)
-    local += (uint64_t)v.sizes[b];
+  const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint64_t quads = v.buckets_num / 4;
+  const int4* q = reinterpret_cast<const int4*>(v.sizes);
+  for (uint64_t b = tid; b < quads; b += stride) {
+    const int4 x = q[b];
+    local += (uint64_t)x.x + (uint64_t)x.y + (uint64_t)x.z + (uint64_t)x.w;
+  }
+  for (uint64_t b = quads * 4 + tid; b < v.buckets_num; b += stride) local += (uint64_t)v.sizes[b];
   __shared__ unsigned long long s_part[4];
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;

@@ -1578,7 +1578,7 @@ int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out) {
     HKV_HIP(g.acquire());
     hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
     const unsigned blocks =
-        (unsigned)std::min<uint64_t>((t->view.buckets_num + 255) / 256, 2048);
+        (unsigned)std::min<uint64_t>((t->view.buckets_num + 4095) / 4096, 128);
     hipLaunchKernelGGL(size_kernel, dim3(blocks), dim3(256), 0, s, t->view, d);
     HKV_HIP(hipGetLastError());
   }
