@@ -902,8 +902,8 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->io_by_cpu = o->io_by_cpu != 0;
   t->io_stage = nullptr;
   t->io_stage_bytes = 0;
-  /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default while the
-   * two-phase path is being tuned), "auto" = two-phase for large batches,
+  /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default: it is the faster
+   * one per find + insert_or_assign step), "auto" = two-phase for large batches,
    * "grouped" = two-phase whenever it is possible (tests) */
   t->upsert_path = 1;
   if (const char* e = getenv("HKV_UPSERT_PATH")) {

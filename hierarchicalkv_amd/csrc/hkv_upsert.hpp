@@ -762,8 +762,9 @@ upsert_kernel(View v, UpsertArgs a) {
 
 /* ---- assign family: update keys that are present, never insert -----------------
  * The score rule is ScoreFunctor::update_without_missed (kernel_utils.cuh:
- * 304-321, 373-392, 436-453, 519-557, 594-612).  Several updaters may run at
- * once (the group lock lets them), so the row changes under the slot lock. */
+ * 304-321, 373-392, 436-453, 519-557, 594-612).  Without the group lock several
+ * updaters may run at once, and a batch may repeat a key: then the row changes under
+ * the slot lock (LOCKFREE == false). */
 
 struct AssignArgs {
   const uint64_t* keys;

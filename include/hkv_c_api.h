@@ -98,7 +98,7 @@ typedef struct hkv_options {
   int32_t evict_strategy; /* hkv_evict_strategy */
   int32_t value_kind;     /* hkv_value_kind */
   uint32_t value_size;    /* sizeof(V) */
-  uint32_t score_size;    /* sizeof(S): 8 (4 is not supported yet) */
+  uint32_t score_size;    /* sizeof(S): 8 (the C++ header maps S = uint32_t onto it) */
 } hkv_options;
 
 /* Raw device layout of a table, for kernels compiled outside the library
