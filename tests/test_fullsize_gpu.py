@@ -150,6 +150,33 @@ def test_config2_throughput_shape_full_size(path, monkeypatch):
         assert torch.equal(io[n // 2:], value_of(fresh2, dim))
         t.find(n // 2, fresh2, out[: n // 2], founds[: n // 2])
         assert bool(founds[: n // 2].all()) and torch.equal(out[: n // 2], value_of(fresh2, dim))
+        # assign (no slot locks: the updater is alone on the table): present keys get the new
+        # rows, absent keys are not inserted
+        absent = dev_keys(seed + 17, pos, n // 2)
+        batch3 = torch.cat([fresh2, absent])
+        rows3 = value_of(batch3, dim) + 0.25
+        before = t.size()
+        t.assign(n, batch3, rows3)
+        assert t.size() == before
+        t.find(n, batch3, out, founds)
+        assert bool(founds[: n // 2].all()) and not bool(founds[n // 2:].any())
+        assert torch.equal(out[: n // 2], rows3[: n // 2])
+        # find_or_insert*: pointers to the rows of present and new keys
+        fresh3 = dev_keys(seed, pos, n // 2)
+        pos += n // 2
+        batch4 = torch.cat([fresh2, fresh3])
+        ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+        t.find_or_insert_ptr(n, batch4, ptrs, founds)
+        assert bool(founds[: n // 2].all()) and not bool(founds[n // 2:].any())
+        assert bool((ptrs != 0).all())
+        v = t.view()
+        off = ptrs - v.values
+        assert bool(((off >= 0) & (off < cap * dim * 4) & (off % (dim * 4) == 0)).all())
+        assert int(torch.unique(off).numel()) == n  # one row per key
+        t.assign_values(n // 2, fresh3, value_of(fresh3, dim))  # rows of the new keys, as a caller would
+        t.find(n, batch4, out, founds)
+        assert bool(founds.all())
+        assert torch.equal(out, torch.cat([rows3[: n // 2], value_of(fresh3, dim)]))
     # the table holds each key once, and as many as it says
     keys, _ = export_keys(t, dim * 4)
     uniq, total = device_unique_count(keys)
