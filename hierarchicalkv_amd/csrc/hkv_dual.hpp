@@ -16,8 +16,10 @@
  *   phase 2  otherwise the minimum score over both buckets decides: the key is
  *            refused when its score is below it, else the slot holding the
  *            minimum is locked (b1 when min1 <= min2), its score is checked
- *            again under the lock and the attempt repeats when it moved.
- * A tile holds at most one lock and never waits while holding it.
+ *            again under the lock and the attempt repeats when it moved or the
+ *            slot was held by another tile.
+ * A tile holds at most one lock, and finishes with it (row written, key word released)
+ * at the place where it took it.
  *
  * find replaces dual_bucket_pipeline_lookup_kernel_with_io
  * (dual_bucket_lookup.cuh:25-140): lookup_kernel probes b1 for the 64 keys of
@@ -107,12 +109,14 @@ dual_upsert_kernel(View v, UpsertArgs a) {
         if (j == 0) {
           uint64_t expect = v.empty_key;
           ok = cas_lock(v.keys + (uint64_t)bkt * kBucketSize + p, expect, v.locked_key) ? 1 : 0;
+          /* counted at once, not when the row is in: the other keys in flight choose their
+           * bucket by these counters, and a stale count sends them to the fuller one */
+          if (ok) atomicAdd(v.sizes + bkt, 1);
         }
         ok = tile_bcast(ok, tile, 0);
         if (ok) {
           slot = (int64_t)bkt * kBucketSize + p;
           is_new = true;
-          grew = true;
           break;
         }
         if (p < 64)
@@ -123,53 +127,78 @@ dual_upsert_kernel(View v, UpsertArgs a) {
     }
   }
 
-  /* phase 2: the minimum score of both buckets */
-  if (slot < 0) {
-    for (int tries = 0; tries < kDualMaxTries; tries++) {
+  /* The critical section of the lock this tile holds: digest and score, the row, and the
+   * release of the key word.  It runs right where the lock was taken, before any tile of this
+   * wavefront goes round the retry loop below again: a tile that still looks for a victim may
+   * be waiting for exactly this lock, and lanes that have left a loop do not run again until
+   * the other lanes have left it too. */
+  auto commit = [&](int64_t at) {
+    if (j == 0) {
+      write_meta(v, a, (uint64_t)at, L.digest, desired, in_score, i, is_new);
+      if (grew) atomicAdd(v.sizes + ((uint64_t)at >> 7), 1);
+    }
+    tile_copy<VEC, true, false>(value_row(v, (uint64_t)at),
+                                a.values_in + i * (uint64_t)v.value_bytes, v.value_bytes, j);
+    wait_stores();
+    if (j == 0) st_unlock(v.keys + at, key);
+  };
+  bool pending = true;
+  if (slot >= 0) {
+    commit(slot);
+    pending = false; /* no return here: the order of this block and the loop below must not be
+                        left to the compiler's layout of two independent branches */
+  }
+
+  /* phase 2: the minimum score of both buckets.  The scan reads scores only: a slot that
+   * another tile holds shows the score it had (it is retried until the tile has released it
+   * with its new score), so the outcome is that of handling the keys one after the other in
+   * some order. */
+  for (int tries = 0; tries < kDualMaxTries && __ballot(pending) != 0; tries++) {
+    int ok = 0; /* 1: a key is evicted, 2: the slot was free or a tombstone */
+    uint64_t vs = 0;
+    if (pending) {
       uint64_t best[2];
       uint32_t pos[2];
 #pragma unroll
       for (int w = 0; w < 2; w++) {
-        uint64_t sc[2 * kTile], kc[2 * kTile];
-        scan_load<true>(v, (uint64_t)L.bkt[w] * kBucketSize, j, sc, kc);
-        scan_reduce<true>(v, sc, kc, j, best[w], pos[w]);
+        uint64_t sc[2 * kTile], kc[1];
+        scan_load<false>(v, (uint64_t)L.bkt[w] * kBucketSize, j, sc, kc);
+        scan_reduce<false>(v, sc, kc, j, best[w], pos[w]);
       }
       const int w = best[0] <= best[1] ? 0 : 1;
       const uint64_t mn = w == 0 ? best[0] : best[1];
-      if (mn == kMaxScore) continue; /* every slot is under another tile's lock right now */
-      if (desired < mn) break;       /* refused */
-      const uint64_t vs = (uint64_t)(w == 0 ? L.bkt[0] : L.bkt[1]) * kBucketSize + (w == 0 ? pos[0] : pos[1]);
-      const uint64_t vk = ld_u64(v.keys + vs);
-      if (vk == v.locked_key || vk == v.empty_key) continue;
-      int ok = 0;
-      if (j == 0) {
-        uint64_t expect = vk;
-        if (cas_lock(v.keys + vs, expect, v.locked_key)) {
-          if (ld_u64(v.scores + vs) <= mn)
-            ok = 1;
-          else
+      if (desired < mn) {
+        pending = false; /* refused */
+      } else {
+        vs = (uint64_t)(w == 0 ? L.bkt[0] : L.bkt[1]) * kBucketSize + (w == 0 ? pos[0] : pos[1]);
+        if (j == 0) {
+          const uint64_t vk = swap_lock(v.keys + vs, v.locked_key);
+          if (vk == v.locked_key) {
+            /* held by another tile; look again */
+          } else if (vk == v.empty_key) {
+            ok = 2; /* freed or never filled: an insert into a free slot after all */
+          } else if (ld_u64(v.scores + vs) <= mn) {
+            ok = vk == v.reclaim_key ? 2 : 1;
+          } else {
             st_unlock(v.keys + vs, vk); /* the score moved: not the minimum any more */
+          }
         }
-      }
-      ok = tile_bcast(ok, tile, 0);
-      if (ok) {
-        slot = (int64_t)vs;
-        is_new = true;
-        grew = vk == v.reclaim_key;
-        break;
+        ok = tile_bcast(ok, tile, 0);
       }
     }
+    if (ok) {
+      is_new = true;
+      grew = ok == 2;
+      commit((int64_t)vs);
+      pending = false;
+    }
+    /* the loop is left by all lanes of the wavefront together, so the commit above is never
+     * deferred to a point after the loop */
+    if (__ballot(pending) == 0) break;
+    __builtin_amdgcn_s_sleep(1);
   }
-  if (slot < 0) return; /* refused */
-
-  if (j == 0) {
-    write_meta(v, a, (uint64_t)slot, L.digest, desired, in_score, i, is_new);
-    if (grew) atomicAdd(v.sizes + ((uint64_t)slot >> 7), 1);
-  }
-  tile_copy<VEC, true, false>(value_row(v, (uint64_t)slot),
-                              a.values_in + i * (uint64_t)v.value_bytes, v.value_bytes, j);
-  wait_stores();
-  if (j == 0) st_unlock(v.keys + slot, key);
+  /* still pending here: given up and treated as refused (the buckets kept changing under
+   * kDualMaxTries looks) */
 }
 
 }  // namespace hkv

@@ -765,14 +765,29 @@ int maybe_dedup(const hkv_table* t, int unique_key, uint64_t n, const uint64_t*&
   return HKV_SUCCESS;
 }
 
-void launch_dual_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)((a.n + kTilesPerWave - 1) / kTilesPerWave)), block(kWave);
-  if (vec == 16)
-    hipLaunchKernelGGL((dual_upsert_kernel<16>), grid, block, 0, s, v, a);
-  else if (vec == 4)
-    hipLaunchKernelGGL((dual_upsert_kernel<4>), grid, block, 0, s, v, a);
-  else
-    hipLaunchKernelGGL((dual_upsert_kernel<1>), grid, block, 0, s, v, a);
+/* Where a key lands depends on the bucket sizes the moment it is handled, and the keys in
+ * flight at once decide on counts that miss each other's claims.  With many buckets that is
+ * noise; on a small table (the reference tests 1024 buckets with batches of 2^17 keys) it
+ * unbalances the two-choice placement enough to drop keys while free slots remain (size after
+ * the first such batch 129 085 against 130 726 for keys handled one by one).  So a batch goes in
+ * as launches of at most 16 keys per bucket: one launch for any table of realistic size. */
+void launch_dual_upsert(int vec, const View& v, const UpsertArgs& whole, hipStream_t s) {
+  const uint64_t chunk = std::max<uint64_t>(v.buckets_num * 16, 4096);
+  for (uint64_t off = 0; off < whole.n; off += chunk) {
+    UpsertArgs a = whole;
+    a.n = std::min<uint64_t>(chunk, whole.n - off);
+    a.keys += off;
+    a.values_in += off * v.value_bytes;
+    if (a.scores) a.scores += off;
+    if (a.clock.mode == 1) a.clock.base += off << 20; /* the deterministic clock: base + (index << 20) */
+    const dim3 grid((unsigned)((a.n + kTilesPerWave - 1) / kTilesPerWave)), block(kWave);
+    if (vec == 16)
+      hipLaunchKernelGGL((dual_upsert_kernel<16>), grid, block, 0, s, v, a);
+    else if (vec == 4)
+      hipLaunchKernelGGL((dual_upsert_kernel<4>), grid, block, 0, s, v, a);
+    else
+      hipLaunchKernelGGL((dual_upsert_kernel<1>), grid, block, 0, s, v, a);
+  }
 }
 
 void launch_dual_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {

@@ -265,10 +265,10 @@ def test_eviction_quality_and_consistency_at_full_load(oracle):
     ideal = set(keys[np.argsort(scores)[::-1][:len(ek)]].tolist())
     quality = sum(1 for k in ek.tolist() if k in ideal) / len(ek)
     print(f"dual-bucket eviction quality {quality:.4f}, load factor {len(ek) / cap:.4f}")
-    # The reference's bound is 0.995.  Which keys survive depends on the order in which the keys
-    # of a batch are handled: the host oracle gives 0.9952 to 0.9956 over random orders of these
-    # batches, the kernel (whose order changes from run to run) has measured 0.9949 to 0.9956.
-    assert quality >= 0.994
+    # The reference's bound.  Which keys survive depends on the order in which the keys of a batch
+    # are handled: the host oracle gives 0.9952 to 0.9956 over random orders of these batches, the
+    # kernel (whose order changes from run to run) has measured 0.9953 to 0.9958.
+    assert quality >= 0.995
     # residents carry their own score and row, and find sees exactly the exported set
     assert np.array_equal(es, scores[ek.astype(np.int64) - 1])
     assert np.array_equal(ev, bytes_of(w.values_from_keys(ek, dim)))
