@@ -782,6 +782,124 @@ static void test_dual_bucket_mode() {
 }
 
 
+// io_by_cpu (tests/merlin_hashtable_test.cc.cu:1760-1905, test_basic_for_cpu_io): every row in
+// pinned host memory, the rows of the writers moved by host threads; the same sequence of calls
+// and counts, plus a check of the rows the reference's test leaves out.
+static void test_basic_for_cpu_io() {
+  constexpr size_t DIM = 16, CAP = 1 << 20, N = 1 << 16;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.reserved_key_start_bit = 10;
+  o.max_hbm_for_vectors = GB(0);
+  o.io_by_cpu = true;
+  using Table = HashTable<K, V, S, EvictStrategy::kCustomized>;
+  {
+    HashTableOptions bad = o;
+    bad.max_hbm_for_vectors = GB(1);  // merlin_hashtable.cuh:1071-1073
+    Table t;
+    bool threw = false;
+    try {
+      t.init(bad);
+    } catch (const MerlinException&) {
+      threw = true;
+    }
+    CHECK(threw);
+  }
+  Table table;
+  table.init(o);
+  hipStream_t stream;
+  HIP(hipStreamCreate(&stream));
+  CHECK(table.size(stream) == 0);
+  std::vector<K> keys;
+  {
+    // the reserved keys sit at bit 10 on this table (types.cuh:80-109)
+    std::mt19937_64 rng(77);
+    std::unordered_set<K> seen;
+    const K mask = ~(UINT64_C(3) << 10) & ~UINT64_C(1);
+    while (keys.size() < N) {
+      K k = rng();
+      if ((k & mask) == mask) continue;
+      if (seen.insert(k).second) keys.push_back(k);
+    }
+  }
+  std::vector<S> scores(N);
+  std::iota(scores.begin(), scores.end(), 1);
+  std::vector<V> ones(N * DIM, 1.0f), twos(N * DIM, 2.0f);
+  DevBuf<K> dk(N), dko(CAP);
+  DevBuf<V> dv(N * DIM), dout(N * DIM), dvo(CAP * DIM);
+  DevBuf<S> ds(N), dso(CAP);
+  DevBuf<bool> df(N);
+  dk.up(keys);
+  ds.up(scores);
+  dv.up(ones);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p, stream);
+  CHECK(table.size(stream) == N);
+  dv.up(twos);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p, stream);
+  CHECK(table.size(stream) == N);
+  table.find(N, dk.p, dout.p, df.p, nullptr, stream);
+  HIP(hipStreamSynchronize(stream));
+  {
+    auto f = df.down(N);
+    auto out = dout.down(N * DIM);
+    size_t found = 0;
+    bool same = true;
+    for (size_t i = 0; i < N; i++) found += f[i];
+    for (size_t i = 0; i < N * DIM; i++) same &= out[i] == 2.0f;
+    CHECK(found == N);
+    CHECK(same);
+  }
+  HIP(hipMemsetAsync(df.p, 0, N, stream));
+  table.contains(N, dk.p, df.p, stream);
+  HIP(hipStreamSynchronize(stream));
+  {
+    auto f = df.down(N);
+    size_t n = 0;
+    for (size_t i = 0; i < N; i++) n += f[i];
+    CHECK(n == N);
+  }
+  table.accum_or_assign(N, dk.p, dv.p, df.p, ds.p, stream);  // every flag says accumulate: 2 + 2
+  CHECK(table.size(stream) == N);
+  // find_or_insert: the first half is there (rows come back), the second half is new
+  {
+    auto more = random_keys(N / 2, 78);
+    std::vector<K> mixed(keys.begin(), keys.begin() + N / 2);
+    mixed.insert(mixed.end(), more.begin(), more.end());
+    DevBuf<K> dm(N);
+    dm.up(mixed);
+    std::vector<V> io(N * DIM, 7.0f);
+    DevBuf<V> dio(N * DIM);
+    dio.up(io);
+    table.find_or_insert(N, dm.p, dio.p, ds.p, stream);
+    HIP(hipStreamSynchronize(stream));
+    auto back = dio.down(N * DIM);
+    bool same = true;
+    for (size_t i = 0; i < N / 2 * DIM; i++) same &= back[i] == 4.0f;
+    for (size_t i = N / 2 * DIM; i < N * DIM; i++) same &= back[i] == 7.0f;
+    CHECK(same);
+    CHECK(table.size(stream) == N + N / 2);
+    table.assign_values(N / 2, dm.p + N / 2, dv.p, stream);  // the new keys get rows of 2.0
+    table.find(N, dm.p, dout.p, df.p, nullptr, stream);
+    HIP(hipStreamSynchronize(stream));
+    auto out = dout.down(N * DIM);
+    same = true;
+    for (size_t i = 0; i < N / 2 * DIM; i++) same &= out[i] == 4.0f;
+    for (size_t i = N / 2 * DIM; i < N * DIM; i++) same &= out[i] == 2.0f;
+    CHECK(same);
+    table.erase(N / 2, dm.p + N / 2, stream);
+  }
+  table.erase(N >> 1, dk.p, stream);
+  CHECK(table.size(stream) == N >> 1);
+  table.clear(stream);
+  CHECK(table.size(stream) == 0);
+  table.insert_or_assign(N, dk.p, dv.p, ds.p, stream);
+  size_t dumped = table.export_batch(table.capacity(), 0, dko.p, dvo.p, dso.p, stream);
+  HIP(hipStreamSynchronize(stream));
+  CHECK(dumped == N);
+  HIP(hipStreamDestroy(stream));
+}
+
 // S = uint32_t (tests/uint32_score_test.cc.cu:48-186): find_or_insert + find return the
 // 32-bit scores handed in, missing keys leave the caller's score entries alone,
 // assign_scores + export_batch round-trip, insert_and_evict hands back 32-bit scores.
@@ -889,6 +1007,7 @@ int main() {
     test_functor_forms();
     test_dual_bucket_mode();
     test_uint32_scores();
+    test_basic_for_cpu_io();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
