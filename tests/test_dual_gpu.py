@@ -289,3 +289,104 @@ def test_eviction_quality_and_consistency_at_full_load(oracle):
     _, gf, _ = gpu_find(t, lowk, dim)
     assert not gf.any()
     t.close()
+
+
+def test_score_ordering_after_eviction():
+    # tests/dual_bucket_test.cc.cu:822-935: a full table of scores 1..N, then 512 keys with far
+    # higher scores; survivors among them carry their score, and some survive
+    cap, dim, n_new = 128 * 64, 8, 512
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    keys = np.arange(1, cap + 1, dtype=np.uint64)
+    t.insert_or_assign(cap, dev(keys), dev(np.ones((cap, dim), np.float32)), dev(keys.copy()))
+    newk = np.arange(cap + 1, cap + 1 + n_new, dtype=np.uint64)
+    news = np.uint64(cap * 10) + np.arange(n_new, dtype=np.uint64)
+    t.insert_or_assign(n_new, dev(newk), dev(np.full((n_new, dim), 2.0, np.float32)), dev(news))
+    ek, ev, es = export_table(t, dim * 4)
+    assert len(ek) == t.size()
+    high = ek > cap
+    assert high.sum() == n_new  # every bucket pair held lower scores: none of them is refused
+    assert (es[high] >= es.min()).all()
+    assert np.array_equal(es[high], news[(ek[high] - np.uint64(cap + 1)).astype(np.int64)])
+    assert (ev[high].view(np.float32) == 2.0).all() and (ev[~high].view(np.float32) == 1.0).all()
+    # the keys that made room are the lowest-scored ones of the bucket pairs they shared: nothing
+    # above the lowest survivor of the old keys can be missing by more than the new keys' count
+    assert len(ek) <= cap and len(ek) >= cap - n_new
+    t.close()
+
+
+def test_multi_stream_upserts():
+    # tests/dual_bucket_test.cc.cu:1527-1660 (four streams, disjoint key ranges, each a full
+    # capacity) and :1666-1757 (four streams, the same keys with different scores)
+    cap, dim, n_streams = 128 * 1024, 8, 4
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    streams = [torch.cuda.Stream() for _ in range(n_streams)]
+    rng = np.random.default_rng(42)
+    keep = []
+    torch.cuda.synchronize()
+    for s, st in enumerate(streams):
+        k = np.arange(s * cap + 1, (s + 1) * cap + 1, dtype=np.uint64)
+        sc = (rng.integers(0, 1 << 63, cap, dtype=np.uint64) >> np.uint64(1)) | np.uint64(1)
+        bufs = (dev(k), dev(np.full((cap, dim), float(s + 1), np.float32)), dev(sc))
+        keep.append(bufs)
+        torch.cuda.synchronize()
+        t.insert_or_assign(cap, *bufs, stream=st)
+    torch.cuda.synchronize()
+    ek, ev, es = export_table(t, dim * 4)
+    assert len(ek) == t.size() and 0 < len(ek) <= cap
+    assert len(np.unique(ek)) == len(ek), "duplicate keys in the table"
+    gv, gf, gs = gpu_find(t, ek, dim)
+    assert gf.all() and np.array_equal(gs, es) and np.array_equal(gv, ev)
+    # rows belong to the stream that inserted the key
+    assert np.array_equal(ev.view(np.float32)[:, 0], ((ek - np.uint64(1)) // np.uint64(cap) + np.uint64(1)).astype(np.float32))
+    t.close()
+    # the same keys from every stream
+    n = 32768
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    k = np.arange(1, n + 1, dtype=np.uint64)
+    keep = []
+    torch.cuda.synchronize()
+    for s, st in enumerate(streams):
+        sc = np.uint64((s + 1) * 1000) + np.arange(n, dtype=np.uint64)
+        bufs = (dev(k), dev(np.full((n, dim), float(s + 1), np.float32)), dev(sc))
+        keep.append(bufs)
+        torch.cuda.synchronize()
+        t.insert_or_assign(n, *bufs, stream=st)
+    torch.cuda.synchronize()
+    assert t.size() == n  # no key twice
+    gv, gf, gs = gpu_find(t, k, dim)
+    assert gf.all()
+    # the inserter role orders the calls as they were issued: the last stream's rows and scores stay
+    assert (gv.view(np.float32) == float(n_streams)).all()
+    assert np.array_equal(gs, np.uint64(n_streams * 1000) + np.arange(n, dtype=np.uint64))
+    t.close()
+
+
+def test_find_without_scores_and_clear_then_reinsert():
+    # tests/dual_bucket_test.cc.cu:1763-1835 (find with scores = nullptr) and :1841-1920
+    cap, dim, n = 128 * 64, 8, 4096
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    keys = np.arange(1, n + 1, dtype=np.uint64)
+    vals = w.values_from_keys(keys, dim)
+    t.insert_or_assign(n, dev(keys), dev(vals), dev(keys.copy()))
+    q = np.concatenate([keys[:1000], np.arange(10 ** 9, 10 ** 9 + 24, dtype=np.uint64)])
+    out = torch.zeros(len(q), dim, dtype=torch.float32, device=DEV)
+    f = torch.zeros(len(q), dtype=torch.bool, device=DEV)
+    t.find(len(q), dev(q), out, f, None)
+    torch.cuda.synchronize()
+    gf = f.cpu().numpy()
+    assert gf[:1000].all() and not gf[1000:].any()
+    assert np.array_equal(out.cpu().numpy()[:1000], vals[:1000])
+    t.clear()
+    assert t.size() == 0
+    _, gf, _ = gpu_find(t, keys, dim)
+    assert not gf.any()
+    t.insert_or_assign(n, dev(keys), dev(vals + 1), dev(keys + np.uint64(5)))
+    assert t.size() == n
+    gv, gf, gs = gpu_find(t, keys, dim)
+    assert gf.all() and np.array_equal(gs, keys + np.uint64(5))
+    assert np.array_equal(gv, bytes_of(vals + 1))
+    t.close()
