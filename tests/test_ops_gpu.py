@@ -741,3 +741,53 @@ def test_find_or_insert_with_locked_key_pointers(oracle):
     ok_, _, os_ = sort_by_key(*o.export_all())
     assert np.array_equal(gk, ok_) and np.array_equal(gs, os_)
     t.close()
+
+
+def test_growth_under_host_threads():
+    """tests/merlin_hashtable_test.cc.cu:1441-1580 (test_dynamic_rehash_on_multi_threads): eight
+    host threads, each on its own stream, insert and look up 256 keys at a time while the table
+    grows from 32 buckets by repeated rehash; every thread finds what it has just inserted."""
+    import threading
+    init_cap, dim, n, n_threads = 4 * 1024 - 128 - 1, 16, 256, 8
+    max_cap = 1024 * init_cap
+    t = HashTable()
+    t.init(default_options(init_capacity=init_cap, max_capacity=max_cap, dim=dim, reserved_key_start_bit=8,
+                           num_of_buckets_per_alloc=16, max_load_factor=0.5, max_hbm_for_vectors=1 << 34,
+                           evict_strategy=EvictStrategy.kLru))
+    assert t.bucket_count() == 32
+    errors, rounds = [], [0] * n_threads
+
+    def worker(tid):
+        try:
+            torch.cuda.set_device(0)
+            st = torch.cuda.Stream()
+            pos = 0
+            while t.capacity() * 2 < max_cap:
+                keys = w.unique_keys(1000 + tid, pos, n)
+                pos += n
+                vals = w.values_from_keys(keys, dim)
+                dk, dv = dev(keys), dev(vals)
+                out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+                founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+                f2 = torch.zeros(n, dtype=torch.bool, device=DEV)
+                torch.cuda.current_stream().synchronize()
+                t.insert_or_assign(n, dk, dv, None, stream=st)
+                st.synchronize()
+                t.find(n, dk, out, founds, None, stream=st)
+                t.contains(n, dk, f2, stream=st)
+                st.synchronize()
+                assert bool(founds.all()) and bool(f2.all()), (tid, rounds[tid])
+                assert np.array_equal(out.cpu().numpy(), vals), (tid, rounds[tid])
+                rounds[tid] += 1
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(n_threads)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors[:3]
+    assert t.capacity() * 2 >= max_cap and min(rounds) > 0
+    assert t.size() <= sum(rounds) * n
+    t.close()
