@@ -900,6 +900,77 @@ static void test_basic_for_cpu_io() {
   HIP(hipStreamDestroy(stream));
 }
 
+// save -> load into a second table, for every strategy (tests/save_and_load_test.cc.cu:30-120):
+// the tables hold the same keys and rows afterwards, and the same scores where the caller
+// supplies them (LRU and EpochLRU scores are clock readings of the loading call).
+template <class Table>
+static std::map<K, std::pair<std::vector<V>, S>> table_contents(Table& t, size_t dim) {
+  const size_t cap = t.capacity();
+  DevBuf<K> dk(cap);
+  DevBuf<V> dv(cap * dim);
+  DevBuf<S> ds(cap);
+  const size_t n = t.export_batch(cap, 0, dk.p, dv.p, ds.p);
+  auto k = dk.down(n);
+  auto v = dv.down(n * dim);
+  auto sc = ds.down(n);
+  std::map<K, std::pair<std::vector<V>, S>> m;
+  for (size_t i = 0; i < n; i++)
+    m[k[i]] = {std::vector<V>(v.begin() + i * dim, v.begin() + (i + 1) * dim), sc[i]};
+  return m;
+}
+template <int Strategy>
+static void run_save_and_load() {
+  constexpr size_t DIM = 8, CAP = 1 << 17, N = 1 << 16;
+  using Table = HashTable<K, V, S, Strategy>;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  auto keys = random_keys(N, 500 + Strategy);
+  auto vals = values_of(keys, DIM);
+  std::vector<S> scores(N);
+  std::iota(scores.begin(), scores.end(), 1000);
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM);
+  DevBuf<S> ds(N);
+  dk.up(keys);
+  dv.up(vals);
+  ds.up(scores);
+  Table t0, t1;
+  t0.init(o);
+  t1.init(o);
+  constexpr bool clocked = Strategy == EvictStrategy::kLru || Strategy == EvictStrategy::kEpochLru;
+  t0.set_global_epoch(101);
+  t0.insert_or_assign(N, dk.p, dv.p, clocked ? nullptr : ds.p);
+  CHECK(t0.size() == N);
+  LocalKVFile<K, V, S> file;
+  CHECK(file.open("/tmp/hkv_sl_k.bin", "/tmp/hkv_sl_v.bin", "/tmp/hkv_sl_s.bin", "wb"));
+  CHECK(t0.save(&file, 64 * 1024) == N);  // a small work space: many windows
+  file.close();
+  CHECK(file.open("/tmp/hkv_sl_k.bin", "/tmp/hkv_sl_v.bin", "/tmp/hkv_sl_s.bin", "rb"));
+  CHECK(t1.load(&file, 48 * 1024) == N);
+  file.close();
+  auto a = table_contents(t0, DIM), b = table_contents(t1, DIM);
+  CHECK(a.size() == N && b.size() == N);
+  bool same = a.size() == b.size();
+  for (auto& kv : a) {
+    auto it = b.find(kv.first);
+    if (it == b.end() || it->second.first != kv.second.first) {
+      same = false;
+      break;
+    }
+    if (it->second.second != kv.second.second) same = false;  // load keeps the saved scores
+  }
+  CHECK(same);
+}
+static void test_save_and_load_all_strategies() {
+  run_save_and_load<EvictStrategy::kLru>();
+  run_save_and_load<EvictStrategy::kLfu>();
+  run_save_and_load<EvictStrategy::kEpochLru>();
+  run_save_and_load<EvictStrategy::kEpochLfu>();
+  run_save_and_load<EvictStrategy::kCustomized>();
+}
+
 // S = uint32_t (tests/uint32_score_test.cc.cu:48-186): find_or_insert + find return the
 // 32-bit scores handed in, missing keys leave the caller's score entries alone,
 // assign_scores + export_batch round-trip, insert_and_evict hands back 32-bit scores.
@@ -1008,6 +1079,7 @@ int main() {
     test_dual_bucket_mode();
     test_uint32_scores();
     test_basic_for_cpu_io();
+    test_save_and_load_all_strategies();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
