@@ -514,19 +514,21 @@ static void decide(const hkvo_table* t, int strategy, uint64_t key,
   const uint64_t* k = t->keys + r->bkt * BUCKET;
   const uint64_t* s = t->scores + r->bkt * BUCKET;
   const int full = t->sizes[r->bkt] == (int32_t)BUCKET;
+  /* The reference meets the key before any EMPTY slot when it probes from the start
+   * position, because its rehash compacts a bucket after moving keys out of it
+   * (defragmentation_for_rehash, core_kernels.cuh:445-492).  The rehash here leaves
+   * the holes where they are, so the key is looked for in the whole bucket first. */
+  for (uint32_t p = 0; p < BUCKET; p++) {
+    if (d[p] == r->digest && k[p] == key) {
+      r->result = OCC_DUPLICATE;
+      r->pos = p;
+      return;
+    }
+  }
   uint32_t base = start & ~15u;
-  for (uint32_t off = 0; off < BUCKET + 16; off += 16) {
+  for (uint32_t off = 0; !full && off < BUCKET + 16; off += 16) {
     uint32_t cur = (base + off) & (BUCKET - 1);
     for (uint32_t w = 0; w < 4; w++) {
-      for (uint32_t b = 0; b < 4; b++) {
-        uint32_t p = cur + w * 4 + b;
-        if (d[p] == r->digest && k[p] == key) {
-          r->result = OCC_DUPLICATE;
-          r->pos = p;
-          return;
-        }
-      }
-      if (full) continue;
       for (uint32_t b = 0; b < 4; b++) {
         uint32_t p = cur + w * 4 + b;
         if (d[p] != t->empty_digest) continue;

@@ -791,3 +791,45 @@ def test_growth_under_host_threads():
     assert t.capacity() * 2 >= max_cap and min(rounds) > 0
     assert t.size() <= sum(rounds) * n
     t.close()
+
+
+def test_rehash_on_big_batches(oracle):
+    """tests/merlin_hashtable_test.cc.cu:1223-1367 (test_rehash_on_big_batch) and :1369-1439
+    (test_rehash_on_big_batch_specific): the capacities the growth loop arrives at."""
+    dim = 8
+    t, o, _ = make_pair(oracle, init_capacity=1024, max_capacity=16 * 1024, dim=dim, reserved_key_start_bit=6,
+                        num_of_buckets_per_alloc=8, max_load_factor=0.6,
+                        evict_strategy=EvictStrategy.kCustomized)
+    keys = w.unique_keys(151, 0, 2048)
+    keys = keys[(keys & np.uint64(~(3 << 6) & M64 & ~1)) != np.uint64(~(3 << 6) & M64 & ~1)]
+    assert len(keys) == 2048
+    vals = w.values_from_keys(keys, dim)
+    for n, cap in ((1024, 2048), (2048, 8192)):
+        t.insert_or_assign(n, dev(keys[:n]), dev(vals[:n]), dev(keys[:n].copy()))
+        o.insert_or_assign(keys[:n], bytes_of(vals[:n]), keys[:n].copy())
+        assert t.size() == o.size() == n
+        assert t.capacity() == o.capacity() == cap
+    ek, ev, es = export_table(t, dim * 4)
+    assert len(ek) == 2048
+    out = torch.zeros(2048, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(2048, dtype=torch.bool, device=DEV)
+    sc = torch.zeros(2048, dtype=torch.int64, device=DEV)
+    t.find(2048, dev(keys), out, founds, sc)
+    torch.cuda.synchronize()
+    assert bool(founds.all()) and np.array_equal(host_u64(sc), keys)
+    assert np.array_equal(out.cpu().numpy(), vals)
+    assert_same_table(t, o, dim * 4)
+    t.close()
+    # 50 000 slots asked for, 100 000 allowed: 512 buckets, and no room to double
+    t, o, _ = make_pair(oracle, init_capacity=50000, max_capacity=100000, dim=dim, reserved_key_start_bit=7,
+                        num_of_buckets_per_alloc=16, max_load_factor=0.6, evict_strategy=EvictStrategy.kLru)
+    t.set_clock(1, 1 << 40)
+    o.set_clock(1, 1 << 40)
+    keys = w.unique_keys(152, 0, 50000)
+    vals = w.values_from_keys(keys, dim)
+    t.insert_or_assign(50000, dev(keys), dev(vals))
+    o.insert_or_assign(keys, bytes_of(vals))
+    assert t.capacity() == o.capacity() == 65536
+    assert t.size() == o.size()
+    assert_same_table(t, o, dim * 4)
+    t.close()

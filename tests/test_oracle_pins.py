@@ -852,3 +852,30 @@ def test_dual_eviction_quality(oracle):
     assert overlap / len(ek) >= 0.995
     assert np.array_equal(es, scores[ek.astype(np.int64) - 1])
     t.close()
+
+
+def test_rehash_on_big_batch_scenario_of_the_reference(oracle):
+    # merlin_hashtable_test.cc.cu:1223-1367: init 1024, max 16384, load factor 0.6; 1024 keys
+    # bring the capacity to 2048, the 2048 keys that contain them to 8192, and the table then
+    # holds 2048 keys (re-inserting keys that a rehash has moved must find them: the reference
+    # compacts buckets after a rehash, here the key is looked for in the whole bucket)
+    o = default_options(init_capacity=1024, max_capacity=16 * 1024, dim=2, reserved_key_start_bit=6,
+                        num_of_buckets_per_alloc=8, max_load_factor=0.6, max_hbm_for_vectors=1 << 30,
+                        evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(151, 0, 2048)
+    vals = np.zeros((2048, 8), np.uint8)
+    for n, cap in ((1024, 2048), (2048, 8192)):
+        t.insert_or_assign(keys[:n], vals[:n], keys[:n].copy())
+        assert t.size() == n and t.capacity() == cap
+    ek, _, es = t.export_all()
+    assert len(ek) == 2048 and len(np.unique(ek)) == 2048 and np.array_equal(np.sort(ek), np.sort(keys))
+    assert np.array_equal(es, ek)
+    # merlin_hashtable_test.cc.cu:1369-1439: 50 000 asked for, 100 000 allowed: 512 buckets, no doubling
+    o = default_options(init_capacity=50000, max_capacity=100000, dim=2, max_load_factor=0.6,
+                        max_hbm_for_vectors=1 << 30, evict_strategy=EvictStrategy.kLru)
+    t = oracle.OracleTable(o)
+    t.set_clock(1, 1 << 40)
+    k = w.unique_keys(152, 0, 50000)
+    t.insert_or_assign(k, np.zeros((50000, 8), np.uint8))
+    assert t.capacity() == 65536
