@@ -383,3 +383,69 @@ def test_config5_update_export_full_size(path, monkeypatch):
     assert bool(founds.all()) and torch.equal(out, value_of(k, dim))
     assert t.size() <= cap
     t.close()
+
+
+# ---- closed-form scenarios of the reference's own tests at (nearly) their sizes --------------------------
+
+def _ref_rows(keys, dim):
+    """test_util.cuh:160-163: every element of a key's row is float(key * 0.00001)."""
+    return np.repeat((keys.astype(np.float64) * 0.00001).astype(np.float32)[:, None], dim, axis=1)
+
+
+def test_basic_when_full_scenario():
+    """tests/merlin_hashtable_test.cc.cu:799-925 (test_basic_when_full): as many random keys as
+    the table has slots in one call; what stays can be found with its row, erasing everything
+    empties the table, and inserting the same batch again fills it to the same size."""
+    from gpu_util import dev
+    cap, dim = 1 << 20, 16
+    t = make_table(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 34, dim=dim,
+                   reserved_key_start_bit=3, num_of_buckets_per_alloc=32,
+                   evict_strategy=EvictStrategy.kCustomized)
+    rng = np.random.default_rng(7)
+    keys = np.unique(rng.integers(0, 1 << 62, cap + 4096, dtype=np.uint64))[:cap]
+    rng.shuffle(keys)
+    scores = rng.integers(1, 1 << 62, cap, dtype=np.uint64)
+    dk, dv, ds = dev(keys), dev(_ref_rows(keys, dim)), dev(scores)
+    t.insert_or_assign(cap, dk, dv, ds)
+    size_after_insert = t.size()
+    assert 0.9 * cap < size_after_insert < cap  # some buckets get more than 128 of the keys
+    out = torch.zeros(cap, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(cap, dtype=torch.bool, device=DEV)
+    t.find(cap, dk, out, founds, None)
+    assert int(founds.sum()) == size_after_insert
+    assert bool((out[founds] == dv[founds]).all())
+    # the survivors of a bucket are its highest scores: the table holds sum(min(128, n_b)) keys
+    t.erase(cap, dk)
+    assert t.size() == 0
+    t.insert_or_assign(cap, dk, dv, ds)
+    assert t.size() == size_after_insert
+    t.close()
+
+
+def test_customized_correct_rate_scenario():
+    """tests/merlin_hashtable_test.cc.cu:3055-3178 (test_evict_strategy_customized_correct_rate) at
+    1/16 of its size: consecutive keys with score = key, three times the capacity in 128 batches
+    per round; after every round at least 96.4 % of the slots hold keys of that round."""
+    from gpu_util import dev, export_table
+    batch, steps, dim, rounds = 1 << 16, 128, 4, 3
+    cap = batch * steps
+    t = make_table(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 34, dim=dim,
+                   reserved_key_start_bit=17, num_of_buckets_per_alloc=128,
+                   evict_strategy=EvictStrategy.kCustomized)
+    start = 100000
+    for r in range(rounds):
+        expected_min, expected_max = start + cap * r, start + cap * (r + 1) - 1
+        for s in range(steps):
+            k = np.arange(start + (r * steps + s) * batch, start + (r * steps + s + 1) * batch, dtype=np.uint64)
+            t.insert_or_assign(batch, dev(k), dev(_ref_rows(k, dim)), dev(k.copy()))
+        size = t.size()
+        assert size >= (int(0.964 * cap) if r == 0 else cap)
+        assert t.capacity() == cap
+        ek, ev, es = export_table(t, dim * 4)
+        assert len(ek) == size and np.array_equal(ek, es)
+        assert np.array_equal(ev.view(np.float32), _ref_rows(ek, dim))
+        rate = float((es >= expected_min).sum()) / cap
+        print(f"[round {r}] correct rate {rate:.4f}, size {size / cap:.4f}")
+        assert int(ek.max()) >= expected_max
+        assert rate >= 0.964
+    t.close()
