@@ -24,6 +24,8 @@
  * the export family, as in the reference; the calls the reference guards throw
  * the same way, and assign, find*, lock_keys / unlock_keys / find_and_update
  * (unguarded but single-bucket in the reference) throw too.
+ * Buckets have 128 slots: init() throws for any other max_bucket_size (the reference takes
+ * powers of two from 8 to 2048; 128 is its default and the length its tuned kernels assume).
  * S = uint32_t (Customized strategy only, as in the reference) is served by widening and
  * narrowing the caller's score arrays around each call: the table keeps 64-bit scores, and
  * such calls allocate a temporary buffer on the stream.
@@ -231,7 +233,7 @@ struct HashTableOptions {
   size_t init_capacity = 0;        ///< The initial capacity of the hash table.
   size_t max_capacity = 0;         ///< The maximum capacity of the hash table.
   size_t max_hbm_for_vectors = 0;  ///< The maximum HBM for vectors, in bytes.
-  size_t max_bucket_size = 128;    ///< The length of each bucket.
+  size_t max_bucket_size = 128;    ///< The length of each bucket (only 128 here).
   size_t dim = 64;                 ///< The dimension of the vectors.
   float max_load_factor = 0.5f;    ///< The max load factor before rehashing.
   int block_size = 128;            ///< Kept for source compatibility; unused.
