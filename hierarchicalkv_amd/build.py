@@ -41,15 +41,18 @@ def build_library(verbose=True):
 def build_cpp_tests(verbose=True):
     """The C++ test of the drop-in header (tests/cpp/api_test.cpp), linked
     against the in-tree library; a GPU test runs the binary."""
-    src = os.path.join(ROOT, "tests", "cpp", "api_test.cpp")
-    out = os.path.join(ROOT, "tests", "cpp", "api_test")
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-I", INCLUDE, src, "-L", PKG_DIR, "-lhkv",
-           "-Wl,-rpath,$ORIGIN/../../hierarchicalkv_amd", "-o", out]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    out = None
+    # api_test: the reference's test scenarios; bench_matrix: the reference's benchmark table
+    for name in ("api_test", "bench_matrix"):
+        src = os.path.join(ROOT, "tests", "cpp", name + ".cpp")
+        out = os.path.join(ROOT, "tests", "cpp", name)
+        cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-I", INCLUDE, src, "-L", PKG_DIR, "-lhkv",
+               "-Wl,-rpath,$ORIGIN/../../hierarchicalkv_amd", "-o", out]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
     return out
 
 
