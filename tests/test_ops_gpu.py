@@ -833,3 +833,44 @@ def test_rehash_on_big_batches(oracle):
     assert t.size() == o.size()
     assert_same_table(t, o, dim * 4)
     t.close()
+
+
+def test_tombstones_are_never_reported_as_evicted(oracle):
+    """tests/insert_and_evict_test.cc.cu:1654-1710 (test_insert_and_evict_bugfix_no_zero_eviction):
+    fill a 2048-slot LRU table, erase half, insert 2048 new keys with insert_and_evict: slots of
+    erased keys are taken without an eviction being reported, and every reported key is a key
+    that was resident."""
+    cap, dim = 2048, 8
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, num_of_buckets_per_alloc=16,
+                        evict_strategy=EvictStrategy.kLru)
+    t.set_clock(1, 1 << 40)
+    o.set_clock(1, 1 << 40)
+
+    def evict_call(keys):
+        n = len(keys)
+        vals = w.values_from_keys(keys, dim)
+        ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+        ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        got = t.insert_and_evict(n, dev(keys), dev(vals), None, ek, ev, None)  # count-returning overload
+        oek, oev, _ = o.insert_and_evict(keys, bytes_of(vals))
+        torch.cuda.synchronize()
+        gk = host_u64(ek)[:got]
+        gv = host_bytes(ev, n, dim * 4)[:got]
+        assert got == len(oek)
+        a, b = np.argsort(gk, kind="stable"), np.argsort(oek, kind="stable")
+        assert np.array_equal(gk[a], oek[b]) and np.array_equal(gv[a], oev[b])
+        return gk
+
+    first = np.arange(1, cap + 1, dtype=np.uint64)
+    evict_call(first)
+    t.erase(1024, dev(first[:1024]))
+    o.erase(first[:1024])
+    assert t.size() == o.size()
+    resident = set(export_table(t, dim * 4)[0].tolist())
+    new = np.arange(3000, 3000 + cap, dtype=np.uint64)
+    gone = evict_call(new)
+    assert 0 not in set(gone.tolist())
+    assert set(gone.tolist()) <= resident | set(new.tolist())  # residents, or refused new keys
+    assert not (set(gone.tolist()) & set(first[:1024].tolist()))  # nothing that had been erased
+    assert_same_table(t, o, dim * 4)
+    t.close()
