@@ -874,3 +874,65 @@ def test_tombstones_are_never_reported_as_evicted(oracle):
     assert not (set(gone.tolist()) & set(first[:1024].tolist()))  # nothing that had been erased
     assert_same_table(t, o, dim * 4)
     t.close()
+
+
+def test_insert_and_evict_beside_find_on_another_thread():
+    """tests/insert_and_evict_test.cc.cu:1713-1790 (test_insert_and_evict_run_with_batch_find): one
+    host thread inserts with eviction, another looks keys up on a stream of its own; the group lock
+    keeps the two kinds of call apart.  Checked here: every lookup sees whole rows, and keys are
+    conserved (inserted = resident + evicted)."""
+    import threading
+    cap, dim, bs, batches = 1 << 18, 16, 1 << 14, 48
+    t = HashTable()
+    t.init(default_options(init_capacity=cap, max_capacity=cap, dim=dim, max_hbm_for_vectors=1 << 34,
+                           num_of_buckets_per_alloc=128, evict_strategy=EvictStrategy.kLru))
+    keys = [w.unique_keys(161, b * bs, bs) for b in range(batches)]
+    step, errors, evicted_total = [0], [], [0]
+
+    def inserter():
+        try:
+            st = torch.cuda.Stream()
+            ek = torch.zeros(bs, dtype=torch.int64, device=DEV)
+            ev = torch.zeros(bs, dim, dtype=torch.float32, device=DEV)
+            for b in range(batches):
+                dk, dv = dev(keys[b]), dev(w.values_from_keys(keys[b], dim))
+                torch.cuda.current_stream().synchronize()
+                got = t.insert_and_evict(bs, dk, dv, None, ek, ev, None, stream=st)
+                st.synchronize()
+                gk = host_u64(ek)[:got]
+                rows = ev.cpu().numpy()[:got]
+                assert np.array_equal(rows, w.values_from_keys(gk, dim)), b  # evicted rows are whole
+                evicted_total[0] += got
+                step[0] = b + 1
+        except BaseException as e:  # noqa: BLE001
+            errors.append(("insert", repr(e)))
+            step[0] = batches
+
+    def finder():
+        try:
+            st = torch.cuda.Stream()
+            out = torch.zeros(bs, dim, dtype=torch.float32, device=DEV)
+            founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+            rounds = 0
+            while step[0] < batches or rounds == 0:
+                b = max(step[0] - 1, 0)
+                dk = dev(keys[b])
+                torch.cuda.current_stream().synchronize()
+                t.find(bs, dk, out, founds, None, stream=st)
+                st.synchronize()
+                f = founds.cpu().numpy()
+                rows = out.cpu().numpy()
+                assert np.array_equal(rows[f], w.values_from_keys(keys[b], dim)[f]), b
+                rounds += 1
+        except BaseException as e:  # noqa: BLE001
+            errors.append(("find", repr(e)))
+
+    th = [threading.Thread(target=finder), threading.Thread(target=inserter)]
+    for x in th:
+        x.start()
+    for x in th:
+        x.join()
+    assert not errors, errors
+    assert t.size() + evicted_total[0] == batches * bs
+    assert t.size() > 0.95 * cap
+    t.close()
