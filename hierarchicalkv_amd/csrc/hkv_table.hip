@@ -274,9 +274,35 @@ int pick_upl(uint32_t value_bytes, int vec) {
   return 8;
 }
 
+/* accum_or_assign adds element by element, so its unit must hold whole elements: the widest of
+ * 16, 8, 4, 2 and 1 bytes that the row size and the pointer allow, or 0 when that is less than
+ * one element (an odd address for 16-bit elements, and the like). */
+int accum_unit(uint32_t value_bytes, const void* p, int kind) {
+  const uint32_t elem[] = {1, 4, 8, 4, 8, 1, 2};
+  const uintptr_t mis = value_bytes | (uintptr_t)p;
+  int unit = 1;
+  for (int u : {16, 8, 4, 2})
+    if ((mis & (uintptr_t)(u - 1)) == 0) {
+      unit = u;
+      break;
+    }
+  return unit >= (int)elem[kind] ? unit : 0;
+}
+
 template <int OP, bool LOCKED_RULE>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
+  if constexpr (OP == kOpAccumOrAssign) {
+    /* the two units that only the element-wise add needs */
+    if (vec == 8) {
+      hipLaunchKernelGGL((upsert_kernel<OP, 8, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      return;
+    }
+    if (vec == 2) {
+      hipLaunchKernelGGL((upsert_kernel<OP, 2, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      return;
+    }
+  }
   if (OP == kOpFindOrInsertPtr) {
     hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE>), grid, block, 0, s, v, a);
     return;
@@ -583,6 +609,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
      * wavefront and pass, which serialises at full size (1.14 ms against 0.53 ms per 2^20
      * keys); only the forced mode of the tests takes it there */
     if (OP == kOpInsertAndEvict && t->upsert_path != 2) plan.feasible = false;
+    if (vec == 8 || vec == 2) plan.feasible = false; /* units only the slot-lock kernel has */
     if (plan.feasible) {
       if constexpr (OP != kOpFindOrInsertPtr)
         HKV_TRY(run_grouped<OP>(t, a, vec, refuse_equal, plan, s));
@@ -896,8 +923,8 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
     return fail(HKV_ERROR_ARGUMENT, "dim and value_size must be positive");
   if (o->dim * (uint64_t)o->value_size > (1u << 20))
     return fail(HKV_ERROR_UNSUPPORTED, "value rows above 1 MiB are not supported");
-  const uint32_t ksz[] = {0, 4, 8, 4, 8};
-  if (o->value_kind < 0 || o->value_kind > 4 ||
+  const uint32_t ksz[] = {0, 4, 8, 4, 8, 1, 2};
+  if (o->value_kind < 0 || o->value_kind > 6 ||
       (o->value_kind != 0 && ksz[o->value_kind] != o->value_size))
     return fail(HKV_ERROR_ARGUMENT, "value_kind does not match value_size");
 
@@ -1165,7 +1192,9 @@ int hkv_accum_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.scores = scores;
   a.n = n;
   a.strategy = strategy;
-  const int vec = pick_vec(t->view.value_bytes, {value_or_deltas});
+  const int vec = accum_unit(t->view.value_bytes, value_or_deltas, t->opts.value_kind);
+  if (vec == 0)
+    return fail(HKV_ERROR_ARGUMENT, "accum_or_assign: value_or_deltas is not aligned to its element type");
   return run_upsert<kOpAccumOrAssign>(t, a, vec, false, (hipStream_t)stream);
 }
 

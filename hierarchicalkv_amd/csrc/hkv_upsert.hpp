@@ -115,6 +115,13 @@ __device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
   st_u64(v.scores + slot, s);
 }
 
+/* wrapping adds of the 8- and 16-bit lanes of a word (signed and unsigned alike) */
+__device__ __forceinline__ uint32_t add_lanes8(uint32_t x, uint32_t y) {
+  return ((x & 0x7F7F7F7Fu) + (y & 0x7F7F7F7Fu)) ^ ((x ^ y) & 0x80808080u);
+}
+__device__ __forceinline__ uint32_t add_lanes16(uint32_t x, uint32_t y) {
+  return ((x & 0x7FFF7FFFu) + (y & 0x7FFF7FFFu)) ^ ((x ^ y) & 0x80008000u);
+}
 /* x + y on one unit of a row, element type by `kind` (accum_or_assign_vector,
  * accum_or_assign.cuh:24-35); one IEEE add per element. */
 __device__ __forceinline__ uint4 add_unit(uint4 x, uint4 y, int kind) {
@@ -123,6 +130,10 @@ __device__ __forceinline__ uint4 add_unit(uint4 x, uint4 y, int kind) {
     x.y = __float_as_uint(__uint_as_float(x.y) + __uint_as_float(y.y));
     x.z = __float_as_uint(__uint_as_float(x.z) + __uint_as_float(y.z));
     x.w = __float_as_uint(__uint_as_float(x.w) + __uint_as_float(y.w));
+  } else if (kind == HKV_VALUE_I8) {
+    x = make_uint4(add_lanes8(x.x, y.x), add_lanes8(x.y, y.y), add_lanes8(x.z, y.z), add_lanes8(x.w, y.w));
+  } else if (kind == HKV_VALUE_I16) {
+    x = make_uint4(add_lanes16(x.x, y.x), add_lanes16(x.y, y.y), add_lanes16(x.z, y.z), add_lanes16(x.w, y.w));
   } else if (kind == HKV_VALUE_I32) {
     x.x += y.x;
     x.y += y.y;
@@ -144,12 +155,32 @@ __device__ __forceinline__ uint4 add_unit(uint4 x, uint4 y, int kind) {
   }
   return x;
 }
+/* The host side picks a unit that is at least one element wide (accum_unit in hkv_table.hip). */
 __device__ __forceinline__ uint32_t add_unit(uint32_t x, uint32_t y, int kind) {
   if (kind == HKV_VALUE_F32) return __float_as_uint(__uint_as_float(x) + __uint_as_float(y));
-  return x + y; /* i32; 8-byte element kinds never take a 4-byte unit (host check) */
+  if (kind == HKV_VALUE_I8) return add_lanes8(x, y);
+  if (kind == HKV_VALUE_I16) return add_lanes16(x, y);
+  return x + y; /* i32 */
 }
-__device__ __forceinline__ uint8_t add_unit(uint8_t x, uint8_t, int) {
-  return x; /* unreachable: arithmetic kinds have 4- or 8-byte elements */
+__device__ __forceinline__ uint2 add_unit(uint2 x, uint2 y, int kind) {
+  if (kind == HKV_VALUE_F64 || kind == HKV_VALUE_I64) {
+    uint64_t a = x.x | ((uint64_t)x.y << 32);
+    const uint64_t b = y.x | ((uint64_t)y.y << 32);
+    if (kind == HKV_VALUE_F64)
+      a = (uint64_t)__double_as_longlong(__longlong_as_double((long long)a) +
+                                         __longlong_as_double((long long)b));
+    else
+      a += b;
+    return make_uint2((uint32_t)a, (uint32_t)(a >> 32));
+  }
+  return make_uint2(add_unit(x.x, y.x, kind), add_unit(x.y, y.y, kind));
+}
+__device__ __forceinline__ uint16_t add_unit(uint16_t x, uint16_t y, int kind) {
+  if (kind == HKV_VALUE_I8) return (uint16_t)add_lanes8(x, y);
+  return (uint16_t)(x + y); /* i16 */
+}
+__device__ __forceinline__ uint8_t add_unit(uint8_t x, uint8_t y, int) {
+  return (uint8_t)(x + y); /* i8 */
 }
 
 /* One VEC-byte unit of a row.  Table rows are read and written coherently
@@ -171,8 +202,14 @@ __device__ __forceinline__ typename VecType<VEC>::type ld_unit(const uint8_t* ro
     const uint64_t* p = reinterpret_cast<const uint64_t*>(row) + 2 * u;
     const uint64_t lo = ld_u64(p), hi = ld_u64(p + 1);
     return make_uint4((uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32));
+  } else if constexpr (VEC == 8) {
+    const uint64_t x = ld_u64(reinterpret_cast<const uint64_t*>(row) + u);
+    return make_uint2((uint32_t)x, (uint32_t)(x >> 32));
   } else if constexpr (VEC == 4) {
     return ld_u32(reinterpret_cast<const uint32_t*>(row) + u);
+  } else if constexpr (VEC == 2) {
+    return __hip_atomic_load(reinterpret_cast<const uint16_t*>(row) + u, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
   } else {
     return ld_u8(row + u);
   }
@@ -194,8 +231,13 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
 #else
     st_u128(row + 16 * (size_t)u, x);
 #endif
+  } else if constexpr (VEC == 8) {
+    st_u64(reinterpret_cast<uint64_t*>(row) + u, x.x | ((uint64_t)x.y << 32));
   } else if constexpr (VEC == 4) {
     st_u32(reinterpret_cast<uint32_t*>(row) + u, x);
+  } else if constexpr (VEC == 2) {
+    __hip_atomic_store(reinterpret_cast<uint16_t*>(row) + u, x, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
   } else {
     st_u8(row + u, x);
   }

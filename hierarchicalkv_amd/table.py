@@ -34,6 +34,8 @@ class ValueKind:
     kF64 = 2
     kI32 = 3
     kI64 = 4
+    kI8 = 5
+    kI16 = 6
 
 
 class Predicate:

@@ -58,8 +58,10 @@ typedef enum hkv_value_kind {
   HKV_VALUE_BYTES = 0, /* opaque bytes: accum_or_assign is refused */
   HKV_VALUE_F32 = 1,
   HKV_VALUE_F64 = 2,
-  HKV_VALUE_I32 = 3,
-  HKV_VALUE_I64 = 4
+  HKV_VALUE_I32 = 3, /* the integer kinds add with wrap-around, signed and unsigned alike */
+  HKV_VALUE_I64 = 4,
+  HKV_VALUE_I8 = 5,
+  HKV_VALUE_I16 = 6
 } hkv_value_kind;
 
 /* Built-in predicates for export_batch_if / size_if.  A caller that needs an

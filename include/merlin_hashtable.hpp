@@ -351,6 +351,8 @@ constexpr int value_kind_of() {
   if (std::is_same<V, double>::value) return HKV_VALUE_F64;
   if (std::is_same<V, int32_t>::value || std::is_same<V, uint32_t>::value) return HKV_VALUE_I32;
   if (std::is_same<V, int64_t>::value || std::is_same<V, uint64_t>::value) return HKV_VALUE_I64;
+  if (std::is_same<V, int8_t>::value || std::is_same<V, uint8_t>::value) return HKV_VALUE_I8;
+  if (std::is_same<V, int16_t>::value || std::is_same<V, uint16_t>::value) return HKV_VALUE_I16;
   return HKV_VALUE_BYTES;
 }
 

@@ -1002,6 +1002,16 @@ static void add_row(int kind, uint8_t* dst, const uint8_t* delta, uint64_t dim) 
       for (uint64_t j = 0; j < dim; j++) d[j] += s[j];
       break;
     }
+    case HKV_VALUE_I8: {
+      for (uint64_t j = 0; j < dim; j++) dst[j] = (uint8_t)(dst[j] + delta[j]);
+      break;
+    }
+    case HKV_VALUE_I16: {
+      uint16_t* d = (uint16_t*)dst;
+      const uint16_t* s = (const uint16_t*)delta;
+      for (uint64_t j = 0; j < dim; j++) d[j] = (uint16_t)(d[j] + s[j]);
+      break;
+    }
     default:
       break;
   }

@@ -85,10 +85,16 @@ def test_find_ptr_contains_and_missed(oracle):
     (np.int8, torch.int8, ValueKind.kBytes, 3),
     (np.uint8, torch.uint8, ValueKind.kBytes, 129),
     (np.int16, torch.int16, ValueKind.kBytes, 66),
-    (np.int32, torch.int32, ValueKind.kI32, 202),
+    (np.int8, torch.int8, ValueKind.kI8, 3),       # 1-byte units
+    (np.uint8, torch.uint8, ValueKind.kI8, 129),
+    (np.int8, torch.int8, ValueKind.kI8, 64),      # 16-byte units
+    (np.int16, torch.int16, ValueKind.kI16, 33),   # 2-byte units
+    (np.uint16, torch.int16, ValueKind.kI16, 66),  # 4-byte units
+    (np.int32, torch.int32, ValueKind.kI32, 202),  # 8-byte units
     (np.float32, torch.float32, ValueKind.kF32, 224),
     (np.float32, torch.float32, ValueKind.kF32, 3),
     (np.float64, torch.float64, ValueKind.kF64, 128),
+    (np.float64, torch.float64, ValueKind.kF64, 63),  # 8-byte units
     (np.int64, torch.int64, ValueKind.kI64, 5),
 ])
 def test_value_types_and_dims(oracle, np_dtype, torch_dtype, kind, dim):
@@ -116,7 +122,12 @@ def test_value_types_and_dims(oracle, np_dtype, torch_dtype, kind, dim):
     if kind != ValueKind.kBytes:
         # accum_or_assign on every arithmetic element type
         keys = q[: bs]
-        delta = (rng.integers(0, 100, size=(bs, dim)).astype(np_dtype))
+        if np.issubdtype(np_dtype, np.integer):
+            # the whole range: carries between the bytes of an element, wrap-around at its top
+            info = np.iinfo(np_dtype)
+            delta = rng.integers(info.min, info.max, size=(bs, dim), dtype=np_dtype, endpoint=True)
+        else:
+            delta = (rng.standard_normal(size=(bs, dim)) * 1000).astype(np_dtype)
         flags = o.contains(keys)
         t.accum_or_assign(bs, dev(keys), dev(bytes_of(delta)), dev(flags.astype(np.uint8)),
                           dev(w.monotone_scores(9, bs)))

@@ -879,3 +879,27 @@ def test_rehash_on_big_batch_scenario_of_the_reference(oracle):
     k = w.unique_keys(152, 0, 50000)
     t.insert_or_assign(k, np.zeros((50000, 8), np.uint8))
     assert t.capacity() == 65536
+
+
+def test_accum_wraps_in_the_element_type(oracle):
+    # accum_or_assign_vector (accum_or_assign.cuh:24-35) adds in V: 8- and 16-bit elements wrap at
+    # their own width, independently of their neighbours in the row
+    for dtype, kind in ((np.uint8, ValueKind.kI8), (np.int16, ValueKind.kI16)):
+        dim = 7
+        o = default_options(init_capacity=1024, max_capacity=1024, dim=dim, value_size=np.dtype(dtype).itemsize,
+                            value_kind=kind, max_hbm_for_vectors=1 << 30, evict_strategy=EvictStrategy.kCustomized)
+        t = oracle.OracleTable(o)
+        rng = np.random.default_rng(5)
+        info = np.iinfo(dtype)
+        keys = w.unique_keys(171, 0, 64)
+        base = rng.integers(info.min, info.max, size=(64, dim), dtype=dtype, endpoint=True)
+        delta = rng.integers(info.min, info.max, size=(64, dim), dtype=dtype, endpoint=True)
+        sc = np.arange(1, 65, dtype=np.uint64)
+        as_bytes = lambda a: np.ascontiguousarray(a).view(np.uint8).reshape(len(a), -1)  # noqa: E731
+        t.insert_or_assign(keys, as_bytes(base), sc)
+        t.accum_or_assign(keys, as_bytes(delta), np.ones(64, np.uint8), sc)
+        vals, founds, _ = t.find(keys)
+        assert founds.all()
+        with np.errstate(over="ignore"):
+            want = (base.astype(np.int64) + delta.astype(np.int64)).astype(dtype)  # modulo 2^bits
+        assert np.array_equal(vals, as_bytes(want))
