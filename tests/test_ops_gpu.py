@@ -804,13 +804,16 @@ def test_growth_under_host_threads():
     t.close()
 
 
-def test_rehash_on_big_batches(oracle):
+@pytest.mark.parametrize("hbm", [1 << 34, 0, 1024 * 8 * 4])
+def test_rehash_on_big_batches(oracle, hbm):
     """tests/merlin_hashtable_test.cc.cu:1223-1367 (test_rehash_on_big_batch) and :1369-1439
-    (test_rehash_on_big_batch_specific): the capacities the growth loop arrives at."""
+    (test_rehash_on_big_batch_specific): the capacities the growth loop arrives at; with all rows
+    in HBM, all in host memory (the reference runs its rehash tests both ways) and with an HBM
+    budget that the growing table leaves behind."""
     dim = 8
-    t, o, _ = make_pair(oracle, init_capacity=1024, max_capacity=16 * 1024, dim=dim, reserved_key_start_bit=6,
-                        num_of_buckets_per_alloc=8, max_load_factor=0.6,
-                        evict_strategy=EvictStrategy.kCustomized)
+    t, o, _ = make_pair(oracle, hybrid=hbm < (1 << 34), init_capacity=1024, max_capacity=16 * 1024, dim=dim,
+                        reserved_key_start_bit=6, num_of_buckets_per_alloc=8, max_load_factor=0.6,
+                        max_hbm_for_vectors=hbm, evict_strategy=EvictStrategy.kCustomized)
     keys = w.unique_keys(151, 0, 2048)
     keys = keys[(keys & np.uint64(~(3 << 6) & M64 & ~1)) != np.uint64(~(3 << 6) & M64 & ~1)]
     assert len(keys) == 2048
@@ -832,8 +835,9 @@ def test_rehash_on_big_batches(oracle):
     assert_same_table(t, o, dim * 4)
     t.close()
     # 50 000 slots asked for, 100 000 allowed: 512 buckets, and no room to double
-    t, o, _ = make_pair(oracle, init_capacity=50000, max_capacity=100000, dim=dim, reserved_key_start_bit=7,
-                        num_of_buckets_per_alloc=16, max_load_factor=0.6, evict_strategy=EvictStrategy.kLru)
+    t, o, _ = make_pair(oracle, hybrid=hbm < (1 << 34), init_capacity=50000, max_capacity=100000, dim=dim,
+                        reserved_key_start_bit=7, num_of_buckets_per_alloc=16, max_load_factor=0.6,
+                        max_hbm_for_vectors=hbm, evict_strategy=EvictStrategy.kLru)
     t.set_clock(1, 1 << 40)
     o.set_clock(1, 1 << 40)
     keys = w.unique_keys(152, 0, 50000)
