@@ -449,3 +449,27 @@ def test_customized_correct_rate_scenario():
         assert int(ek.max()) >= expected_max
         assert rate >= 0.964
     t.close()
+
+
+@pytest.mark.parametrize("hbm", [1 << 34, 0])
+def test_insert_or_assign_values_check_scenario(hbm):
+    """tests/merlin_hashtable_test.cc.cu:3621-3660 (test_insert_or_assign_values_check): an LRU table
+    that grows from 1024 slots to 2^19, batches of 2^19 + 13 random keys out of a range 16 times
+    as large (more keys than the table can ever hold, and many of them met before); after every
+    call the export has as many entries as size() says and every row is the row of its key."""
+    from gpu_util import dev, export_table
+    cap, dim = 524288, 64
+    n = cap + 13
+    t = make_table(init_capacity=1024, max_capacity=cap, max_hbm_for_vectors=hbm, dim=dim,
+                   evict_strategy=EvictStrategy.kLru)
+    rng = np.random.default_rng(11)
+    for it in range(6):
+        keys = rng.choice(n * 16, size=n, replace=False).astype(np.uint64)
+        t.insert_or_assign(n, dev(keys), dev(_ref_rows(keys, dim)))
+        size = t.size()
+        ek, ev, es = export_table(t, dim * 4)
+        assert len(ek) == size and len(np.unique(ek)) == size
+        assert np.array_equal(ev.view(np.float32), _ref_rows(ek, dim))
+        assert t.capacity() == cap and size > 0.9 * cap
+        assert np.isin(ek, keys).mean() > 0.9  # LRU: what stays is mostly the newest batch
+    t.close()
