@@ -465,7 +465,14 @@ def test_insert_or_assign_values_check_scenario(hbm):
     rng = np.random.default_rng(11)
     for it in range(6):
         keys = rng.choice(n * 16, size=n, replace=False).astype(np.uint64)
-        t.insert_or_assign(n, dev(keys), dev(_ref_rows(keys, dim)))
+        if it % 2 == 0:
+            t.insert_or_assign(n, dev(keys), dev(_ref_rows(keys, dim)))
+        else:
+            # find_or_insert_test.cc.cu (test_find_or_insert_values_check): keys that are there hand
+            # their row back, new keys store theirs; either way the caller holds the key's row
+            io = dev(_ref_rows(keys, dim))
+            t.find_or_insert(n, dev(keys), io)
+            assert np.array_equal(io.cpu().numpy(), _ref_rows(keys, dim))
         size = t.size()
         ek, ev, es = export_table(t, dim * 4)
         assert len(ek) == size and len(np.unique(ek)) == size
