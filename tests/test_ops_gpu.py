@@ -951,3 +951,42 @@ def test_insert_and_evict_beside_find_on_another_thread():
     assert t.size() + evicted_total[0] == batches * bs
     assert t.size() > 0.95 * cap
     t.close()
+
+
+def test_insert_and_evict_with_export_batch_scenario():
+    """tests/insert_and_evict_test.cc.cu:1311-1385: 4096 + 13 consecutive keys (row = key) in one
+    insert_and_evict call into an LRU table that grows from 2048 to its maximum of 4096 slots;
+    what was evicted and what export_batch finds, window by window, is every key once with its row."""
+    dim, n = 16, 4096 + 13
+    t = HashTable()
+    t.init(default_options(init_capacity=2048, max_capacity=4096, dim=dim, max_hbm_for_vectors=1 << 30,
+                           num_of_buckets_per_alloc=16, evict_strategy=EvictStrategy.kLru))
+    keys = np.arange(n, dtype=np.uint64)
+    rows = np.repeat(keys.astype(np.float32)[:, None], dim, axis=1)
+    ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+    ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+    got = t.insert_and_evict(n, dev(keys), dev(rows), None, ek, ev, None)
+    torch.cuda.synchronize()
+    assert t.capacity() == 4096
+    seen = {}
+    gk, gv = host_u64(ek)[:got], ev.cpu().numpy()[:got]
+    for k, r in zip(gk.tolist(), gv):
+        assert k not in seen
+        seen[k] = r
+    window = t.capacity() >> 2
+    dk = torch.zeros(window, dtype=torch.int64, device=DEV)
+    dv = torch.zeros(window, dim, dtype=torch.float32, device=DEV)
+    dc = torch.zeros(1, dtype=torch.int64, device=DEV)
+    total = 0
+    for off in range(0, t.capacity(), window):
+        t.export_batch(window, off, dc, dk, dv, None)
+        torch.cuda.synchronize()
+        c = int(dc.item())
+        total += c
+        for k, r in zip(host_u64(dk)[:c].tolist(), dv.cpu().numpy()[:c]):
+            assert k not in seen
+            seen[k] = r
+    assert total == t.size() and got + total == n
+    assert sorted(seen) == list(range(n))
+    assert all((r == np.float32(k)).all() for k, r in seen.items())
+    t.close()
