@@ -1,8 +1,9 @@
-"""find and insert_or_assign launch kernels only (no allocation, no memset, no host
+"""Calls that return nothing to the host launch kernels only (no allocation, no memset, no host
 synchronisation on a table that cannot grow), so a serving loop can capture them into a HIP
-graph.  The graph is replayed several times with new contents in its static buffers, with
-eager calls and synchronisations in between, and every replay is checked against the oracle
-stepping through the same sequence."""
+graph: find and insert_or_assign in the first test, contains, assign, find_or_insert,
+insert_and_evict with a device counter and erase in the second.  The graph is replayed several
+times with new contents in its static buffers, with eager calls and synchronisations in between,
+and every replay is checked against the oracle stepping through the same sequence."""
 import numpy as np
 import pytest
 import torch
@@ -114,5 +115,108 @@ def _run(oracle, stream):
         ot.insert_or_assign(ek, bytes_of(ev), esc)
         torch.cuda.synchronize()
         assert t.size() == ot.size()
+    t.close()
+    ot.close()
+
+
+def test_writers_with_device_counters_replay_from_a_graph(oracle):
+    """The other calls that return nothing to the host: contains, assign, find_or_insert,
+    insert_and_evict with a device counter (cleared inside the graph by a fill kernel), erase."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        _run_writers(oracle, stream)
+    torch.cuda.synchronize()
+
+
+def _run_writers(oracle, stream):
+    cap, dim, n = 1 << 14, 8, 1024
+    o = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 30, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    t = HashTable()
+    t.init(o)
+    ot = oracle.OracleTable(o)
+    seq = 0
+    for b in range(20):  # a full table
+        seq += 1
+        k, v, sc = w.unique_keys(91, b * n, n), w.uniform_values(91, b * n, n, dim), w.monotone_scores(seq, n)
+        t.insert_or_assign(n, dev(k), dev(v), dev(sc))
+        ot.insert_or_assign(k, bytes_of(v), sc)
+    assert_same_table(t, ot, dim * 4)
+
+    def buf(shape, dtype):
+        return torch.zeros(shape, dtype=dtype, device=DEV)
+    ak, av, asc = buf(n, torch.int64), buf((n, dim), torch.float32), buf(n, torch.int64)      # assign
+    fk, fio, fsc = buf(n, torch.int64), buf((n, dim), torch.float32), buf(n, torch.int64)     # find_or_insert
+    ek, ev, esc = buf(n, torch.int64), buf((n, dim), torch.float32), buf(n, torch.int64)      # insert_and_evict
+    ok_, ov_, os_, cnt = buf(n, torch.int64), buf((n, dim), torch.float32), buf(n, torch.int64), buf(1, torch.int64)
+    rk, cf = buf(n // 4, torch.int64), buf(n // 4, torch.bool)                                # erase, contains
+
+    def load_inputs(step):
+        nonlocal seq
+        a_keys = w.unique_keys(91, 19 * n, n)  # resident throughout: its scores are raised every step
+        seq += 1
+        a_sc = w.monotone_scores(seq, n)
+        f_keys = w.unique_keys(92, step * n, n)  # all new
+        seq += 1
+        f_sc = w.monotone_scores(seq, n)
+        e_keys = w.unique_keys(93, step * n, n)  # all new
+        seq += 1
+        e_sc = w.monotone_scores(seq, n)
+        r_keys = f_keys[: n // 4]  # erase a quarter of what find_or_insert has just put in
+        vals = [w.uniform_values(94 + i, step * n, n, dim) for i in range(3)]
+        for d, h in ((ak, a_keys), (asc, a_sc), (fk, f_keys), (fsc, f_sc), (ek, e_keys), (esc, e_sc), (rk, r_keys)):
+            d.copy_(dev(h))
+        for d, h in ((av, vals[0]), (fio, vals[1]), (ev, vals[2])):
+            d.copy_(dev(h))
+        return a_keys, a_sc, f_keys, f_sc, e_keys, e_sc, r_keys, vals
+
+    def calls():
+        t.assign(n, ak, av, asc)
+        t.find_or_insert(n, fk, fio, fsc)
+        cnt.zero_()
+        t.insert_and_evict(n, ek, ev, esc, ok_, ov_, os_, cnt)
+        t.erase(n // 4, rk)
+        t.contains(n // 4, rk, cf)
+
+    def check(inp, step):
+        a_keys, a_sc, f_keys, f_sc, e_keys, e_sc, r_keys, vals = inp
+        ot.assign(a_keys, bytes_of(vals[0]), a_sc)
+        fio_want = bytes_of(vals[1]).copy()
+        ot.find_or_insert(f_keys, fio_want, f_sc)
+        oek, oev, oes = ot.insert_and_evict(e_keys, bytes_of(vals[2]), e_sc)
+        ot.erase(r_keys)
+        assert np.array_equal(bytes_of(fio.cpu().numpy()), fio_want), step
+        c = int(cnt.item())
+        assert c == len(oek), step
+        a = np.argsort(host_u64(ok_)[:c], kind="stable")
+        b = np.argsort(oek, kind="stable")
+        assert np.array_equal(host_u64(ok_)[:c][a], oek[b]), step
+        assert np.array_equal(bytes_of(ov_.cpu().numpy())[:c][a], oev[b]), step
+        assert np.array_equal(host_u64(os_)[:c][a], oes[b]), step
+        assert not cf.cpu().numpy().any(), step
+        assert_same_table(t, ot, dim * 4)
+
+    inp = load_inputs(0)
+    torch.cuda.synchronize()
+    calls()  # warm-up of the exact calls
+    torch.cuda.synchronize()
+    check(inp, 0)
+    g = torch.cuda.CUDAGraph()
+    inp = load_inputs(1)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g, stream=stream):
+        calls()
+    assert_same_table(t, ot, dim * 4)  # capture has not run anything
+    for step in range(1, 5):
+        if step > 1:
+            inp = load_inputs(step)
+        g.replay()
+        torch.cuda.synchronize()
+        check(inp, step)
+        seq += 1  # eager work between the replays
+        k, v, sc = w.unique_keys(95, step * n, n), w.uniform_values(95, step * n, n, dim), w.monotone_scores(seq, n)
+        t.insert_or_assign(n, dev(k), dev(v), dev(sc))
+        ot.insert_or_assign(k, bytes_of(v), sc)
+        torch.cuda.synchronize()
     t.close()
     ot.close()
