@@ -96,6 +96,10 @@ def test_find_ptr_contains_and_missed(oracle):
     (np.float64, torch.float64, ValueKind.kF64, 128),
     (np.float64, torch.float64, ValueKind.kF64, 63),  # 8-byte units
     (np.int64, torch.int64, ValueKind.kI64, 5),
+    (np.float32, torch.float32, ValueKind.kF32, 520),   # 2080-byte rows: several passes of 16-byte units
+    (np.float32, torch.float32, ValueKind.kF32, 1025),  # 4100-byte rows, 4-byte units
+    (np.int16, torch.int16, ValueKind.kI16, 2051),      # 4102-byte rows, 2-byte units
+    (np.float64, torch.float64, ValueKind.kF64, 257),   # 2056-byte rows, 8-byte units
 ])
 def test_value_types_and_dims(oracle, np_dtype, torch_dtype, kind, dim):
     # the matrix of test_find_using_pipeline (merlin_hashtable_test.cc.cu:675-798, 3816-3830)
