@@ -994,3 +994,86 @@ def test_insert_and_evict_with_export_batch_scenario():
     assert sorted(seen) == list(range(n))
     assert all((r == np.float32(k)).all() for k, r in seen.items())
     t.close()
+
+
+@pytest.mark.parametrize("row_bytes", [3, 66, 256, 520 * 4, 1025 * 4])
+def test_every_row_moving_call_with_odd_and_long_rows(oracle, row_bytes):
+    """Row sizes that take the 1-, 4- and 16-byte units and more than one pass of a tile: every call
+    that moves rows (insert_or_assign, find_or_insert, insert_and_evict, assign, assign_values,
+    find, export) against the oracle."""
+    cap, bs = 1 << 12, 700
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=row_bytes, value_size=1,
+                        value_kind=ValueKind.kBytes, evict_strategy=EvictStrategy.kCustomized)
+    rng = np.random.Generator(np.random.PCG64(row_bytes))
+    rows = lambda n: rng.integers(0, 256, size=(n, row_bytes), dtype=np.uint8)  # noqa: E731
+    seq = 0
+    for b in range(8):  # past capacity
+        seq += 1
+        k, v, sc = w.unique_keys(181, b * bs, bs), rows(bs), w.monotone_scores(seq, bs)
+        t.insert_or_assign(bs, dev(k), dev(v), dev(sc))
+        o.insert_or_assign(k, v, sc)
+    assert_same_table(t, o, row_bytes)
+    recent = w.unique_keys(181, 7 * bs, bs)
+    # find_or_insert: residents hand their rows back
+    io = rows(bs)
+    d_io = dev(io)
+    seq += 1
+    sc = w.monotone_scores(seq, bs)
+    t.find_or_insert(bs, dev(recent), d_io, dev(sc))
+    oio = io.copy()
+    o.find_or_insert(recent, oio, sc)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_io.cpu().numpy(), oio) and not np.array_equal(oio, io)
+    # find_or_insert: new keys store theirs
+    fresh = w.unique_keys(182, 0, bs)
+    io = rows(bs)
+    d_io = dev(io)
+    seq += 1
+    sc = w.monotone_scores(seq, bs)
+    t.find_or_insert(bs, dev(fresh), d_io, dev(sc))
+    oio = io.copy()
+    o.find_or_insert(fresh, oio, sc)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_io.cpu().numpy(), oio)
+    assert_same_table(t, o, row_bytes)
+    # insert_and_evict: the evicted rows come out whole
+    k2, v2 = w.unique_keys(183, 0, bs), rows(bs)
+    seq += 1
+    sc = w.monotone_scores(seq, bs)
+    ek = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    ev = torch.zeros(bs, row_bytes, dtype=torch.uint8, device=DEV)
+    es = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    c = t.insert_and_evict(bs, dev(k2), dev(v2), dev(sc), ek, ev, es)
+    oek, oev, oes = o.insert_and_evict(k2, v2, sc)
+    torch.cuda.synchronize()
+    assert c == len(oek) and c > 0
+    a, b = np.argsort(host_u64(ek)[:c], kind="stable"), np.argsort(oek, kind="stable")
+    assert np.array_equal(host_u64(ek)[:c][a], oek[b])
+    assert np.array_equal(ev.cpu().numpy()[:c][a], oev[b])
+    assert np.array_equal(host_u64(es)[:c][a], oes[b])
+    # assign and assign_values on a half-resident batch
+    mixed = np.concatenate([k2[: bs // 2], w.unique_keys(184, 0, bs - bs // 2)])
+    v3 = rows(bs)
+    seq += 1
+    sc = w.monotone_scores(seq, bs)
+    t.assign(bs, dev(mixed), dev(v3), dev(sc))
+    o.assign(mixed, v3, sc)
+    v4 = rows(bs)
+    t.assign_values(bs, dev(mixed), dev(v4))
+    o.assign_values(mixed, v4)
+    assert_same_table(t, o, row_bytes)
+    # find and find* read what is there
+    out = torch.zeros(bs, row_bytes, dtype=torch.uint8, device=DEV)
+    founds = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    ptrs = torch.zeros(bs, dtype=torch.int64, device=DEV)
+    f2 = torch.zeros(bs, dtype=torch.bool, device=DEV)
+    t.find(bs, dev(mixed), out, founds, None)
+    t.find_ptr(bs, dev(mixed), ptrs, f2, None)
+    torch.cuda.synchronize()
+    ov, of, _ = o.find(mixed)
+    assert np.array_equal(founds.cpu().numpy(), of) and np.array_equal(f2.cpu().numpy(), of)
+    assert np.array_equal(out.cpu().numpy()[of], ov[of])
+    gp = ptrs.cpu().numpy()
+    for i in np.flatnonzero(of)[:: 53]:
+        assert np.array_equal(read_device(int(gp[i]), row_bytes), ov[i])
+    t.close()
