@@ -140,8 +140,10 @@ typedef struct hkv_allocator {
  * K=uint64, V=float, S=uint64, LRU. */
 void hkv_options_default(hkv_options* opts);
 
+/* Text of the last error on this thread (the reference throws: debug.hpp:27-72). */
 const char* hkv_last_error(void);
-/* Version string of the library, and the gfx target it was compiled for. */
+/* Version string of the library, and the gfx target it was compiled for (no counterpart in
+ * the reference). */
 const char* hkv_version(void);
 
 /* HashTable::init, merlin_hashtable.cuh:984-1085 (+ create_table,
@@ -291,8 +293,8 @@ int hkv_size_if(const hkv_table* t, int predicate, uint64_t pattern,
 
 /* HashTable::size, merlin_hashtable.cuh:3424-3451.  Synchronises `stream`. */
 int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out);
-/* HashTable::empty :3416, capacity :3487, load_factor :3551, dim :3586,
- * max_bucket_size :3593, bucket_count :3602 */
+/* HashTable::empty merlin_hashtable.cuh:3416, capacity :3487, load_factor :3551, dim :3586,
+ * max_bucket_size :3593, bucket_count :3602 (same file) */
 int hkv_empty(const hkv_table* t, hkv_stream_t stream, int* out);
 uint64_t hkv_capacity(const hkv_table* t);
 int hkv_load_factor(const hkv_table* t, hkv_stream_t stream, float* out);
@@ -305,7 +307,8 @@ int hkv_is_pure_hbm(const hkv_table* t);
 /* HashTable::set_global_epoch, merlin_hashtable.cuh:3760-3762 */
 int hkv_set_global_epoch(hkv_table* t, uint64_t epoch);
 
-/* Layout handle for kernels compiled by the caller (C++ header). */
+/* Layout handle for kernels compiled by the caller (C++ header): what the reference's
+ * templates read from Table<K,V,S> directly (types.cuh:178-220). */
 int hkv_table_get_view(const hkv_table* t, hkv_table_view* out);
 /* The C++ header brackets a caller-compiled kernel with the table's group
  * lock (group_lock.cuh:217-337): role 0 = reader, 1 = updater, 2 = inserter.
