@@ -182,6 +182,12 @@ int table_alloc(hkv_table* t, int type, void** p, size_t bytes) {
   if (!t->own_alloc) {
     if (t->alloc.alloc(t->alloc.ctx, type, p, bytes) != 0 || !*p)
       return fail(HKV_ERROR_RUNTIME, "allocator failed for %zu bytes (type %d)", bytes, type);
+    /* the kernels address the arenas in 16-byte units and 128-byte lines */
+    if (((uintptr_t)*p & 255) != 0) {
+      t->alloc.free(t->alloc.ctx, type, *p);
+      *p = nullptr;
+      return fail(HKV_ERROR_ARGUMENT, "the allocator must return memory aligned to 256 bytes");
+    }
     return HKV_SUCCESS;
   }
   if (type == 0) {
