@@ -71,6 +71,11 @@ def main():
                     help="instead of the one-line benchmark: every entry point at the metric shape "
                          "(capacity 2^26, dim 64, batch 2^20, load factor 1.0), kernel time by HIP "
                          "events and algorithmic GB/s against the 8 TB/s peak, printed as markdown")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="instead of the one-line benchmark: what the memory system needs for the access "
+                         "patterns of find and insert_or_assign at the same shape with no table logic "
+                         "(hierarchicalkv_amd/csrc/hkv_ceilings.hip), and the streaming / gather / scatter / "
+                         "small-access rates they are made of; one JSON line and a markdown table")
     ap.add_argument("--matrix-hybrid", action="store_true",
                     help="with --matrix: the hybrid table of README.md:289-303 (dim 64, capacity "
                          "128M, 16 GB of the rows in HBM, the rest in pinned host memory)")
@@ -94,6 +99,9 @@ def main():
         return
     if args.ops:
         run_ops(args, np, torch, dev, w)
+        return
+    if args.ceilings:
+        run_ceilings(args)
         return
     cap = 1 << args.capacity_log2
     dim = args.dim
@@ -452,6 +460,66 @@ def run_ops(args, np, torch, dev, w):
         print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f |" % (name, ms, n / ms / 1e6, bpk, gbs, gbs / HBM_PEAK_GBS),
               flush=True)
     table.close()
+
+
+CEILING_PATTERNS = [
+    # name, what one launch does, unit of the rate
+    ("stream_read", "16-byte streaming loads over 1 GiB", "GB/s"),
+    ("stream_write", "16-byte streaming stores over 1 GiB", "GB/s"),
+    ("stream_copy", "1 GiB read + 1 GiB written", "GB/s"),
+    ("row_gather", "random table rows -> dense array (read + written bytes)", "GB/s"),
+    ("row_scatter", "dense array -> random table rows, write-through stores (read + written bytes)", "GB/s"),
+    ("find_pattern_1line", "find's accesses, one key line per key, no logic (algorithmic bytes)", "GB/s"),
+    ("find_pattern", "find's accesses, 1.44 key lines per key (false digest matches), no logic "
+                     "(algorithmic bytes)", "GB/s"),
+    ("upsert_pattern", "insert_or_assign's accesses, 50 % absent keys into full buckets, no locks, no logic "
+                       "(algorithmic bytes)", "GB/s"),
+    ("upsert_pattern_locks", "the same plus the slot-lock protocol's atomics, re-reads and unlock stores "
+                             "(algorithmic bytes)", "GB/s"),
+    ("small_load8", "8-byte loads, one per random 128-byte line", "G ops/s"),
+    ("small_store8", "8-byte write-through stores, one per random line", "G ops/s"),
+    ("small_store1", "1-byte write-through stores, one per random line", "G ops/s"),
+    ("small_store16", "16-byte write-through stores, one per random line", "G ops/s"),
+    ("small_chunk64", "aligned 64-byte chunks written by 4 lanes, one per random line", "G ops/s"),
+    ("small_cas64", "64-bit compare-and-swap, one per random line", "G ops/s"),
+    ("small_xchg64", "64-bit exchange, one per random line", "G ops/s"),
+    ("small_xchg32_side", "32-bit exchange on a 4-byte-per-bucket array (fits the Infinity Cache)", "G ops/s"),
+]
+
+
+def run_ceilings(args):
+    """Access-pattern ceilings at the benchmark's shape; see hkv_ceilings.hip."""
+    import ctypes
+
+    path = os.path.join(ROOT, "hierarchicalkv_amd", "libhkv_ceilings.so")
+    if not os.path.exists(path):
+        raise SystemExit("libhkv_ceilings.so is not built: run python hierarchicalkv_amd/build.py ceilings")
+    lib = ctypes.CDLL(path)
+    lib.hkv_ceilings_last_error.restype = ctypes.c_char_p
+    lib.hkv_ceilings_setup.argtypes = [ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint64]
+    lib.hkv_ceilings_run.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                     ctypes.POINTER(ctypes.c_double)]
+    buckets = (1 << args.capacity_log2) // 128
+    vb = args.dim * 4
+    n = 1 << args.batch_log2
+    if lib.hkv_ceilings_setup(buckets, vb, n):
+        raise SystemExit(lib.hkv_ceilings_last_error().decode())
+    reps = max(args.steps, 5)
+    out = {}
+    print("| pattern | what one launch does | ms per launch | rate | fraction of 8 TB/s |")
+    print("|---|---|---|---|---|")
+    for name, what, unit in CEILING_PATTERNS:
+        ms, moved = ctypes.c_double(), ctypes.c_double()
+        if lib.hkv_ceilings_run(name.encode(), reps, ctypes.byref(ms), ctypes.byref(moved)):
+            raise SystemExit(lib.hkv_ceilings_last_error().decode())
+        rate = moved.value / (ms.value * 1e-3) / 1e9
+        out[name] = {"ms": round(ms.value, 5), "rate": round(rate, 2), "unit": unit}
+        frac = "%.3f" % (rate / HBM_PEAK_GBS) if unit == "GB/s" else ""
+        print("| %s | %s | %.4f | %.1f %s | %s |" % (name, what, ms.value, rate, unit, frac), flush=True)
+    lib.hkv_ceilings_release()
+    print(json.dumps({"ceilings": out, "config": {"workload": f"capacity 2^{args.capacity_log2}, dim "
+                                                  f"{args.dim} fp32, batch 2^{args.batch_log2}",
+                                                  "launches_per_pattern": reps}}))
 
 
 def cpu_baseline(args, np, w):

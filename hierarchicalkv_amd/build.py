@@ -38,6 +38,16 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+def build_ceilings(verbose=True):
+    """The access-pattern ceilings of bench.py --ceilings: a measurement tool in a library of its own."""
+    out = os.path.join(PKG_DIR, "libhkv_ceilings.so")
+    cmd = [HIPCC, *HIP_FLAGS, os.path.join(CSRC, "hkv_ceilings.hip"), "-o", out]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
+
+
 def build_cpp_tests(verbose=True):
     """The C++ test of the drop-in header (tests/cpp/api_test.cpp), linked
     against the in-tree library; a GPU test runs the binary."""
@@ -65,9 +75,11 @@ def build_oracle(verbose=True):
 
 
 if __name__ == "__main__":
-    what = sys.argv[1:] or ["lib", "oracle", "cpp"]
+    what = sys.argv[1:] or ["lib", "ceilings", "oracle", "cpp"]
     if "lib" in what:
         build_library()
+    if "ceilings" in what:
+        build_ceilings()
     if "cpp" in what:
         build_cpp_tests()
     if "oracle" in what:

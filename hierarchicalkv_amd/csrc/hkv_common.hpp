@@ -181,11 +181,13 @@ __device__ __forceinline__ uint4 ld_u128_at(const void* base, uint64_t bytes, ui
  * and two 8-byte ones per lane interleave inside a 128-byte line, which the
  * memory side then writes as two half-filled lines each.  The instruction is
  * issued from inline assembly: the wavefront's store counter still covers it
- * (wait_stores), and the s_nop keeps the next instruction from overwriting
- * the data registers while the store reads them. */
+ * (wait_stores).  On gfx940 and later a store of more than 64 bits needs two wait states
+ * before a VALU instruction may overwrite its data registers; the compiler's hazard
+ * recognizer does not look inside inline assembly, so the s_nop 1 (two wait states)
+ * provides them whatever gets scheduled next. */
 __device__ __forceinline__ void st_u128(void* p, const uint4& x) {
   u32x4_t d = {x.x, x.y, x.z, x.w};
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" : : "v"(p), "v"(d) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(p), "v"(d) : "memory");
 }
 /* Slot lock: CAS(expected -> LOCKED) on the key word (the reference's
  * compare_exchange_strong, upsert.cuh:104-110).  On failure `expected` holds
@@ -217,14 +219,18 @@ __device__ __forceinline__ void st_unlock(uint64_t* p, uint64_t x) {
 
 struct Clock {
   uint64_t base;        /* deterministic mode: now(i) = base + (i << 20) */
+  uint64_t offset;      /* hardware mode: Unix-epoch ns at tick 0 of the device counter */
   uint32_t mode;        /* 0 hardware, 1 deterministic */
   uint32_t ns_per_tick; /* hardware mode: constant-rate counter -> ns */
 };
 
-/* device_nano (utils.cuh:75-80) */
+/* device_nano (utils.cuh:75-80): the reference reads %globaltimer, nanoseconds since the Unix
+ * epoch.  The constant-rate counter of the device restarts with the device, so the table keeps
+ * the epoch time of its tick 0 (sampled against the host's CLOCK_REALTIME when the table is
+ * created): scores stay comparable with host time, across processes and after load(). */
 __device__ __forceinline__ uint64_t now_ns(const Clock& c, uint64_t i) {
   if (c.mode == 1) return c.base + (i << 20);
-  return (uint64_t)wall_clock64() * c.ns_per_tick;
+  return c.offset + (uint64_t)wall_clock64() * c.ns_per_tick;
 }
 
 /* ---- row copies by an 8-lane tile ------------------------------------------ */

@@ -43,22 +43,6 @@
 
 #include "hkv_upsert.hpp"
 
-/* phase timing of tuning builds: the first lane of a workgroup adds the ticks
- * since the previous mark to a slot in LDS; one atomic per slot and workgroup
- * at the end */
-#ifdef HKV_STATS
-#define HKV_LMARK_INIT() unsigned long long hkv_lt_ = wall_clock64()
-#define HKV_LMARK(acc, slot)                                  \
-  do {                                                        \
-    const unsigned long long now_ = wall_clock64();           \
-    if (threadIdx.x == 0) (acc)[slot] += now_ - hkv_lt_;      \
-    hkv_lt_ = now_;                                           \
-  } while (0)
-#else
-#define HKV_LMARK_INIT() ((void)0)
-#define HKV_LMARK(acc, slot) ((void)0)
-#endif
-
 namespace hkv {
 
 constexpr int kBinThreads = 1024;   /* histogram / scatter workgroup */
@@ -293,7 +277,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
     const bool needs_old = a.strategy == HKV_LFU || a.strategy == HKV_EPOCH_LFU;
     const uint64_t old = needs_old ? v.scores[slot] : 0;
     uint64_t snew;
-    if (final_score(a, false, desired, in_score, old, snew) && !HKV_EXP_FLAG(256)) v.scores[slot] = snew;
+    if (final_score(a, false, desired, in_score, old, snew)) v.scores[slot] = snew;
   }
   if (OP == kOpAccumOrAssign) {
     /* rows move for the keys that stay "present" only */
@@ -313,7 +297,6 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
   uint8_t* usr_base = (OP == kOpFindOrInsert ? a.values_io : const_cast<uint8_t*>(a.values_in)) +
                       base * v.value_bytes;
   for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
-    if (HKV_EXP_FLAG(1024)) break;
     T buf[kBatch];
     T tab[OP == kOpAccumOrAssign ? kBatch : 1];
 #pragma unroll
@@ -349,7 +332,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
           } else if (OP == kOpAccumOrAssign) {
             st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, add_unit(tab[b], buf[b], a.value_kind));
           } else {
-            if (!HKV_EXP_FLAG(512)) st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
+            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
           }
         }
       }
@@ -469,7 +452,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
   const int tile_base = lane & ~(kTile - 1);
   const uint64_t bslot = (uint64_t)bkt * kBucketSize;
   const uint8_t* rows_in = OP == kOpFindOrInsert ? a.values_io : a.values_in;
-  HKV_LMARK_INIT();
 
   bool dg_dirty = false;
   int size_delta = 0;
@@ -512,7 +494,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       }
     }
 
-    HKV_LMARK(acc, 5); /* free-slot mask, row loads issued */
     /* outcome of key q of the pass, the same in every lane of the tile */
     int got[kGrpKeys];
     uint32_t pos[kGrpKeys];
@@ -632,7 +613,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       dg_dirty = true;
     }
 
-    HKV_LMARK(acc, 6); /* placement */
     /* ---- victims: live key or tombstone ------------------------------------------------------------- */
     uint64_t victim[kGrpKeys];
 #pragma unroll
@@ -731,7 +711,7 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
           (got[q] == kStEmpty || got[q] == kStReclaimed || got[q] == kStEvict) && !cancelled[q];
       if (!writes) continue;
       const uint64_t slot = bslot + pos[q];
-      if (j == 0 && !HKV_EXP_FLAG(128)) {
+      if (j == 0) {
         v.keys[slot] = s_key[q0 + q];
         if (wrs[q]) v.scores[slot] = snew[q];
       }
@@ -740,7 +720,7 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
 #pragma unroll
         for (int w = 0; w < UPL; w++) {
           const uint32_t u = j + w * kTile;
-          if (u < units && !HKV_EXP_FLAG(64)) st_unit<VEC, true>(tb, u, xin[q][w]);
+          if (u < units) st_unit<VEC, true>(tb, u, xin[q][w]);
         }
       } else {
         const uint8_t* us = rows_in + (uint64_t)s_idx[q0 + q] * v.value_bytes;
@@ -760,12 +740,10 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
         }
       }
     }
-    HKV_LMARK(acc, 7); /* victims, keys, rows */
   }
 
-  if (dg_dirty && !HKV_EXP_FLAG(32)) st_u128(v.digests + bslot + j * 16, dg);
+  if (dg_dirty) st_u128(v.digests + bslot + j * 16, dg);
   if (size_delta && j == 0) atomicAdd(v.sizes + bkt, size_delta);
-  HKV_LMARK(acc, 8); /* score and digest write-back */
 }
 
 #ifndef HKV_GROUPED_WAVES_PER_EU
@@ -782,13 +760,7 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
   extern __shared__ uint32_t s_dyn[];
   __shared__ uint32_t s_wsum[kGrpThreads / kWave];
   __shared__ uint32_t s_nwork, s_next;
-#ifdef HKV_STATS
-  __shared__ unsigned long long s_acc[16];
-  if (threadIdx.x < 16) s_acc[threadIdx.x] = 0;
-  __syncthreads();
-#else
   unsigned long long* const s_acc = nullptr;
-#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -800,14 +772,7 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
   const uint32_t first = g.bin_start[bin], last = g.bin_start[bin + 1];
   const uint32_t units = v.value_bytes / VEC;
 
-#ifdef HKV_STATS
-  const unsigned long long t_begin = wall_clock64();
-  unsigned long long t_setup = 0, t_loop = 0;
-#endif
   for (uint32_t c0 = first; c0 < last; c0 += kGrpChunk) {
-#ifdef HKV_STATS
-    const unsigned long long t_c0 = wall_clock64();
-#endif
     const uint32_t cn = last - c0 < (uint32_t)kGrpChunk ? last - c0 : (uint32_t)kGrpChunk;
     for (uint32_t t = tid; t <= bpb; t += kGrpThreads) s_seg[t] = 0;
     if (tid == 0) {
@@ -902,46 +867,23 @@ grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
       return *reinterpret_cast<const uint4*>(v.digests + (uint64_t)(bkt0 + s_work[w]) * kBucketSize +
                                              j * 16);
     };
-#ifdef HKV_STATS
-    const unsigned long long t_c1 = wall_clock64();
-    t_setup += t_c1 - t_c0;
-#endif
     /* the digest line of the next bucket is asked for before the current one is
      * worked on */
     uint32_t w0 = take();
     uint4 dg0 = make_uint4(0, 0, 0, 0);
     if (w0 < nwork) dg0 = digests_of(w0);
-    HKV_LMARK_INIT();
     while (w0 < nwork) {
       const uint32_t w1 = take();
       uint4 dg1 = make_uint4(0, 0, 0, 0);
       if (w1 < nwork) dg1 = digests_of(w1);
       const uint32_t lb = s_work[w0];
-      HKV_LMARK(s_acc, 9); /* take + prefetch issue */
       group_bucket<OP, VEC, UPL>(v, a, g, bkt0 + lb, s_seg[lb], s_seg[lb + 1], s_key, s_idx, s_info,
                                  units, lane, dg0, s_acc);
-      HKV_LMARK(s_acc, 10); /* bucket */
-#ifdef HKV_STATS
-      if (tid == 0) s_acc[4] += 1; /* buckets per workgroup */
-#endif
       w0 = w1;
       dg0 = dg1;
     }
-#ifdef HKV_STATS
-    const unsigned long long t_c2 = wall_clock64();
-    t_loop += t_c2 - t_c1;
-#endif
     __syncthreads();
   }
-#ifdef HKV_STATS
-  if (tid == 0 && first < last) {
-    HKV_COUNT(0, wall_clock64() - t_begin);
-    HKV_COUNT(1, t_setup);
-    HKV_COUNT(2, t_loop);
-    HKV_COUNT(3, 1);
-    for (int k = 4; k < 12; k++) HKV_COUNT(k, s_acc[k]);
-  }
-#endif
 }
 
 }  // namespace hkv

@@ -20,6 +20,7 @@ struct TouchArgs {
   uint64_t** key_ptrs;   /* lock_keys */
   void** value_ptrs;     /* find_and_update */
   uint8_t* flags;        /* success / founds, may be null */
+  unsigned long long* locked_count; /* lock_keys: the table's count of slots left LOCKED */
   uint64_t n;
   uint64_t epoch;
   Clock clock;
@@ -58,11 +59,10 @@ touch_kernel(View v, TouchArgs t) {
   __syncthreads();
   probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
-  if (i >= t.n) return;
   const int64_t slot = s_slot[lane];
   bool ok = false;
   uint64_t score = 0;
-  if (slot >= 0) {
+  if (i < t.n && slot >= 0) {
     /* several updaters may run at once: the slot lock is taken as everywhere */
     uint64_t seen = key;
     for (int tries = 0; tries < kMaxLockedWaits && !ok; tries++) {
@@ -79,6 +79,12 @@ touch_kernel(View v, TouchArgs t) {
       }
     }
   }
+  if (KEEP_LOCKED) {
+    /* one update of the table's count per wavefront */
+    const unsigned long long kept = __ballot(ok);
+    if (kept && lane == (int)__ffsll(kept) - 1) atomicAdd(t.locked_count, (unsigned long long)__popcll(kept));
+  }
+  if (i >= t.n) return;
   if (t.flags) t.flags[i] = ok;
   if (KEEP_LOCKED) {
     t.key_ptrs[i] = ok ? v.keys + slot : nullptr;
@@ -91,16 +97,18 @@ touch_kernel(View v, TouchArgs t) {
 /* unlock_keys_kernel, core_kernels.cuh:1180-1204 */
 __global__ void __launch_bounds__(256)
 unlock_keys_kernel(View v, uint64_t n, uint64_t* const* key_ptrs, const uint64_t* keys,
-                   uint8_t* success) {
+                   uint8_t* success, unsigned long long* locked_count) {
   const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  uint64_t* p = key_ptrs[i];
+  uint64_t* p = i < n ? key_ptrs[i] : nullptr;
   bool ok = false;
   if (p != nullptr && ld_u64(p) == v.locked_key) {
     st_u64(p, keys[i]);
     ok = true;
   }
-  if (success) success[i] = ok;
+  const unsigned long long freed = __ballot(ok);
+  if (freed && (threadIdx.x & (kWave - 1)) == (int)__ffsll(freed) - 1)
+    atomicAdd(locked_count, 0ull - (unsigned long long)__popcll(freed)) /* wraps: a subtraction */;
+  if (i < n && success) success[i] = ok;
 }
 
 }  // namespace hkv

@@ -15,9 +15,9 @@
  *          16 of the 128 digest bytes, so a tile reads one whole 128-byte line
  *          per round; the 8 rounds are issued back to back so 8 KB of digests
  *          are in flight per wavefront;
- *   verify every digest match is checked against the 8-byte key (two
- *          candidates per lane and round are fetched in the batched pass, the
- *          rare third and later ones in a loop); the hit slot goes to LDS;
+ *   verify every digest match is checked against the 8-byte key, the first
+ *          lane's candidates first and the others only if those were not it;
+ *          the hit slot goes to LDS;
  *   copy   the whole wavefront copies the found rows, VEC bytes per lane,
  *          so the output side is written in fully coalesced 1 KB pieces.
  */
@@ -69,7 +69,13 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     if (m.info & 0x100u)
       dg[r] = *reinterpret_cast<const uint4*>(v.digests + (uint64_t)m.bkt * kBucketSize + j * 16);
   }
-  uint32_t cm[kTile];
+  /* Candidates are verified in two steps.  An 8-byte key load costs a whole 128-byte line of
+   * memory traffic, a key that is present has one true candidate, and a false 8-bit match
+   * turns up in every second bucket: so step 1 fetches only the candidates of the first
+   * lane of the tile that has any (a lane's 16 slots share one key line), and the other
+   * lanes' candidates are fetched in step 2 only for the keys step 1 did not find. */
+  uint32_t cm[kTile];    /* this lane's digest matches, bw order */
+  uint32_t later[kTile]; /* lanes of the tile whose candidates wait for step 2 */
   uint64_t k0[kTile], k1[kTile];
 #pragma unroll
   for (int r = 0; r < kTile; r++) {
@@ -79,18 +85,20 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     if (WRITER && s_em != nullptr)
       s_em[tile * kTile + r][j] =
           (uint16_t)(valid ? match16_natural(dg[r], v.empty_digest * 0x01010101u) : 0u);
+    const uint32_t lanes = tile_ballot(cm[r] != 0, tile);
+    later[r] = lanes & (lanes - 1);
     const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
     k0[r] = v.empty_key;
     k1[r] = v.empty_key;
-    if (cm[r]) {
+    if (cm[r] && !((later[r] >> j) & 1u)) {
       k0[r] = kb[bw_to_pos(__ffs(cm[r]) - 1)];
       const uint32_t rest = cm[r] & (cm[r] - 1);
       if (rest) k1[r] = kb[bw_to_pos(__ffs(rest) - 1)];
     }
   }
-#pragma unroll
-  for (int r = 0; r < kTile; r++) {
-    if (!cm[r]) continue;
+  /* checks the candidates of this lane for key r against the fetched words (the third and
+   * later candidates of a lane, rare, are loaded here) */
+  auto check = [&](int r) {
     const int kk = tile * kTile + r;
     const uint64_t key = s_meta[kk].key;
     const uint64_t slot0 = (uint64_t)bkt[r] * kBucketSize + j * 16;
@@ -113,6 +121,29 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
       s_slot[kk] = (int64_t)(slot0 + hit);
     else if (WRITER && unsure)
       s_unsure[kk] = 1;
+    return hit >= 0;
+  };
+  bool more = false;
+#pragma unroll
+  for (int r = 0; r < kTile; r++) {
+    const bool mine = cm[r] && !((later[r] >> j) & 1u);
+    const bool hit = mine && check(r);
+    if (tile_ballot(hit, tile)) later[r] = 0;
+    more |= later[r] != 0;
+  }
+  if (__ballot(more)) {
+#pragma unroll
+    for (int r = 0; r < kTile; r++) {
+      if ((later[r] >> j) & 1u) {
+        const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
+        k0[r] = kb[bw_to_pos(__ffs(cm[r]) - 1)];
+        const uint32_t rest = cm[r] & (cm[r] - 1);
+        if (rest) k1[r] = kb[bw_to_pos(__ffs(rest) - 1)];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kTile; r++)
+      if ((later[r] >> j) & 1u) check(r);
   }
 }
 
@@ -212,16 +243,26 @@ __device__ __forceinline__ void restage_second_bucket(const View& v, KeyMeta* s_
 
 enum LookupMode { kLookupValues = 0, kLookupPtr = 1, kLookupContains = 2 };
 
-template <int MODE, int VEC, bool DUAL = false>
-__global__ void __launch_bounds__(kWave)
+/* WAVES wavefronts per workgroup, each with its own 64 keys and its own staging area.  One
+ * wavefront per workgroup everywhere except the missed-keys variant, whose workgroups are
+ * large so that the list of misses is claimed with one atomic per 1024 keys (updates of one
+ * word are served one at a time, about 15 ns each: one per wavefront would take longer than
+ * the lookup itself). */
+template <int MODE, int VEC, bool DUAL = false, int WAVES = 1>
+__global__ void __launch_bounds__(kWave * WAVES)
 lookup_kernel(View v, FindArgs a) {
-  __shared__ KeyMeta s_meta[kWave];
-  __shared__ int64_t s_slot[kWave];
-  const int lane = threadIdx.x;
-  const uint64_t base = (uint64_t)blockIdx.x * kWave;
+  __shared__ KeyMeta s_meta_all[WAVES][kWave];
+  __shared__ int64_t s_slot_all[WAVES][kWave];
+  __shared__ int32_t s_missed[2]; /* misses of the workgroup, start of its part of the list */
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  KeyMeta* const s_meta = s_meta_all[wave];
+  int64_t* const s_slot = s_slot_all[wave];
+  const uint64_t base = ((uint64_t)blockIdx.x * WAVES + wave) * kWave;
   const uint64_t i = base + lane;
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   if (DUAL) restage_first_bucket(v, s_meta, lane);
+  if (WAVES > 1 && threadIdx.x == 0) s_missed[0] = 0;
   __syncthreads();
   probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
@@ -240,13 +281,28 @@ lookup_kernel(View v, FindArgs a) {
       if (MODE == kLookupPtr) a.out_ptrs[i] = value_row(v, (uint64_t)my_slot);
     } else {
       if (MODE == kLookupPtr) a.out_ptrs[i] = nullptr;
-      if (a.missed_size) {
-        /* missed-keys variant (lookup.cuh:36-60): compact list of misses;
-         * reserved keys are not probed and count as missed. */
-        const int at = atomicAdd(a.missed_size, 1);
-        a.missed_keys[at] = key;
-        a.missed_indices[at] = (int32_t)i;
-      }
+    }
+  }
+  if (a.missed_size) {
+    /* missed-keys variant (lookup.cuh:36-60): compact list of misses, in no particular
+     * order; reserved keys are not probed and count as missed. */
+    const bool miss = i < a.n && my_slot < 0;
+    const unsigned long long mm = __ballot(miss);
+    int32_t at = 0;
+    if (WAVES > 1) {
+      if (lane == 0 && mm) at = atomicAdd(&s_missed[0], (int32_t)__popcll(mm));
+      __syncthreads();
+      if (threadIdx.x == 0 && s_missed[0]) s_missed[1] = atomicAdd(a.missed_size, s_missed[0]);
+      __syncthreads();
+      at = __shfl(at, 0) + s_missed[1];
+    } else {
+      if (lane == 0 && mm) at = atomicAdd(a.missed_size, (int32_t)__popcll(mm));
+      at = __shfl(at, 0);
+    }
+    if (miss) {
+      at += (int32_t)__popcll(mm & ((1ull << lane) - 1));
+      a.missed_keys[at] = key;
+      a.missed_indices[at] = (int32_t)i;
     }
   }
   if (MODE != kLookupValues) return;

@@ -32,7 +32,17 @@ fill_kernel(View v, int zero_scores) {
   if (t < v.buckets_num) v.sizes[t] = 0;
 }
 
-/* remove_kernel (core_kernels.cuh:679-741): tombstone the slot. */
+/* one sample of the constant-rate device counter (table creation: see Clock) */
+__global__ void clock_sample_kernel(unsigned long long* out) { *out = wall_clock64(); }
+
+/* remove_kernel (core_kernels.cuh:679-741): tombstone the slot.
+ * EXCLUSIVE: the call is the only one on the table while it runs (it holds the inserter role
+ * of the group lock), so the key word is overwritten with a plain store as in the reference
+ * (core_kernels.cuh:723-737; like there, a batch that names a key twice in different
+ * wavefronts may count it twice).  Otherwise the slot changes hands with a compare-and-swap.
+ * Keys of an 8-lane tile that fall into one bucket share one update of its size, and a key
+ * that the tile holds twice is erased once. */
+template <bool EXCLUSIVE>
 __global__ void __launch_bounds__(kWave)
 erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   __shared__ KeyMeta s_meta[kWave];
@@ -44,12 +54,39 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   const int64_t slot = s_slot[lane];
-  uint64_t seen = key;
-  if (slot >= 0 && cas_lock(v.keys + slot, seen, v.reclaim_key)) {
-    v.digests[slot] = v.reclaim_digest;
-    v.scores[slot] = 0;
-    atomicSub(v.sizes + (slot >> 7), 1);
+  const int tile_base = lane & ~(kTile - 1), j = lane & (kTile - 1);
+  bool mine = slot >= 0;
+#pragma unroll
+  for (int q = 0; q < kTile; q++) {
+    const int64_t other = __shfl((long long)slot, tile_base + q);
+    if (q < j && other == slot) mine = false; /* the same key earlier in the tile */
   }
+  bool erased = false;
+  if (mine) {
+    if (EXCLUSIVE) {
+      erased = true;
+      v.keys[slot] = v.reclaim_key;
+    } else {
+      uint64_t seen = key;
+      erased = cas_lock(v.keys + slot, seen, v.reclaim_key);
+    }
+    if (erased) {
+      v.digests[slot] = v.reclaim_digest;
+      v.scores[slot] = 0;
+    }
+  }
+  const uint32_t bkt = erased ? (uint32_t)(slot >> 7) : 0xFFFFFFFFu;
+  int same = 0;
+  bool first = true;
+#pragma unroll
+  for (int q = 0; q < kTile; q++) {
+    const uint32_t other = __shfl(bkt, tile_base + q);
+    if (other == bkt) {
+      same++;
+      if (q < j) first = false;
+    }
+  }
+  if (erased && first) atomicSub(v.sizes + bkt, same);
 }
 
 /* Sum of the per-bucket sizes (SumOp over buckets_size, core_kernels.cuh:1395-1423) */

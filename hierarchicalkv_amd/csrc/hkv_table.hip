@@ -10,10 +10,12 @@
 
 #include <algorithm>
 #include <atomic>
+#include <condition_variable>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <map>
 #include <mutex>
 #include <new>
@@ -156,9 +158,11 @@ struct hkv_table {
   uint64_t meta_bytes;
   void* d_values;        /* value rows in HBM */
   void* h_values;        /* host address of the pinned value rows (hybrid) */
-  unsigned long long* d_counters; /* ring of scratch words for size / size_if /
-                                     the count-returning insert_and_evict */
-  mutable std::atomic<unsigned> counter_next;
+  unsigned long long* d_counters; /* scratch words for size / size_if / the count-returning
+                                     insert_and_evict: one per call in flight (CounterLease) */
+  mutable std::mutex counter_mu;
+  mutable std::condition_variable counter_cv;
+  mutable std::vector<unsigned> counter_free;
   uint64_t epoch;
   Clock clock;
   mutable StreamGroupLock lock;
@@ -168,7 +172,10 @@ struct hkv_table {
   uint64_t scratch_bytes;
   int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
-  bool keys_may_be_locked; /* lock_keys has been called: LOCKED key words may sit in the table */
+  bool keys_may_be_locked; /* LOCKED key words may sit in the table (lock_keys, the pointer
+                              overload with locked_key_ptrs), until the count below reads 0 */
+  bool locked_recount;     /* unlock_keys has run since the count was last read */
+  unsigned long long* d_locked; /* device word: slots left LOCKED by those calls, less the unlocked */
   bool dual;               /* TableMode::kMemory: two candidate buckets per key */
   bool io_by_cpu;          /* value rows of the writers are moved by host threads */
   std::mutex io_mutex;     /* one CPU-IO call at a time uses the staging area */
@@ -438,19 +445,73 @@ int run_grouped(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule,
   return HKV_SUCCESS;
 }
 
-constexpr unsigned kCounterRing = 32;
+constexpr unsigned kCounterWords = 128;
 
-/* Calls that return a count synchronise before they return, so at most one
- * word per concurrently calling host thread is in use. */
-unsigned long long* take_counter(const hkv_table* t) {
-  return t->d_counters + (t->counter_next.fetch_add(1) % kCounterRing);
-}
+/* A device word for a call that returns a count.  The word belongs to the call from the
+ * lease to its end (the call zeroes it on its stream, a kernel adds to it, the host reads it
+ * back after a stream synchronisation), so host threads inside such calls never share one;
+ * when all words are out, the next caller waits for one to come back. */
+class CounterLease {
+ public:
+  CounterLease(const hkv_table* t, hipStream_t s) : t_(t), s_(s) {
+    std::unique_lock<std::mutex> g(t->counter_mu);
+    t->counter_cv.wait(g, [&] { return !t->counter_free.empty(); });
+    idx_ = t->counter_free.back();
+    t->counter_free.pop_back();
+  }
+  ~CounterLease() {
+    /* an early return may have left work on the stream that still writes the word */
+    if (!read_) (void)hipStreamSynchronize(s_);
+    {
+      std::lock_guard<std::mutex> g(t_->counter_mu);
+      t_->counter_free.push_back(idx_);
+    }
+    t_->counter_cv.notify_one();
+  }
+  CounterLease(const CounterLease&) = delete;
+  CounterLease& operator=(const CounterLease&) = delete;
+  unsigned long long* word() const { return t_->d_counters + idx_; }
+  /* the word's value once everything enqueued on the stream so far has run */
+  int read(uint64_t* out) {
+    unsigned long long h = 0;
+    HKV_HIP(hipMemcpyAsync(&h, word(), sizeof h, hipMemcpyDeviceToHost, s_));
+    HKV_HIP(hipStreamSynchronize(s_));
+    read_ = true;
+    *out = h;
+    return HKV_SUCCESS;
+  }
 
-int read_counter(unsigned long long* d, hipStream_t s, uint64_t* out) {
-  unsigned long long h = 0;
-  HKV_HIP(hipMemcpyAsync(&h, d, sizeof h, hipMemcpyDeviceToHost, s));
-  HKV_HIP(hipStreamSynchronize(s));
-  *out = h;
+ private:
+  const hkv_table* t_;
+  hipStream_t s_;
+  unsigned idx_ = 0;
+  bool read_ = false;
+};
+
+/* Ties the device counter to the host's CLOCK_REALTIME: the best of a few samples (shortest
+ * host interval around the launch) gives the epoch time of tick 0. */
+int sync_clock(hkv_table* t) {
+  auto host_ns = []() {
+    struct timespec ts;
+    clock_gettime(CLOCK_REALTIME, &ts);
+    return (uint64_t)ts.tv_sec * UINT64_C(1000000000) + (uint64_t)ts.tv_nsec;
+  };
+  unsigned long long* d = t->d_counters;
+  uint64_t best_span = ~UINT64_C(0);
+  for (int rep = 0; rep < 4; rep++) {
+    const uint64_t t0 = host_ns();
+    hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(1), 0, 0, d);
+    HKV_HIP(hipGetLastError());
+    HKV_HIP(hipDeviceSynchronize());
+    const uint64_t t1 = host_ns();
+    unsigned long long ticks = 0;
+    HKV_HIP(hipMemcpy(&ticks, d, sizeof ticks, hipMemcpyDeviceToHost));
+    if (t1 - t0 < best_span) {
+      best_span = t1 - t0;
+      t->clock.offset = t0 + (t1 - t0) / 2 - (uint64_t)ticks * t->clock.ns_per_tick;
+    }
+  }
+  HKV_HIP(hipMemset(d, 0, (kCounterWords + 1) * sizeof(unsigned long long)));
   return HKV_SUCCESS;
 }
 
@@ -570,7 +631,8 @@ int reserve_impl(hkv_table* t, uint64_t new_capacity, hipStream_t s) {
  * 1024) buckets stand for the table; the incoming batch counts as all new */
 int fast_load_factor(hkv_table* t, uint64_t delta, hipStream_t s, float* out) {
   const uint32_t n = (uint32_t)std::min<uint64_t>(t->view.buckets_num, 1024);
-  unsigned long long* d = take_counter(t);
+  CounterLease lease(t, s);
+  unsigned long long* d = lease.word();
   {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
@@ -578,7 +640,7 @@ int fast_load_factor(hkv_table* t, uint64_t delta, hipStream_t s, float* out) {
     HKV_HIP(hipGetLastError());
   }
   uint64_t sum = 0;
-  HKV_TRY(read_counter(d, s, &sum));
+  HKV_TRY(lease.read(&sum));
   *out = (float)((delta * 1.0) / (t->view.capacity * 1.0) + (sum * 1.0) / (kBucketSize * n * 1.0));
   return HKV_SUCCESS;
 }
@@ -592,6 +654,20 @@ int grow_for(hkv_table* t, uint64_t n, hipStream_t s) {
     if (!(lf > t->opts.max_load_factor)) break;
     HKV_TRY(reserve_impl(t, t->view.capacity * 2, s));
   }
+  return HKV_SUCCESS;
+}
+
+/* Slots left LOCKED between calls make the upserts scan key words beside the scores and keep
+ * them off the two-phase path.  After an unlock_keys the device count is read once (the caller
+ * holds the inserter role on `s`, so the unlock has been ordered before this point); at zero
+ * the table is back to the plain kernels. */
+int settle_locked_count(hkv_table* t, hipStream_t s) {
+  if (!t->keys_may_be_locked || !t->locked_recount) return HKV_SUCCESS;
+  long long left = 0;
+  HKV_HIP(hipMemcpyAsync(&left, t->d_locked, sizeof left, hipMemcpyDeviceToHost, s));
+  HKV_HIP(hipStreamSynchronize(s));
+  t->locked_recount = false;
+  if (left <= 0) t->keys_may_be_locked = false;
   return HKV_SUCCESS;
 }
 
@@ -609,6 +685,8 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
+    HKV_TRY(settle_locked_count(t, s));
+    if (OP == kOpFindOrInsertPtr && a.locked_key_ptrs) t->keys_may_be_locked = true;
     GroupPlan plan{};
     if constexpr (OP != kOpFindOrInsertPtr) plan = plan_grouped(t, a.n);
     /* insert_and_evict: the second phase updates the one evicted-counter word once per
@@ -844,6 +922,18 @@ void launch_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((lookup_kernel<MODE, 1>), grid, block, 0, s, v, a);
 }
 
+/* the missed-keys find: 16 wavefronts per workgroup (see lookup_kernel) */
+void launch_lookup_missed(int vec, const View& v, const FindArgs& a, hipStream_t s) {
+  constexpr int kWaves = 16;
+  const dim3 grid((unsigned)((a.n + kWave * kWaves - 1) / (kWave * kWaves))), block(kWave * kWaves);
+  if (vec == 16)
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 16, false, kWaves>), grid, block, 0, s, v, a);
+  else if (vec == 4)
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 4, false, kWaves>), grid, block, 0, s, v, a);
+  else
+    hipLaunchKernelGGL((lookup_kernel<kLookupValues, 1, false, kWaves>), grid, block, 0, s, v, a);
+}
+
 template <bool LOCKFREE>
 void launch_assign(int vec, const View& v, const AssignArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
@@ -946,6 +1036,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->d_scratch = nullptr;
   t->scratch_bytes = 0;
   t->keys_may_be_locked = false;
+  t->locked_recount = false;
   t->dual = o->table_mode == 1;
   t->io_by_cpu = o->io_by_cpu != 0;
   t->io_stage = nullptr;
@@ -959,10 +1050,10 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
     if (!strcmp(e, "locked")) t->upsert_path = 1;
     if (!strcmp(e, "grouped")) t->upsert_path = 2;
   }
-  t->counter_next = 0;
   memset(&t->view, 0, sizeof t->view);
   t->epoch = kIgnoredEpoch;
   t->clock.base = 0;
+  t->clock.offset = 0;
   t->clock.mode = 0;
   t->clock.ns_per_tick = 10;
 
@@ -1040,10 +1131,16 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->pure_hbm = v.hbm_slots == v.capacity;
   void* cnt = nullptr;
   {
-    int rc = table_alloc(t, 0, &cnt, kCounterRing * sizeof(unsigned long long));
+    int rc = table_alloc(t, 0, &cnt, (kCounterWords + 1) * sizeof(unsigned long long));
     if (rc) return bail(rc);
   }
   t->d_counters = (unsigned long long*)cnt;
+  for (unsigned w = 0; w < kCounterWords; w++) t->counter_free.push_back(w);
+  t->d_locked = t->d_counters + kCounterWords;
+  {
+    int rc = sync_clock(t);
+    if (rc) return bail(rc);
+  }
   t->reach_max_capacity = t->dual || o->init_capacity * 2 > o->max_capacity; /* merlin_hashtable.cuh:1064-1069 */
   *out = t;
   return HKV_SUCCESS;
@@ -1174,12 +1271,13 @@ int hkv_insert_and_evict_count(hkv_table* t, uint64_t n, const uint64_t* keys,
   *n_evicted = 0;
   if (n == 0) return HKV_SUCCESS;
   hipStream_t s = (hipStream_t)stream;
-  unsigned long long* d = take_counter(t);
+  CounterLease lease(t, s);
+  unsigned long long* d = lease.word();
   hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
   HKV_TRY(hkv_insert_and_evict(t, n, keys, values, scores, evicted_keys,
                                evicted_values, evicted_scores, (uint64_t*)d,
                                stream, unique_key, ignore));
-  return read_counter(d, s, n_evicted);
+  return lease.read(n_evicted);
 }
 
 int hkv_accum_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
@@ -1250,7 +1348,7 @@ int hkv_find_or_insert_ptr_lock(hkv_table* t, uint64_t n, const uint64_t* keys, 
   a.locked_key_ptrs = locked_key_ptrs;
   a.n = n;
   a.strategy = strategy;
-  t->keys_may_be_locked = true; /* LOCKED key words stay behind until unlock_keys */
+  a.locked_count = t->d_locked; /* LOCKED key words stay behind until unlock_keys */
   return run_upsert<kOpFindOrInsertPtr>(t, a, 16, true, (hipStream_t)stream);
 }
 
@@ -1409,7 +1507,7 @@ int hkv_find_missed(const hkv_table* t, uint64_t n, const uint64_t* keys,
   hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(1), 0, s, missed_size);
   LockGuard g(t, StreamGroupLock::kReader, s);
   HKV_HIP(g.acquire());
-  launch_lookup<kLookupValues>(vec, t->view, a, s);
+  launch_lookup_missed(vec, t->view, a, s);
   HKV_HIP(hipGetLastError());
   return HKV_SUCCESS;
 }
@@ -1461,6 +1559,7 @@ int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys, uint64_t** loc
   a.scores = const_cast<uint64_t*>(scores);
   a.key_ptrs = locked_key_ptrs;
   a.flags = success;
+  a.locked_count = t->d_locked;
   a.n = n;
   a.epoch = t->epoch;
   a.clock = t->clock;
@@ -1484,8 +1583,9 @@ int hkv_unlock_keys(hkv_table* t, uint64_t n, uint64_t** locked_key_ptrs, const 
   LockGuard g(t, StreamGroupLock::kInserter, s);
   HKV_HIP(g.acquire());
   hipLaunchKernelGGL(unlock_keys_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, t->view,
-                     n, locked_key_ptrs, keys, success);
+                     n, locked_key_ptrs, keys, success, t->d_locked);
   HKV_HIP(hipGetLastError());
+  t->locked_recount = true;
   return HKV_SUCCESS;
 }
 
@@ -1521,7 +1621,11 @@ int hkv_erase(hkv_table* t, uint64_t n, const uint64_t* keys, hkv_stream_t strea
   hipStream_t s = (hipStream_t)stream;
   LockGuard g(t, StreamGroupLock::kInserter, s);
   HKV_HIP(g.acquire());
-  hipLaunchKernelGGL(erase_kernel, dim3(grid_for(n)), dim3(kWave), 0, s, t->view, keys, n);
+  /* with the group lock on, the inserter role makes this call the only one on the table */
+  if (t->opts.api_lock)
+    hipLaunchKernelGGL(erase_kernel<true>, dim3(grid_for(n)), dim3(kWave), 0, s, t->view, keys, n);
+  else
+    hipLaunchKernelGGL(erase_kernel<false>, dim3(grid_for(n)), dim3(kWave), 0, s, t->view, keys, n);
   HKV_HIP(hipGetLastError());
   return HKV_SUCCESS;
 }
@@ -1541,10 +1645,13 @@ int hkv_set_max_capacity(hkv_table* t, uint64_t new_max_capacity) {
 }
 
 int hkv_clear(hkv_table* t, hkv_stream_t stream) {
-  t->keys_may_be_locked = false;
   hipStream_t s = (hipStream_t)stream;
   LockGuard g(t, StreamGroupLock::kInserter, s);
   HKV_HIP(g.acquire());
+  /* every key word becomes EMPTY, the LOCKED ones included */
+  t->keys_may_be_locked = false;
+  t->locked_recount = false;
+  hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, t->d_locked);
   const uint64_t groups = t->view.capacity / 16;
   hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s,
                      t->view, 0);
@@ -1602,7 +1709,8 @@ int hkv_size_if(const hkv_table* t, int predicate, uint64_t pattern,
   hipStream_t s = (hipStream_t)stream;
   if (predicate < HKV_PRED_ALWAYS || predicate > HKV_PRED_KEY_HIGH16_EQ_AND_SCORE_LT)
     return fail(HKV_ERROR_ARGUMENT, "unknown predicate %d", predicate);
-  unsigned long long* d = take_counter(t);
+  CounterLease lease(t, s);
+  unsigned long long* d = lease.word();
   {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
@@ -1617,12 +1725,13 @@ int hkv_size_if(const hkv_table* t, int predicate, uint64_t pattern,
     }
     HKV_HIP(hipGetLastError());
   }
-  return read_counter(d, s, out);
+  return lease.read(out);
 }
 
 int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out) {
   hipStream_t s = (hipStream_t)stream;
-  unsigned long long* d = take_counter(t);
+  CounterLease lease(t, s);
+  unsigned long long* d = lease.word();
   {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
@@ -1632,7 +1741,7 @@ int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out) {
     hipLaunchKernelGGL(size_kernel, dim3(blocks), dim3(256), 0, s, t->view, d);
     HKV_HIP(hipGetLastError());
   }
-  return read_counter(d, s, out);
+  return lease.read(out);
 }
 
 int hkv_empty(const hkv_table* t, hkv_stream_t stream, int* out) {
@@ -1679,26 +1788,6 @@ int hkv_lock_end(const hkv_table* t, int role, hkv_stream_t stream) {
   HKV_HIP(t->lock.end((StreamGroupLock::Role)role, (hipStream_t)stream));
   return HKV_SUCCESS;
 }
-
-#ifdef HKV_STATS
-/* tuning builds only: read and clear the event counters */
-int hkv_debug_stats(uint64_t* out16) {
-  HKV_HIP(hipDeviceSynchronize());
-  HKV_HIP(hipMemcpyFromSymbol(out16, HIP_SYMBOL(g_hkv_stats), 16 * sizeof(uint64_t)));
-  uint64_t z[16] = {0};
-  HKV_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_hkv_stats), z, sizeof z));
-  return HKV_SUCCESS;
-}
-#endif
-
-#ifdef HKV_EXP
-/* tuning builds only: select the phases the upsert kernel skips */
-int hkv_debug_set_exp(int flags) {
-  HKV_HIP(hipDeviceSynchronize());
-  HKV_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_hkv_exp), &flags, sizeof flags));
-  return HKV_SUCCESS;
-}
-#endif
 
 int hkv_set_clock(hkv_table* t, int mode, uint64_t base) {
   if (mode != 0 && mode != 1) return fail(HKV_ERROR_ARGUMENT, "bad clock mode %d", mode);

@@ -58,6 +58,7 @@ struct UpsertArgs {
   uint64_t** locked_key_ptrs; /* same overload: when given, the slots stay LOCKED and their key
                                  addresses go here (find_ptr_or_insert.cuh:232-242) */
   uint8_t* founds;
+  unsigned long long* locked_count;   /* with locked_key_ptrs: the table's count of slots left LOCKED */
   uint64_t n;
   uint64_t epoch;
   Clock clock;
@@ -226,11 +227,7 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
       reinterpret_cast<T*>(row)[u] = x;
     }
   } else if constexpr (VEC == 16) {
-#ifdef HKV_EXP_PLAIN_ROW_STORES
-    reinterpret_cast<T*>(row)[u] = x;
-#else
     st_u128(row + 16 * (size_t)u, x);
-#endif
   } else if constexpr (VEC == 8) {
     st_u64(reinterpret_cast<uint64_t*>(row) + u, x.x | ((uint64_t)x.y << 32));
   } else if constexpr (VEC == 4) {
@@ -242,42 +239,6 @@ __device__ __forceinline__ void st_unit(uint8_t* row, uint32_t u, typename VecTy
     st_u8(row + u, x);
   }
 }
-
-/* Optional event counters for tuning builds (-DHKV_STATS): trips of the retry
- * loop, scans, failed lock attempts.  Not compiled into the shipped library. */
-#ifdef HKV_STATS
-__device__ unsigned long long g_hkv_stats[16];
-#define HKV_COUNT(slot, n) atomicAdd(&g_hkv_stats[slot], (unsigned long long)(n))
-/* phase timing: lane 0 adds the cycles since the previous mark to a counter */
-#define HKV_MARK_INIT() unsigned long long hkv_t_ = wall_clock64()
-#define HKV_MARK(slot)                                                   \
-  do {                                                                   \
-    const unsigned long long now_ = wall_clock64();                      \
-    if (threadIdx.x == 0) atomicAdd(&g_hkv_stats[slot], now_ - hkv_t_);  \
-    hkv_t_ = now_;                                                       \
-  } while (0)
-#else
-#define HKV_COUNT(slot, n) ((void)0)
-#define HKV_MARK_INIT() ((void)0)
-#define HKV_MARK(slot) ((void)0)
-#endif
-
-/* Knock-out switches for tuning builds (-DHKV_EXP): a device word selects
- * phases to skip, to apportion a launch's time.  Results are wrong by design. */
-#ifdef HKV_EXP
-__device__ int g_hkv_exp;
-#define HKV_EXP_FLAG(bit) ((g_hkv_exp & (bit)) != 0)
-#else
-#define HKV_EXP_FLAG(bit) false
-#endif
-
-#ifndef HKV_SCAN_PAIR
-#define HKV_SCAN_PAIR 1
-#endif
-#ifndef HKV_UPSERT_MIN_WAVES
-#define HKV_UPSERT_MIN_WAVES 1
-#endif
-constexpr bool kScanPair = HKV_SCAN_PAIR;
 
 enum : int {
   kStNone = 0, /* no lock taken (yet) */
@@ -553,7 +514,7 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * refused at score == min is a separate switch (UpsertArgs::refuse_equal).
  */
 template <int OP, int VEC, int UPL, bool LOCKED_RULE>
-__global__ void __launch_bounds__(kWave, HKV_UPSERT_MIN_WAVES)
+__global__ void __launch_bounds__(kWave)
 upsert_kernel(View v, UpsertArgs a) {
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
@@ -565,14 +526,12 @@ upsert_kernel(View v, UpsertArgs a) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
 
-  HKV_MARK_INIT();
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
   s_unsure[lane] = 0;
   __syncthreads();
   probe_wave<true>(v, s_meta, s_slot, s_em, s_unsure, lane);
   __syncthreads();
-  HKV_MARK(9); /* probe */
 
   /* ---- state of the key this lane owns ---------------------------------------------- */
   const KeyMeta me = s_meta[lane];
@@ -587,7 +546,6 @@ upsert_kernel(View v, UpsertArgs a) {
     em_hi = e.z | ((uint64_t)e.w << 32);
   }
   bool pending = (me.info & 0x100u) != 0;
-  if (HKV_EXP_FLAG(4)) pending = false;
   bool reprobe = pending && hit < 0 && s_unsure[lane];
   int waited = 0;
 
@@ -602,11 +560,6 @@ upsert_kernel(View v, UpsertArgs a) {
     const bool active = pending && !reprobe;
     const uint64_t desired = desired_when_missed(a, in_score, i);
     int got = kStNone;
-    if (lane == 0) {
-      HKV_COUNT(0, 1);                                   /* trips */
-      HKV_COUNT(1, __popcll(pend_mask));                 /* pending keys over trips */
-      HKV_COUNT(2, __popcll(__ballot(pending && reprobe))); /* unsettled reprobes */
-    }
     uint32_t pos = 0;
     uint64_t victim = 0;
 
@@ -624,10 +577,7 @@ upsert_kernel(View v, UpsertArgs a) {
            * batch, or the probe was looking at somebody else's lock */
           hit = -1;
           reprobe = true;
-          HKV_COUNT(3, 1);
-        } else {
-          HKV_COUNT(4, 1); /* hit slot locked by somebody else */
-        }
+        } /* else: the hit slot is locked by somebody else right now; next trip */
       } else if (em_lo | em_hi) {
         /* up to three free slots, the first at or after the key's start position
          * so that keys of one bucket spread over the free slots */
@@ -643,20 +593,13 @@ upsert_kernel(View v, UpsertArgs a) {
             got = kStEmpty;
             pos = p;
             victim = v.empty_key;
-          } else {
-            HKV_COUNT(5, 1); /* lost a free slot */
           }
         }
       } else {
-        if (HKV_EXP_FLAG(2))
-          got = kStRefused;
-        else
-          want_scan = true;
-        HKV_COUNT(6, 1); /* scans */
+        want_scan = true;
       }
     }
 
-    HKV_MARK(10); /* step 1 */
     /* ---- step 2: full buckets: min-score scan by the tile, two buckets in flight ------------ */
     uint64_t best = kMaxScore;
     uint32_t bpos = 0;
@@ -667,8 +610,8 @@ upsert_kernel(View v, UpsertArgs a) {
         if (need) {
           const int r0 = __ffs(need) - 1;
           need &= need - 1;
-          const int r1 = (kScanPair && need) ? __ffs(need) - 1 : r0;
-          if (kScanPair) need &= need - 1; /* no-op when need is already 0 */
+          const int r1 = need ? __ffs(need) - 1 : r0;
+          need &= need - 1; /* no-op when need is already 0 */
           const uint64_t bs0 = __shfl((unsigned long long)bslot, lane_base + r0);
           const uint64_t bs1 = __shfl((unsigned long long)bslot, lane_base + r1);
           uint64_t sc0[2 * kTile], sc1[2 * kTile];
@@ -691,11 +634,10 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
-    HKV_MARK(11); /* scans */
     /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
     bool refused_now = false;
     if (want_scan) {
-      const bool refuse = (a.refuse_equal ? (desired <= best) : (desired < best)) || HKV_EXP_FLAG(16);
+      const bool refuse = (a.refuse_equal ? (desired <= best) : (desired < best));
       if (refuse) {
         refused_now = true;
         got = kStRefused;
@@ -715,15 +657,11 @@ upsert_kernel(View v, UpsertArgs a) {
             pos = bpos;
           } else {
             st_unlock(kp, vk); /* nothing was written under this lock */
-            HKV_COUNT(7, 1); /* score was raised between scan and lock */
           }
-        } else {
-          HKV_COUNT(8, 1); /* victim locked or taken by somebody else */
-        }
+        } /* else: the victim is locked or was taken by somebody else; next trip */
       }
     }
 
-    HKV_MARK(12); /* victim lock */
     /* ---- step 4: critical sections of every lock taken in this trip ------------------------------ */
     const bool locked = got != kStNone && got != kStRefused;
     const uint64_t slot = bslot + pos;
@@ -744,17 +682,15 @@ upsert_kernel(View v, UpsertArgs a) {
       if (votes) {
         const int leader = (int)__ffsll(votes) - 1;
         unsigned long long base_idx = 0;
-        if (HKV_EXP_FLAG(128))
-          base_idx = (unsigned long long)blockIdx.x * 32;
-        else if (lane == leader)
+        if (lane == leader)
           base_idx = atomicAdd(a.evicted_counter, (unsigned long long)__popcll(votes));
         base_idx = __shfl(base_idx, leader);
         const unsigned long long idx = base_idx + __popcll(votes & ((1ull << lane) - 1));
-        if (emit && !HKV_EXP_FLAG(64)) {
+        if (emit) {
           a.evicted_keys[idx] = refused_now ? key : victim;
           if (a.evicted_scores) a.evicted_scores[idx] = refused_now ? desired : best;
         }
-        bulk_evicted<VEC, UPL>(emit && !HKV_EXP_FLAG(32) ? (refused_now ? 1 : 2) : 0,
+        bulk_evicted<VEC, UPL>(emit ? (refused_now ? 1 : 2) : 0,
                                refused_now ? a.values_in + i * v.value_bytes : row,
                                a.evicted_values + idx * v.value_bytes, units, lane);
       }
@@ -764,7 +700,7 @@ upsert_kernel(View v, UpsertArgs a) {
       a.founds[i] = got == kStDuplicate;
       if (a.locked_key_ptrs) a.locked_key_ptrs[i] = locked ? v.keys + slot : nullptr;
     }
-    if (commit && !HKV_EXP_FLAG(8)) {
+    if (commit) {
       write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
       if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
     }
@@ -783,19 +719,20 @@ upsert_kernel(View v, UpsertArgs a) {
           usr = const_cast<uint8_t*>(a.values_in) + i * v.value_bytes;
         }
       }
-      if (HKV_EXP_FLAG(1)) move = kMoveNone;
       if (__ballot(move != kMoveNone))
         bulk_rows<VEC, UPL, OP == kOpFindOrInsert, OP == kOpAccumOrAssign>(
             move, row, usr, units, a.value_kind, lane);
     }
 
-    HKV_MARK(13); /* meta + bulk issue */
     /* ---- step 5: everything written under the locks is out; release them --------------------------- */
     wait_stores();
-    HKV_MARK(14); /* store drain */
     /* the pointer overload may be asked to leave its slots locked for unlock_keys */
     const bool keep_locked = OP == kOpFindOrInsertPtr && a.locked_key_ptrs != nullptr;
     if (locked && !keep_locked) st_unlock(v.keys + slot, commit ? key : victim);
+    if (keep_locked) {
+      const unsigned long long kept = __ballot(locked);
+      if (kept && lane == (int)__ffsll(kept) - 1) atomicAdd(a.locked_count, (unsigned long long)__popcll(kept));
+    }
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
     if (pend_mask) __builtin_amdgcn_s_sleep(1);

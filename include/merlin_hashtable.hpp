@@ -449,6 +449,61 @@ inline int free_cb(void* ctx, int type, void* ptr) {
   }
 }
 
+/* A staging array of save / load: device memory or pinned host memory, freed by the destructor. */
+template <class T>
+class StageBuffer {
+ public:
+  StageBuffer(size_t count, bool pinned_host) : host_(pinned_host) {
+    void* p = nullptr;
+    if (host_)
+      HKV_HIP_CHECK(hipHostMalloc(&p, count * sizeof(T)));
+    else
+      HKV_HIP_CHECK(hipMalloc(&p, count * sizeof(T)));
+    p_ = static_cast<T*>(p);
+  }
+  ~StageBuffer() {
+    if (p_ == nullptr) return;
+    if (host_)
+      (void)hipHostFree(p_);
+    else
+      (void)hipFree(p_);
+  }
+  StageBuffer(const StageBuffer&) = delete;
+  StageBuffer& operator=(const StageBuffer&) = delete;
+  T* get() const { return p_; }
+
+ private:
+  bool host_;
+  T* p_ = nullptr;
+};
+
+/* One device word from the stream-ordered allocator for a call that returns a count; given
+ * back on every way out of the call. */
+template <class T>
+class DeviceWord {
+ public:
+  explicit DeviceWord(hipStream_t s) : s_(s) {
+    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&p_), sizeof(T), s_));
+  }
+  ~DeviceWord() {
+    if (p_ != nullptr) (void)hipFreeAsync(p_, s_);
+  }
+  DeviceWord(const DeviceWord&) = delete;
+  DeviceWord& operator=(const DeviceWord&) = delete;
+  T* get() const { return p_; }
+  /* the word's value once the stream has run everything enqueued so far */
+  T read() const {
+    T h{};
+    HKV_HIP_CHECK(hipMemcpyAsync(&h, p_, sizeof h, hipMemcpyDeviceToHost, s_));
+    HKV_HIP_CHECK(hipStreamSynchronize(s_));
+    return h;
+  }
+
+ private:
+  hipStream_t s_;
+  T* p_ = nullptr;
+};
+
 /* RAII bracket of the table's group lock around a caller-compiled kernel */
 struct RoleGuard {
   const hkv_table* t;
@@ -695,14 +750,16 @@ class HashTable : public HashTableBase<K, V, S> {
    * returns how many (merlin_hashtable.cuh:2963-2996).  Synchronises `stream`. */
   template <template <typename, typename> class PredFunctor>
   size_type erase_if(const key_type& pattern, const score_type& threshold, hipStream_t stream = 0) {
-    hkv_table_view v;
-    throw_on_error_(hkv_table_get_view(table_, &v));
-    unsigned long long* d_count = nullptr;
-    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
+    detail::DeviceWord<unsigned long long> count(stream);
+    unsigned long long* d_count = count.get();
     hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
                        d_count);
     {
+      /* the role is taken first: it keeps other host threads from growing the table (which
+       * frees the arenas the view points at) until this call has enqueued its kernel */
       detail::RoleGuard g(table_, 2, stream);
+      hkv_table_view v;
+      throw_on_error_(hkv_table_get_view(table_, &v));
       const unsigned blocks = hkv::scan_grid(v.capacity, 256);
       hipLaunchKernelGGL((hkv::erase_if_kernel<detail::PredAdapter<K, S, PredFunctor>>),
                          dim3(blocks), dim3(256), 0, stream, v,
@@ -710,25 +767,21 @@ class HashTable : public HashTableBase<K, V, S> {
                          static_cast<uint64_t>(threshold), d_count);
       HKV_HIP_CHECK(hipGetLastError());
     }
-    unsigned long long h = 0;
-    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
-    HKV_HIP_CHECK(hipStreamSynchronize(stream));
-    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
-    return static_cast<size_type>(h);
+    return static_cast<size_type>(count.read());
   }
 
   /* merlin_hashtable.cuh:3008-3052: pred.template operator()<GroupSize>(key, value, score, tile)
    * decides; returns how many entries were erased.  Synchronises `stream`. */
   template <typename PredFunctor>
   size_type erase_if_v2(PredFunctor& pred, hipStream_t stream = 0) {
-    hkv_table_view v;
-    throw_on_error_(hkv_table_get_view(table_, &v));
-    unsigned long long* d_count = nullptr;
-    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
+    detail::DeviceWord<unsigned long long> count(stream);
+    unsigned long long* d_count = count.get();
     hipLaunchKernelGGL((hkv::zero_word_kernel<unsigned long long>), dim3(1), dim3(1), 0, stream,
                        d_count);
     {
       detail::RoleGuard g(table_, 2, stream);
+      hkv_table_view v;
+      throw_on_error_(hkv_table_get_view(table_, &v));
       const uint64_t n = v.capacity;
       const unsigned blocks = hkv::scan_grid(n, 128);
       const uint64_t dim = options_.dim;
@@ -746,11 +799,7 @@ class HashTable : public HashTableBase<K, V, S> {
                            dim3(128), 0, stream, v, n, pred, d_count);
       HKV_HIP_CHECK(hipGetLastError());
     }
-    unsigned long long h = 0;
-    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
-    HKV_HIP_CHECK(hipStreamSynchronize(stream));
-    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
-    return static_cast<size_type>(h);
+    return static_cast<size_type>(count.read());
   }
 
   /* merlin_hashtable.cuh:3307-3348 */
@@ -758,9 +807,9 @@ class HashTable : public HashTableBase<K, V, S> {
   void export_batch_if_v2(PredFunctor& pred, size_type n, const size_type offset,
                           size_type* d_counter, key_type* keys, value_type* values,
                           score_type* scores = nullptr, hipStream_t stream = 0) const {
+    detail::RoleGuard g(table_, 0, stream);
     hkv_table_view v;
     throw_on_error_(hkv_table_get_view(table_, &v));
-    detail::RoleGuard g(table_, 0, stream);
     hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
     if (offset >= v.capacity) return;
     n = std::min<size_type>(v.capacity - offset, n);
@@ -788,10 +837,10 @@ class HashTable : public HashTableBase<K, V, S> {
   template <typename ExecutionFunc>
   void for_each(const size_type first, const size_type last, ExecutionFunc& f,
                 hipStream_t stream = 0) {
+    detail::RoleGuard g(table_, 2, stream);
     hkv_table_view v;
     throw_on_error_(hkv_table_get_view(table_, &v));
     if (first >= v.capacity || last > v.capacity || first >= last) return;
-    detail::RoleGuard g(table_, 2, stream);
     const uint64_t n = last - first;
     const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
     const uint64_t dim = options_.dim;
@@ -824,15 +873,9 @@ class HashTable : public HashTableBase<K, V, S> {
   size_type export_batch(const size_type n, const size_type offset, key_type* keys,
                          value_type* values, score_type* scores = nullptr,
                          hipStream_t stream = 0) const override {
-    size_type* d_counter = nullptr;
-    size_type h_counter = 0;
-    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_counter), sizeof(size_type), stream));
-    export_batch(n, offset, d_counter, keys, values, scores, stream);
-    HKV_HIP_CHECK(
-        hipMemcpyAsync(&h_counter, d_counter, sizeof(size_type), hipMemcpyDeviceToHost, stream));
-    HKV_HIP_CHECK(hipStreamSynchronize(stream));
-    HKV_HIP_CHECK(hipFreeAsync(d_counter, stream));
-    return h_counter;
+    detail::DeviceWord<size_type> count(stream);
+    export_batch(n, offset, count.get(), keys, values, scores, stream);
+    return count.read();
   }
 
   /* merlin_hashtable.cuh:3193-3276: the caller's device functor decides. */
@@ -841,9 +884,9 @@ class HashTable : public HashTableBase<K, V, S> {
                        const size_type offset, size_type* d_counter, key_type* keys,
                        value_type* values, score_type* scores = nullptr,
                        hipStream_t stream = 0) const {
+    detail::RoleGuard g(table_, 0, stream);
     hkv_table_view v;
     throw_on_error_(hkv_table_get_view(table_, &v));
-    detail::RoleGuard g(table_, 0, stream);
     hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
     if (offset >= v.capacity) return;
     n = std::min<size_type>(v.capacity - offset, n);
@@ -864,9 +907,9 @@ class HashTable : public HashTableBase<K, V, S> {
   template <template <typename, typename> class PredFunctor>
   void size_if(const key_type& pattern, const score_type& threshold, size_type* d_counter,
                hipStream_t stream = 0) const {
+    detail::RoleGuard g(table_, 0, stream);
     hkv_table_view v;
     throw_on_error_(hkv_table_get_view(table_, &v));
-    detail::RoleGuard g(table_, 0, stream);
     hipLaunchKernelGGL((hkv::zero_word_kernel<size_type>), dim3(1), dim3(1), 0, stream, d_counter);
     const unsigned blocks = hkv::scan_grid(v.capacity, 256);
     hipLaunchKernelGGL((hkv::size_if_kernel<detail::PredAdapter<K, S, PredFunctor>>), dim3(blocks),
@@ -881,14 +924,9 @@ class HashTable : public HashTableBase<K, V, S> {
   template <template <typename, typename> class PredFunctor>
   size_type size_if(const key_type& pattern, const score_type& threshold,
                     hipStream_t stream = 0) const {
-    unsigned long long* d_count = nullptr;
-    HKV_HIP_CHECK(hipMallocAsync(reinterpret_cast<void**>(&d_count), sizeof(*d_count), stream));
-    size_if<PredFunctor>(pattern, threshold, reinterpret_cast<size_type*>(d_count), stream);
-    unsigned long long h = 0;
-    HKV_HIP_CHECK(hipMemcpyAsync(&h, d_count, sizeof h, hipMemcpyDeviceToHost, stream));
-    HKV_HIP_CHECK(hipStreamSynchronize(stream));
-    HKV_HIP_CHECK(hipFreeAsync(d_count, stream));
-    return static_cast<size_type>(h);
+    detail::DeviceWord<size_type> count(stream);
+    size_if<PredFunctor>(pattern, threshold, count.get(), stream);
+    return count.read();
   }
 
   bool empty(hipStream_t stream = 0) const override { return size(stream) == 0; }
@@ -937,18 +975,13 @@ class HashTable : public HashTableBase<K, V, S> {
                  "[HierarchicalKV] max_workspace_size is smaller than a single `key + score + value` tuple! Please set a larger value!");
     const size_type total = capacity();
     const size_type window = std::max<size_type>(max_workspace_size / tuple_size, 1);
-    K* d_keys = nullptr;
-    V* d_vals = nullptr;
-    S* d_scores = nullptr;
-    K* h_keys = nullptr;
-    V* h_vals = nullptr;
-    S* h_scores = nullptr;
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_keys), window * sizeof(K)));
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_vals), window * sizeof(V) * dim()));
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_scores), window * sizeof(S)));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_keys), window * sizeof(K)));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_vals), window * sizeof(V) * dim()));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_scores), window * sizeof(S)));
+    /* released on every way out, also when export_batch or the file throws */
+    detail::StageBuffer<K> dk(window, false), hk(window, true);
+    detail::StageBuffer<V> dv(window * dim(), false), hv(window * dim(), true);
+    detail::StageBuffer<S> ds(window, false), hs(window, true);
+    K *d_keys = dk.get(), *h_keys = hk.get();
+    V *d_vals = dv.get(), *h_vals = hv.get();
+    S *d_scores = ds.get(), *h_scores = hs.get();
     size_type written = 0;
     for (size_type off = 0; off < total; off += window) {
       const size_type c = export_batch(window, off, d_keys, d_vals, d_scores, stream);
@@ -959,12 +992,6 @@ class HashTable : public HashTableBase<K, V, S> {
       HKV_HIP_CHECK(hipStreamSynchronize(stream));
       written += file->write(c, dim(), h_keys, h_vals, h_scores);
     }
-    HKV_HIP_CHECK(hipFree(d_keys));
-    HKV_HIP_CHECK(hipFree(d_vals));
-    HKV_HIP_CHECK(hipFree(d_scores));
-    HKV_HIP_CHECK(hipHostFree(h_keys));
-    HKV_HIP_CHECK(hipHostFree(h_vals));
-    HKV_HIP_CHECK(hipHostFree(h_scores));
     return written;
   }
 
@@ -974,18 +1001,13 @@ class HashTable : public HashTableBase<K, V, S> {
     MERLIN_CHECK(max_workspace_size >= tuple_size,
                  "[HierarchicalKV] max_workspace_size is smaller than a single `key + score + value` tuple! Please set a larger value!");
     const size_type window = std::max<size_type>(max_workspace_size / tuple_size, 1);
-    K* d_keys = nullptr;
-    V* d_vals = nullptr;
-    S* d_scores = nullptr;
-    K* h_keys = nullptr;
-    V* h_vals = nullptr;
-    S* h_scores = nullptr;
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_keys), window * sizeof(K)));
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_vals), window * sizeof(V) * dim()));
-    HKV_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&d_scores), window * sizeof(S)));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_keys), window * sizeof(K)));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_vals), window * sizeof(V) * dim()));
-    HKV_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&h_scores), window * sizeof(S)));
+    /* released on every way out, also when export_batch or the file throws */
+    detail::StageBuffer<K> dk(window, false), hk(window, true);
+    detail::StageBuffer<V> dv(window * dim(), false), hv(window * dim(), true);
+    detail::StageBuffer<S> ds(window, false), hs(window, true);
+    K *d_keys = dk.get(), *h_keys = hk.get();
+    V *d_vals = dv.get(), *h_vals = hv.get();
+    S *d_scores = ds.get(), *h_scores = hs.get();
     size_type loaded = 0;
     while (true) {
       const size_type c = file->read(window, dim(), h_keys, h_vals, h_scores);
@@ -997,12 +1019,6 @@ class HashTable : public HashTableBase<K, V, S> {
       HKV_HIP_CHECK(hipStreamSynchronize(stream));
       loaded += c;
     }
-    HKV_HIP_CHECK(hipFree(d_keys));
-    HKV_HIP_CHECK(hipFree(d_vals));
-    HKV_HIP_CHECK(hipFree(d_scores));
-    HKV_HIP_CHECK(hipHostFree(h_keys));
-    HKV_HIP_CHECK(hipHostFree(h_vals));
-    HKV_HIP_CHECK(hipHostFree(h_scores));
     return loaded;
   }
 

@@ -328,7 +328,7 @@ uint64_t hkvo_size(const hkvo_table* t) {
 static inline uint64_t now_ns(const hkvo_table* t, uint64_t i) {
   if (t->clock_mode == 1) return t->clock_base + (i << 20);
   struct timespec ts;
-  clock_gettime(CLOCK_MONOTONIC, &ts);
+  clock_gettime(CLOCK_REALTIME, &ts); /* %globaltimer counts from the Unix epoch */
   return (uint64_t)ts.tv_sec * UINT64_C(1000000000) + (uint64_t)ts.tv_nsec;
 }
 

@@ -254,29 +254,20 @@ def test_eviction_quality_and_consistency_at_full_load(oracle):
     rng = np.random.default_rng(42)
     keys = np.arange(1, total + 1, dtype=np.uint64)
     scores = (rng.integers(0, 1 << 63, total, dtype=np.uint64) >> np.uint64(1)) | np.uint64(1)
-    # Which keys survive depends on the order in which the keys of a batch are handled, and that
-    # order changes from run to run on a GPU: over 40 runs of this protocol the kernel measured
-    # 0.9951 to 0.9956 (the host oracle over random orders of the batches: 0.9952 to 0.9956).
-    # The reference's bound of 0.995 is held against the mean of three runs, which a chance
-    # outcome of one run does not move across it.
-    qualities = []
-    for run in range(3):
-        t = HashTable()
-        t.init(dual_options(cap, dim))
-        for lo in range(0, total, cap):
-            k = keys[lo:lo + cap]
-            t.insert_or_assign(cap, dev(k), dev(w.values_from_keys(k, dim)), dev(scores[lo:lo + cap]))
-        ek, ev, es = export_table(t, dim * 4)
-        assert len(ek) == t.size() and len(ek) > 0.99 * cap
-        assert len(np.unique(ek)) == len(ek), "a key sits in both of its buckets"
-        ideal = set(keys[np.argsort(scores)[::-1][:len(ek)]].tolist())
-        qualities.append(sum(1 for k in ek.tolist() if k in ideal) / len(ek))
-        if run < 2:
-            t.close()
-    print("dual-bucket eviction quality " + ", ".join(f"{q:.4f}" for q in qualities)
-          + f", load factor {len(ek) / cap:.4f}")
-    assert min(qualities) >= 0.9945
-    assert sum(qualities) / len(qualities) >= 0.995
+    # one run, held to the reference's bound as the reference holds it (which keys survive depends
+    # on the order in which the hardware takes the keys of a batch: 0.9951 to 0.9956 over 40 runs)
+    t = HashTable()
+    t.init(dual_options(cap, dim))
+    for lo in range(0, total, cap):
+        k = keys[lo:lo + cap]
+        t.insert_or_assign(cap, dev(k), dev(w.values_from_keys(k, dim)), dev(scores[lo:lo + cap]))
+    ek, ev, es = export_table(t, dim * 4)
+    assert len(ek) == t.size() and len(ek) > 0.99 * cap
+    assert len(np.unique(ek)) == len(ek), "a key sits in both of its buckets"
+    ideal = set(keys[np.argsort(scores)[::-1][:len(ek)]].tolist())
+    quality = sum(1 for k in ek.tolist() if k in ideal) / len(ek)
+    print(f"dual-bucket eviction quality {quality:.4f}, load factor {len(ek) / cap:.4f}")
+    assert quality >= 0.995
     # residents carry their own score and row, and find sees exactly the exported set
     assert np.array_equal(es, scores[ek.astype(np.int64) - 1])
     assert np.array_equal(ev, bytes_of(w.values_from_keys(ek, dim)))

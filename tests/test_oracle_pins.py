@@ -673,6 +673,98 @@ def test_find_and_update_touches_scores(oracle):
     t.close()
 
 
+def test_find_or_insert_pointer_truth_table(oracle):
+    # find_or_insert_ptr_kernel_lock_key (find_ptr_or_insert.cuh:27-246), one full bucket, Customized:
+    #   reserved key     -> value pointer and found flag left as they were (:66-70)
+    #   present          -> found, its own slot, score := input (update_with_digest, :108-113)
+    #   absent, score > min          -> not found, takes the slot of the minimum score (:195-224)
+    #   absent, score == min or less -> refused: null pointer, not found (:196-199, "<=")
+    untouched_slot, untouched_flag = 0x5555555555555555, 2   # what the binding pre-fills
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(41, 0, 128)
+    sc = np.arange(1000, 1128, dtype=np.uint64)
+    t.insert_or_assign(keys, vals_of(keys, 1), sc)
+    where, f, _ = t.find_slot(keys)
+    assert f.all() and sorted(where.tolist()) == list(range(128))
+    fresh = w.unique_keys(42, 0, 3)
+    batch = np.concatenate([np.array([M64, M64 - 1, M64 - 2, M64 - 3], np.uint64),  # the four reserved keys
+                            keys[5:7],            # present
+                            fresh])               # absent: above the minimum, equal to it, below it
+    # key 0 holds the minimum (1000); after fresh[0] has taken its slot with 5000 the minimum is 1001
+    bsc = np.array([1, 1, 1, 1, 7005, 7006, 5000, 1001, 3], np.uint64)
+    slots, founds = t.find_or_insert_slot(batch, bsc)
+    assert (slots[:4] == np.uint64(untouched_slot)).all() and (founds[:4] == untouched_flag).all()
+    assert founds[4:6].tolist() == [1, 1] and slots[4:6].tolist() == where[5:7].tolist()
+    assert founds[6] == 0 and slots[6] == where[0]          # victim = the minimum score's slot
+    assert founds[7] == 0 and slots[7] == np.uint64(M64)    # equal to the minimum: refused
+    assert founds[8] == 0 and slots[8] == np.uint64(M64)    # below the minimum: refused
+    _, f, s2 = t.find(np.concatenate([keys[:1], keys[5:7], fresh]))
+    assert f.tolist() == [False, True, True, True, False, False]
+    assert s2[1:4].tolist() == [7005, 7006, 5000]
+    assert t.size() == 128
+    t.close()
+
+
+def test_find_or_insert_pointer_never_takes_locked_or_empty_slots(oracle):
+    # the victim scan of the lock-key kernels skips slots whose key word is LOCKED or EMPTY
+    # (find_ptr_or_insert.cuh:170-180): with the two lowest scores locked, the third goes
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(43, 0, 128)
+    sc = np.arange(100, 228, dtype=np.uint64)
+    t.insert_or_assign(keys, vals_of(keys, 1), sc)
+    where, _, _ = t.find_slot(keys)
+    locked, ok = t.lock_keys(keys[:2], sc[:2].copy())
+    assert ok.all() and locked.tolist() == where[:2].tolist()
+    newk = w.unique_keys(44, 0, 1)
+    slots, founds = t.find_or_insert_slot(newk, np.array([900], np.uint64))
+    assert founds[0] == 0 and slots[0] == where[2]
+    # a key that cannot beat the lowest visible score (102 left; 103 is next) is refused, not parked
+    # on a locked slot
+    again = w.unique_keys(45, 0, 1)
+    slots2, founds2 = t.find_or_insert_slot(again, np.array([103], np.uint64))
+    assert founds2[0] == 0 and slots2[0] == np.uint64(M64)
+    assert t.unlock_keys(locked, keys[:2]).all()
+    _, f, _ = t.find(np.concatenate([keys[:3], newk, again]))
+    assert f.tolist() == [True, True, False, True, False]
+    # free slots come before victims: erase one key, the next absent key lands in that slot
+    t.erase(keys[10:11])
+    third = w.unique_keys(46, 0, 1)
+    slots3, founds3 = t.find_or_insert_slot(third, np.array([1], np.uint64))  # the lowest score of all
+    assert founds3[0] == 0 and slots3[0] == where[10]
+    t.close()
+
+
+def test_find_pointer_truth_table(oracle):
+    # tlp_lookup_ptr_kernel_with_filter / lookup_ptr_kernel (lookup_ptr.cuh:25-152, 379-435):
+    # present -> its slot, found, its score; absent -> null, not found, score output untouched;
+    # reserved keys and keys held by lock_keys are not found; the table does not change
+    o = default_options(init_capacity=1024, max_capacity=1024, dim=2, evict_strategy=EvictStrategy.kCustomized)
+    t = oracle.OracleTable(o)
+    keys = w.unique_keys(47, 0, 300)
+    sc = np.arange(2000, 2300, dtype=np.uint64)
+    t.insert_or_assign(keys, vals_of(keys, 2), sc)
+    q = np.concatenate([keys[:40], w.unique_keys(48, 0, 8), np.array([M64, M64 - 1, M64 - 2, M64 - 3], np.uint64)])
+    slots, f, s = t.find_slot(q)
+    assert f.tolist() == [True] * 40 + [False] * 12
+    assert (slots[40:] == np.uint64(M64)).all() and (s[40:] == 0).all()
+    assert (s[:40] == sc[:40]).all()
+    # the slot is where the key's row lives: bucket of the key, and distinct per key
+    nb = 1024 // 128
+    assert [int(x) // 128 for x in slots[:40]] == [oracle.locate(int(k), nb)[0] for k in keys[:40]]
+    assert len(set(slots[:40].tolist())) == 40
+    locked, ok = t.lock_keys(keys[:3], sc[:3].copy())
+    assert ok.all()
+    _, f2, _ = t.find_slot(keys[:5])
+    assert f2.tolist() == [False, False, False, True, True]
+    assert t.unlock_keys(locked, keys[:3]).all()
+    slots3, f3, s3 = t.find_slot(keys[:5])
+    assert f3.all() and slots3.tolist() == slots[:5].tolist() and (s3 == sc[:5]).all()
+    assert t.size() == 300
+    t.close()
+
+
 # ---- dual-bucket mode (TableMode::kMemory) -------------------------------------------------
 
 def dual_options(capacity, dim=4, strategy=EvictStrategy.kCustomized, **kw):
