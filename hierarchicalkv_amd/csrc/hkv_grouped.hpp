@@ -9,34 +9,30 @@
  * group_lock.cuh:43-56), so the only conflicts are between keys of the same
  * batch, and only between keys that are absent: a key that is present owns its
  * slot (keys of a batch are unique), absent keys of one bucket compete for its
- * free slots and victims.  Hence two phases, each a kernel:
+ * free slots and victims.  Hence two phases, each one kernel:
  *
  *   upsert_hits_kernel   every key is probed as in find.  A key that is present
- *                        gets its new score and row at once, without a lock;
- *                        an absent key goes to a list.
- *   grouped_miss_kernel  the absent keys, partitioned by bucket.  Each bucket
- *                        is owned by one 8-lane tile, which reads the digest
- *                        line once and the 128 scores once, keeps both in
- *                        registers, places its keys one after the other there
- *                        (free slot, else minimum score, ties to the lowest
- *                        slot), and writes back whole 64-byte pieces.
+ *                        gets its new score and row at once, without a lock.
+ *                        An absent key is hung into the list of its bucket:
+ *                        one exchange on the bucket's head word (a 4-byte-per-
+ *                        bucket array that stays in the last-level cache), and
+ *                        the previous head goes into next[i], which is written
+ *                        for all 64 keys of the wavefront in one coalesced line.
+ *   chained_miss_kernel  one lane per bucket reads (and clears) the head word
+ *                        and walks the list; each bucket that has keys is then
+ *                        owned by one 8-lane tile, which reads the digest line
+ *                        once and the 128 scores once, places its keys one
+ *                        after the other there (free slot, else minimum score,
+ *                        ties to the lowest slot) and writes the digest line
+ *                        back whole.
  *
  * The serial order this amounts to - all present keys, then the absent ones
  * bucket by bucket - is one of the orders the slot-lock kernel could have
- * produced.  What is saved: on this memory system an atomic on a random line
- * costs about as much as moving two and a half full 128-byte lines and a
- * scattered 8-byte store about one and a half, and the slot-lock protocol
- * spends a CAS, an unlock store and two small loads per key on top of the
- * score and digest stores; a bucket that takes several keys of a batch is
- * scanned once instead of once per key.
- *
- * Partition of the absent keys: bins are aligned runs of 2^s buckets.
- *   bin_hist_kernel      per-block histogram of the keys' bins (LDS)
- *   bin_colscan_kernel   per bin: running sum over the blocks
- *   bin_scatter_kernel   per block: scan of the bin totals, then every key's
- *                        index goes to its place in `order`
- * grouped_miss_kernel then runs one wavefront per bin: counting sort of the
- * bin's keys by bucket in LDS, and its 8 tiles take buckets from a work list.
+ * produced.  What is saved: the slot-lock protocol spends a compare-and-swap
+ * and an unlock store per present key and an exchange and a score re-read per
+ * absent key, each of them a small access that the memory side serves as a
+ * read-modify-write of a 64-byte piece, and a bucket that takes several keys of
+ * a batch is scanned once instead of once per key.
  */
 #ifndef HKV_GROUPED_HPP_
 #define HKV_GROUPED_HPP_
@@ -45,144 +41,9 @@
 
 namespace hkv {
 
-constexpr int kBinThreads = 1024;   /* histogram / scatter workgroup */
-constexpr int kMaxBins = 8192;      /* LDS histogram: 32 KB */
-constexpr int kGrpThreads = 64;     /* grouped_miss_kernel workgroup: one wavefront, no barriers to wait at */
-constexpr int kGrpChunk = 256;      /* keys of a bin staged per pass */
-constexpr int kGrpStage = kGrpChunk / kGrpThreads; /* keys a thread stages */
-constexpr int kGrpMaxBpbShift = 10; /* at most 1024 buckets per bin */
-constexpr int kGrpMaxBpb = 1 << kGrpMaxBpbShift;
-constexpr int kGrpKeys = 2;         /* keys of one bucket handled per pass of a tile */
-
-struct BinArgs {
-  const uint64_t* keys;
-  const uint8_t* absent; /* per key of the batch: 1 = goes to the second phase */
-  uint64_t n;
-  uint32_t bpb_shift; /* buckets per bin = 1 << bpb_shift */
-  uint32_t nbins;
-  uint32_t blocks;    /* histogram blocks */
-  uint32_t slice;     /* keys per histogram block */
-  uint32_t* hist;     /* [blocks][nbins] */
-  uint32_t* total;    /* [nbins] */
-  uint32_t* bin_start; /* [nbins + 1] */
-  uint32_t* order;    /* [n] key indices grouped by bin */
-};
-
-/* bin of key i of the batch (never a reserved key: the probe filtered those) */
-__device__ __forceinline__ uint32_t bin_of(const View& v, const BinArgs& b, uint64_t key) {
-  uint32_t bkt, start, digest;
-  locate(v, key, bkt, start, digest);
-  return bkt >> b.bpb_shift;
-}
-
-constexpr int kBinUnroll = 8; /* keys a thread has in flight */
-
-__global__ void __launch_bounds__(kBinThreads)
-bin_hist_kernel(View v, BinArgs b) {
-  extern __shared__ uint32_t s_hist[];
-  for (uint32_t t = threadIdx.x; t < b.nbins; t += kBinThreads) s_hist[t] = 0;
-  __syncthreads();
-  const uint64_t lo = (uint64_t)blockIdx.x * b.slice;
-  const uint64_t hi = lo + b.slice < b.n ? lo + b.slice : b.n;
-  for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += (uint64_t)kBinThreads * kBinUnroll) {
-    uint64_t key[kBinUnroll];
-    uint8_t take[kBinUnroll];
-#pragma unroll
-    for (int e = 0; e < kBinUnroll; e++) {
-      const uint64_t i = i0 + (uint64_t)e * kBinThreads;
-      take[e] = 0;
-      key[e] = 0;
-      if (i < hi) {
-        take[e] = b.absent[i];
-        key[e] = b.keys[i];
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < kBinUnroll; e++)
-      if (take[e]) atomicAdd(&s_hist[bin_of(v, b, key[e])], 1u);
-  }
-  __syncthreads();
-  uint32_t* out = b.hist + (uint64_t)blockIdx.x * b.nbins;
-  for (uint32_t t = threadIdx.x; t < b.nbins; t += kBinThreads) out[t] = s_hist[t];
-}
-
-/* hist[g][bin] becomes the number of keys of that bin in blocks before g.
- * The column is read kColBatch entries at a time, loads before stores. */
-constexpr int kMaxHistBlocks = 128;
-constexpr int kColBatch = 32;
-__global__ void __launch_bounds__(256)
-bin_colscan_kernel(BinArgs b) {
-  const uint32_t bin = blockIdx.x * 256 + threadIdx.x;
-  if (bin >= b.nbins) return;
-  uint32_t run = 0;
-  for (uint32_t g0 = 0; g0 < b.blocks; g0 += kColBatch) {
-    uint32_t c[kColBatch];
-#pragma unroll
-    for (int g = 0; g < kColBatch; g++)
-      c[g] = g0 + g < b.blocks ? b.hist[(uint64_t)(g0 + g) * b.nbins + bin] : 0u;
-#pragma unroll
-    for (int g = 0; g < kColBatch; g++) {
-      if (g0 + g < b.blocks) b.hist[(uint64_t)(g0 + g) * b.nbins + bin] = run;
-      run += c[g];
-    }
-  }
-  b.total[bin] = run;
-}
-
-__global__ void __launch_bounds__(kBinThreads)
-bin_scatter_kernel(View v, BinArgs b) {
-  extern __shared__ uint32_t s_cursor[]; /* [nbins] */
-  __shared__ uint32_t s_wave[kBinThreads / kWave];
-  /* exclusive scan of total[]: thread t owns the bins [t * per, t * per + per) */
-  const uint32_t per = (b.nbins + kBinThreads - 1) / kBinThreads;
-  const uint32_t b0 = threadIdx.x * per;
-  uint32_t sum = 0;
-  for (uint32_t e = 0; e < per; e++)
-    if (b0 + e < b.nbins) sum += b.total[b0 + e];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  uint32_t inc = sum;
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const uint32_t y = __shfl_up(inc, off);
-    if (lane >= off) inc += y;
-  }
-  if (lane == kWave - 1) s_wave[wave] = inc;
-  __syncthreads();
-  uint32_t run = inc - sum;
-  for (int w = 0; w < wave; w++) run += s_wave[w];
-  const uint32_t* rel = b.hist + (uint64_t)blockIdx.x * b.nbins;
-  for (uint32_t e = 0; e < per; e++) {
-    const uint32_t bin = b0 + e;
-    if (bin < b.nbins) {
-      if (blockIdx.x == 0) b.bin_start[bin] = run;
-      s_cursor[bin] = run + rel[bin];
-      run += b.total[bin];
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x == kBinThreads - 1) b.bin_start[b.nbins] = run;
-  __syncthreads();
-  const uint64_t lo = (uint64_t)blockIdx.x * b.slice;
-  const uint64_t hi = lo + b.slice < b.n ? lo + b.slice : b.n;
-  for (uint64_t i0 = lo + threadIdx.x; i0 < hi; i0 += (uint64_t)kBinThreads * kBinUnroll) {
-    uint64_t key[kBinUnroll];
-    uint8_t take[kBinUnroll];
-#pragma unroll
-    for (int e = 0; e < kBinUnroll; e++) {
-      const uint64_t i = i0 + (uint64_t)e * kBinThreads;
-      take[e] = 0;
-      key[e] = 0;
-      if (i < hi) {
-        take[e] = b.absent[i];
-        key[e] = b.keys[i];
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < kBinUnroll; e++)
-      if (take[e])
-        b.order[atomicAdd(&s_cursor[bin_of(v, b, key[e])], 1u)] =
-            (uint32_t)(i0 + (uint64_t)e * kBinThreads);
-  }
-}
+constexpr int kGrpKeys = 2;       /* keys of one bucket handled per pass of a tile */
+constexpr int kChainStage = 4;    /* keys of one bucket staged per walk of its list */
+constexpr uint32_t kChainEnd = 0; /* head / next hold key index + 1 */
 
 /* ---- register-resident bucket state ------------------------------------------------ */
 
@@ -228,15 +89,13 @@ __device__ __forceinline__ bool final_score(const UpsertArgs& a, bool new_insert
   return true;
 }
 
-struct GroupArgs {
-  const uint32_t* order;
-  const uint32_t* bin_start;
-  uint32_t bpb_shift;
+/* The lists of absent keys, one per bucket: head[bucket] is the batch index + 1 of the key
+ * hung in last (0: none), next[i] the index + 1 of the key hung in before key i.  head[] is
+ * all zero between calls: the second phase clears what it reads. */
+struct ChainArgs {
+  uint32_t* head;       /* [buckets_num] */
+  uint32_t* next;       /* [n] */
   uint32_t locked_rule; /* refuse when score <= min, not < (upsert.cuh:1478-1524) */
-};
-
-struct HitArgs {
-  uint8_t* absent; /* [n] out: 1 = the key goes to the second phase */
 };
 
 /*
@@ -244,13 +103,13 @@ struct HitArgs {
  *   present  new score (update_with_digest with the slot's old score where the
  *            strategy needs it) and the row traffic of the operation, the whole
  *            wavefront moving the rows of its keys, VEC bytes per lane;
- *   absent   flagged for the second phase.
+ *   absent   hung into the list of its bucket for the second phase.
  * accum_or_assign drops the keys whose flag disagrees with what was found
  * (accum_or_assign.cuh:139-156).
  */
 template <int OP, int VEC>
 __global__ void __launch_bounds__(kWave)
-upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
+upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
   const int lane = threadIdx.x;
@@ -259,7 +118,7 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
   stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  probe_wave<false, true>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
 
   const bool valid = (s_meta[lane].info & 0x100u) != 0;
@@ -271,7 +130,13 @@ upsert_hits_kernel(View v, UpsertArgs a, HitArgs h) {
     if (hit && !is_accum) hit = false;
     if (miss && is_accum) miss = false;
   }
-  if (i < a.n) h.absent[i] = miss;
+  if (i < a.n) {
+    uint32_t before = kChainEnd;
+    if (miss)
+      before = __hip_atomic_exchange(h.head + s_meta[lane].bkt, (uint32_t)i + 1, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+    h.next[i] = before;
+  }
   if (hit) {
     const uint64_t desired = desired_when_missed(a, in_score, i);
     const bool needs_old = a.strategy == HKV_LFU || a.strategy == HKV_EPOCH_LFU;
@@ -441,11 +306,10 @@ __device__ __forceinline__ Top2 tile_top2(const View& v, uint64_t bslot, int j, 
  */
 template <int OP, int VEC, int UPL>
 __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
-                                             const GroupArgs& g, uint32_t bkt, uint32_t sb,
+                                             const ChainArgs& g, uint32_t bkt, uint32_t sb,
                                              uint32_t se, const uint64_t* s_key,
                                              const uint32_t* s_idx, const uint32_t* s_info,
-                                             uint32_t units, int lane, uint4 dg,
-                                             unsigned long long* acc) {
+                                             uint32_t units, int lane, uint4 dg) {
   static_assert(kGrpKeys == 2, "tile_top2 serves a pass of two keys");
   const int j = lane & (kTile - 1);
   const int tile = lane >> 3;
@@ -746,143 +610,91 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
   if (size_delta && j == 0) atomicAdd(v.sizes + bkt, size_delta);
 }
 
-#ifndef HKV_GROUPED_WAVES_PER_EU
-#define HKV_GROUPED_WAVES_PER_EU 3
-#endif
+/*
+ * Phase 2.  One wavefront per 64 consecutive buckets.
+ *   walk   lane L reads the head word of bucket 64 w + L, clears it, and follows the list:
+ *          up to kChainStage keys go to the lane's part of the LDS staging arrays (key,
+ *          batch index, digest and start slot); the 64 lists are walked side by side, one
+ *          memory round trip per step for the whole wavefront;
+ *   place  the buckets that have keys are dealt out to the 8 tiles in turn; a tile works
+ *          through its buckets with group_bucket, the digest line of its next bucket being
+ *          asked for before the current one is worked on.
+ * A list longer than kChainStage is finished in further rounds of walk and place.
+ */
 template <int OP, int VEC, int UPL>
-__global__ void __launch_bounds__(kGrpThreads)
-__attribute__((amdgpu_waves_per_eu(HKV_GROUPED_WAVES_PER_EU)))
-grouped_miss_kernel(View v, UpsertArgs a, GroupArgs g) {
-  __shared__ uint64_t s_key[kGrpChunk];
-  __shared__ uint32_t s_idx[kGrpChunk];
-  __shared__ uint32_t s_info[kGrpChunk]; /* digest | start << 8 | bucket inside the bin << 16 */
-  /* sized by the launch: (bpb + 1) segment starts, bpb cursors, bpb work items */
-  extern __shared__ uint32_t s_dyn[];
-  __shared__ uint32_t s_wsum[kGrpThreads / kWave];
-  __shared__ uint32_t s_nwork, s_next;
-  unsigned long long* const s_acc = nullptr;
+__global__ void __launch_bounds__(kWave)
+__attribute__((amdgpu_waves_per_eu(3)))
+chained_miss_kernel(View v, UpsertArgs a, ChainArgs g) {
+  __shared__ uint64_t s_key[kWave * kChainStage];
+  __shared__ uint32_t s_idx[kWave * kChainStage];
+  __shared__ uint32_t s_info[kWave * kChainStage]; /* digest | start << 8 */
+  __shared__ uint8_t s_count[kWave];
+  __shared__ uint8_t s_list[kWave]; /* lanes (buckets) that have keys in this round */
 
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const uint32_t bin = blockIdx.x;
-  const uint32_t bpb = 1u << g.bpb_shift;
-  uint32_t* const s_seg = s_dyn;
-  uint32_t* const s_cur = s_dyn + bpb + 1;
-  uint16_t* const s_work = reinterpret_cast<uint16_t*>(s_dyn + 2 * bpb + 1);
-  const uint32_t first = g.bin_start[bin], last = g.bin_start[bin + 1];
+  const int lane = threadIdx.x;
+  const int tile = lane >> 3, j = lane & (kTile - 1);
+  const uint64_t b0 = (uint64_t)blockIdx.x * kWave;
+  const uint64_t my_bkt = b0 + lane;
   const uint32_t units = v.value_bytes / VEC;
 
-  for (uint32_t c0 = first; c0 < last; c0 += kGrpChunk) {
-    const uint32_t cn = last - c0 < (uint32_t)kGrpChunk ? last - c0 : (uint32_t)kGrpChunk;
-    for (uint32_t t = tid; t <= bpb; t += kGrpThreads) s_seg[t] = 0;
-    if (tid == 0) {
-      s_nwork = 0;
-      s_next = 0;
-    }
-    __syncthreads();
-
-    /* ---- stage: kGrpStage keys per thread, counted by bucket ------------------------------------- */
-    uint64_t mk[kGrpStage];
-    uint32_t mi[kGrpStage], minfo[kGrpStage];
-    bool have[kGrpStage];
-#pragma unroll
-    for (int e = 0; e < kGrpStage; e++) {
-      const uint32_t p = tid + e * kGrpThreads;
-      have[e] = p < cn;
-      mk[e] = 0;
-      mi[e] = 0;
-      minfo[e] = 0;
-      if (have[e]) {
-        mi[e] = g.order[c0 + p];
-        mk[e] = a.keys[mi[e]];
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < kGrpStage; e++) {
-      if (have[e]) {
-        uint32_t bkt, start, digest;
-        locate(v, mk[e], bkt, start, digest);
-        const uint32_t lb = bkt - (bin << g.bpb_shift);
-        minfo[e] = digest | (start << 8) | (lb << 16);
-        atomicAdd(&s_seg[lb], 1u);
-      }
-    }
-    __syncthreads();
-
-    /* ---- exclusive scan of the counts; list of the buckets that have keys ---------------------------- */
-    {
-      const uint32_t per = (bpb + kGrpThreads - 1) / kGrpThreads;
-      const uint32_t t0 = tid * per;
-      uint32_t sum = 0;
-      for (uint32_t e = 0; e < per; e++)
-        if (t0 + e < bpb) sum += s_seg[t0 + e];
-      uint32_t inc = sum;
-#pragma unroll
-      for (int off = 1; off < kWave; off <<= 1) {
-        const uint32_t y = __shfl_up(inc, off);
-        if (lane >= off) inc += y;
-      }
-      if (lane == kWave - 1) s_wsum[tid >> 6] = inc;
+  uint32_t h = kChainEnd;
+  if (my_bkt < v.buckets_num) {
+    h = g.head[my_bkt];
+    if (h != kChainEnd) g.head[my_bkt] = kChainEnd;
+  }
+  bool again = false;
+  while (__ballot(h != kChainEnd)) {
+    /* a further round re-reads digest lines and scores that the round before has written */
+    const bool again_round = again;
+    if (again) {
+      wait_stores();
       __syncthreads();
-      uint32_t run = inc - sum;
-      for (int w = 0; w < (tid >> 6); w++) run += s_wsum[w];
-      for (uint32_t e = 0; e < per; e++) {
-        const uint32_t t = t0 + e;
-        if (t < bpb) {
-          const uint32_t c = s_seg[t];
-          s_seg[t] = run;
-          s_cur[t] = run;
-          if (c) s_work[atomicAdd(&s_nwork, 1u)] = (uint16_t)t;
-          run += c;
-        }
-      }
-      if (tid == kGrpThreads - 1) s_seg[bpb] = run;
     }
-    __syncthreads();
-
-    /* ---- place ------------------------------------------------------------------------------------------ */
-#pragma unroll
-    for (int e = 0; e < kGrpStage; e++) {
-      if (have[e]) {
-        const uint32_t p = atomicAdd(&s_cur[minfo[e] >> 16], 1u);
-        s_key[p] = mk[e];
-        s_idx[p] = mi[e];
-        s_info[p] = minfo[e];
+    again = true;
+    /* ---- walk -------------------------------------------------------------------------------- */
+    int cnt = 0;
+    while (__ballot(h != kChainEnd && cnt < kChainStage)) {
+      if (h != kChainEnd && cnt < kChainStage) {
+        const uint32_t i = h - 1;
+        const uint64_t key = a.keys[i];
+        h = g.next[i];
+        uint32_t bkt, start, digest;
+        locate(v, key, bkt, start, digest);
+        const int at = lane * kChainStage + cnt;
+        s_key[at] = key;
+        s_idx[at] = i;
+        s_info[at] = digest | (start << 8);
+        cnt++;
       }
     }
+    s_count[lane] = (uint8_t)cnt;
+    const unsigned long long have = __ballot(cnt > 0);
+    if (cnt > 0) s_list[__popcll(have & ((1ull << lane) - 1))] = (uint8_t)lane;
     __syncthreads();
 
-    /* ---- tiles take buckets from the work list; the digest line of the next
-     * bucket is asked for before the current one is worked on ---------------------------------------------- */
-    const uint32_t nwork = s_nwork;
-    const int tile_base = lane & ~(kTile - 1);
-    const int j = lane & (kTile - 1);
-    const uint32_t bkt0 = bin << g.bpb_shift;
-    auto take = [&]() {
-      uint32_t w = 0;
-      if (j == 0) w = atomicAdd(&s_next, 1u);
-      return (uint32_t)__shfl(w, tile_base);
+    /* ---- place -------------------------------------------------------------------------------- */
+    const int nwork = __popcll(have);
+    /* a round after the first reads lines that this wavefront has written: past the caches */
+    const bool reread = again_round;
+    auto digests_of = [&](int w) {
+      const uint64_t bkt = b0 + s_list[w];
+      if (reread) return ld_digests16(v, (uint32_t)bkt, j);
+      return *reinterpret_cast<const uint4*>(v.digests + bkt * kBucketSize + j * 16);
     };
-    auto digests_of = [&](uint32_t w) {
-      return *reinterpret_cast<const uint4*>(v.digests + (uint64_t)(bkt0 + s_work[w]) * kBucketSize +
-                                             j * 16);
-    };
-    /* the digest line of the next bucket is asked for before the current one is
-     * worked on */
-    uint32_t w0 = take();
+    int w0 = tile;
     uint4 dg0 = make_uint4(0, 0, 0, 0);
     if (w0 < nwork) dg0 = digests_of(w0);
     while (w0 < nwork) {
-      const uint32_t w1 = take();
+      const int w1 = w0 + kTilesPerWave;
       uint4 dg1 = make_uint4(0, 0, 0, 0);
       if (w1 < nwork) dg1 = digests_of(w1);
-      const uint32_t lb = s_work[w0];
-      group_bucket<OP, VEC, UPL>(v, a, g, bkt0 + lb, s_seg[lb], s_seg[lb + 1], s_key, s_idx, s_info,
-                                 units, lane, dg0, s_acc);
+      const uint32_t lb = s_list[w0];
+      const uint32_t sb = lb * kChainStage;
+      group_bucket<OP, VEC, UPL>(v, a, g, (uint32_t)(b0 + lb), sb, sb + s_count[lb], s_key, s_idx,
+                                 s_info, units, lane, dg0);
       w0 = w1;
       dg0 = dg1;
     }
-    __syncthreads();
   }
 }
 

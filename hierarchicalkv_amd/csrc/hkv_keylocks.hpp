@@ -57,7 +57,7 @@ touch_kernel(View v, TouchArgs t) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint64_t key = stage_keys(v, t.keys, t.n, i, s_meta, s_slot, lane);
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  probe_wave<false, false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   const int64_t slot = s_slot[lane];
   bool ok = false;

@@ -51,7 +51,7 @@ struct FindArgs {
  *     another tile's lock, so s_unsure[k] is raised and the writer settles the
  *     question with a second, coherent probe of its own (tile_reprobe).
  */
-template <bool WRITER>
+template <bool WRITER, bool TWO_STEP>
 __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
                                            int64_t* s_slot,
                                            uint16_t (*s_em)[kTile],
@@ -69,11 +69,14 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     if (m.info & 0x100u)
       dg[r] = *reinterpret_cast<const uint4*>(v.digests + (uint64_t)m.bkt * kBucketSize + j * 16);
   }
-  /* Candidates are verified in two steps.  An 8-byte key load costs a whole 128-byte line of
-   * memory traffic, a key that is present has one true candidate, and a false 8-bit match
-   * turns up in every second bucket: so step 1 fetches only the candidates of the first
-   * lane of the tile that has any (a lane's 16 slots share one key line), and the other
-   * lanes' candidates are fetched in step 2 only for the keys step 1 did not find. */
+  /* TWO_STEP: candidates are verified in two steps.  An 8-byte key load costs a whole
+   * 128-byte line of memory traffic, a key that is present has one true candidate, and a
+   * false 8-bit match turns up in every second bucket: so step 1 fetches only the
+   * candidates of the first lane of the tile that has any (a lane's 16 slots share one key
+   * line), and the other lanes' candidates are fetched in step 2 only for the keys step 1
+   * did not find: 1.27 key lines per key that is present instead of 1.44.  It pays where the
+   * kernel is bound by bytes (find with its rows); a kernel that moves little besides the
+   * probe is bound by its dependent round trips and takes all candidates at once. */
   uint32_t cm[kTile];    /* this lane's digest matches, bw order */
   uint32_t later[kTile]; /* lanes of the tile whose candidates wait for step 2 */
   uint64_t k0[kTile], k1[kTile];
@@ -85,7 +88,7 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
     if (WRITER && s_em != nullptr)
       s_em[tile * kTile + r][j] =
           (uint16_t)(valid ? match16_natural(dg[r], v.empty_digest * 0x01010101u) : 0u);
-    const uint32_t lanes = tile_ballot(cm[r] != 0, tile);
+    const uint32_t lanes = TWO_STEP ? tile_ballot(cm[r] != 0, tile) : 0u;
     later[r] = lanes & (lanes - 1);
     const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
     k0[r] = v.empty_key;
@@ -128,10 +131,12 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
   for (int r = 0; r < kTile; r++) {
     const bool mine = cm[r] && !((later[r] >> j) & 1u);
     const bool hit = mine && check(r);
-    if (tile_ballot(hit, tile)) later[r] = 0;
-    more |= later[r] != 0;
+    if (TWO_STEP) {
+      if (tile_ballot(hit, tile)) later[r] = 0;
+      more |= later[r] != 0;
+    }
   }
-  if (__ballot(more)) {
+  if (TWO_STEP && __ballot(more)) {
 #pragma unroll
     for (int r = 0; r < kTile; r++) {
       if ((later[r] >> j) & 1u) {
@@ -146,6 +151,9 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
       if ((later[r] >> j) & 1u) check(r);
   }
 }
+
+/* the writers' probes (upsert and assign families) */
+constexpr bool kTwoStepWriters = false;
 
 /* the 16 digest bytes of lane j of a tile, read past the caches */
 __device__ __forceinline__ uint4 ld_digests16(const View& v, uint32_t bkt, int j) {
@@ -264,12 +272,12 @@ lookup_kernel(View v, FindArgs a) {
   if (DUAL) restage_first_bucket(v, s_meta, lane);
   if (WAVES > 1 && threadIdx.x == 0) s_missed[0] = 0;
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  probe_wave<false, MODE == kLookupValues>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   if (DUAL) {
     restage_second_bucket(v, s_meta, s_slot, lane);
     __syncthreads();
-    probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+    probe_wave<false, MODE == kLookupValues>(v, s_meta, s_slot, nullptr, nullptr, lane);
     __syncthreads();
   }
 

@@ -51,7 +51,7 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint64_t key = stage_keys(v, keys, n, i, s_meta, s_slot, lane);
   __syncthreads();
-  probe_wave<false>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  probe_wave<false, false>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   const int64_t slot = s_slot[lane];
   const int tile_base = lane & ~(kTile - 1), j = lane & (kTile - 1);
@@ -178,6 +178,12 @@ partial_size_kernel(View v, uint32_t n, unsigned long long* out) {
 
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
 __global__ void zero_i32_kernel(int32_t* p) { *p = 0; }
+/* n 32-bit words from p on become zero (n a multiple of 4, p aligned to 16 bytes) */
+__global__ void __launch_bounds__(256)
+zero_words_kernel(uint32_t* p, uint64_t n) {
+  const uint64_t q = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q * 4 < n) reinterpret_cast<uint4*>(p)[q] = make_uint4(0, 0, 0, 0);
+}
 
 /* ---- built-in predicates (hkv_predicate) -------------------------------------- */
 

@@ -166,10 +166,9 @@ struct hkv_table {
   uint64_t epoch;
   Clock clock;
   mutable StreamGroupLock lock;
-  /* bucket-grouped upserts: partition scratch (histograms, bin starts, key
-   * order), grown on demand; only ever used under the inserter role */
-  void* d_scratch;
-  uint64_t scratch_bytes;
+  void* d_scratch;          /* two-phase upserts: list heads per bucket + links per key */
+  uint64_t scratch_buckets; /* bucket count the heads were laid out for */
+  uint64_t scratch_keys;    /* links allocated */
   int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
   bool keys_may_be_locked; /* LOCKED key words may sit in the table (lock_keys, the pointer
@@ -334,37 +333,15 @@ void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   }
 }
 
-/* Geometry of a two-phase upsert, or feasible == false when the batch is
- * better served by the slot-lock kernel. */
-struct GroupPlan {
-  bool feasible;
-  uint32_t bpb_shift, nbins, blocks, slice;
-  uint64_t off_total, off_start, off_order, off_absent, bytes;
-};
-
-GroupPlan plan_grouped(const hkv_table* t, uint64_t n) {
-  GroupPlan p{};
-  const uint64_t buckets = t->view.buckets_num;
+/* Whether a batch goes through the two-phase path (hkv_grouped.hpp). */
+bool two_phase_feasible(const hkv_table* t, uint64_t n) {
   /* the second phase has no locks: it needs the inserter's exclusivity */
-  if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return p;
-  if (t->keys_may_be_locked) return p; /* the second phase does not look at key words */
-  /* bins of about 128 keys if every key of the batch were absent */
-  uint32_t shift = 0;
-  while (shift < (uint32_t)kGrpMaxBpbShift && (n << (shift + 1)) <= 128 * buckets) shift++;
-  p.bpb_shift = shift;
-  p.nbins = (uint32_t)((buckets + (UINT64_C(1) << shift) - 1) >> shift);
-  if (p.nbins > (uint32_t)kMaxBins) return p;
-  if (t->upsert_path == 0 && (n < 32768 || n < 32 * (uint64_t)p.nbins)) return p;
-  p.blocks = (uint32_t)std::min<uint64_t>(kMaxHistBlocks, (n + 8191) / 8192);
-  p.slice = (uint32_t)((n + p.blocks - 1) / p.blocks);
-  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
-  p.off_total = up((uint64_t)p.blocks * p.nbins * 4);
-  p.off_start = p.off_total + up((uint64_t)p.nbins * 4);
-  p.off_order = p.off_start + up(((uint64_t)p.nbins + 1) * 4);
-  p.off_absent = p.off_order + up(n * 4);
-  p.bytes = p.off_absent + up(n);
-  p.feasible = true;
-  return p;
+  if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return false;
+  if (t->keys_may_be_locked) return false; /* the second phase does not look at key words */
+  if (t->upsert_path == 2) return true;
+  /* the second phase visits every bucket's head word: worth it for batches that reach a fair
+   * share of the buckets */
+  return n >= 32768 && n * 8 >= t->view.buckets_num;
 }
 
 template <template <int, int, int> class Launcher, int OP, class... Args>
@@ -385,63 +362,50 @@ void dispatch_vec_upl(int vec, uint32_t value_bytes, Args&&... args) {
 
 template <int OP, int VEC, int UPL>
 struct LaunchHits {
-  static void go(const View& v, const UpsertArgs& a, const HitArgs& h, hipStream_t s) {
-    hipLaunchKernelGGL((upsert_hits_kernel<OP, VEC>), dim3(grid_for(a.n)), dim3(kWave), 0, s, v, a,
-                       h);
+  static void go(const View& v, const UpsertArgs& a, const ChainArgs& c, hipStream_t s) {
+    hipLaunchKernelGGL((upsert_hits_kernel<OP, VEC>), dim3(grid_for(a.n)), dim3(kWave), 0, s, v, a, c);
   }
 };
 template <int OP, int VEC, int UPL>
 struct LaunchMisses {
-  static void go(const View& v, const UpsertArgs& a, const GroupArgs& g, uint32_t nbins,
-                 hipStream_t s) {
-    const size_t bpb = (size_t)1 << g.bpb_shift;
-    const size_t lds = (2 * bpb + 1) * 4 + bpb * 2;
-    hipLaunchKernelGGL((grouped_miss_kernel<OP, VEC, UPL>), dim3(nbins), dim3(kGrpThreads), lds, s, v, a,
-                       g);
+  static void go(const View& v, const UpsertArgs& a, const ChainArgs& c, hipStream_t s) {
+    hipLaunchKernelGGL((chained_miss_kernel<OP, VEC, UPL>), dim3(grid_for(v.buckets_num)), dim3(kWave), 0,
+                       s, v, a, c);
   }
 };
 
-/* Caller holds the inserter role on `s`. */
-template <int OP>
-int run_grouped(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule,
-                const GroupPlan& p, hipStream_t s) {
-  if (p.bytes > t->scratch_bytes) {
-    /* kernels of earlier calls may still use the old block */
-    HKV_HIP(hipDeviceSynchronize());
+/* Scratch of the two-phase path: the per-bucket list heads (all zero between calls) and the
+ * per-key links.  Grown when a larger batch or a larger table comes along; the caller holds the
+ * inserter role on `s`, so once `s` has drained nothing uses the old block any more. */
+int two_phase_scratch(hkv_table* t, uint64_t n, hipStream_t s, ChainArgs& c) {
+  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
+  const uint64_t head_bytes = up(t->view.buckets_num * 4);
+  if (t->scratch_buckets != t->view.buckets_num || n > t->scratch_keys) {
+    HKV_HIP(hipStreamSynchronize(s));
     table_free(t, 0, t->d_scratch);
     t->d_scratch = nullptr;
-    t->scratch_bytes = 0;
-    const uint64_t want = p.bytes + p.bytes / 4;
-    HKV_TRY(table_alloc(t, 0, &t->d_scratch, want));
-    t->scratch_bytes = want;
+    t->scratch_buckets = t->scratch_keys = 0;
+    const uint64_t keys = std::max<uint64_t>(n + n / 4, 1 << 16);
+    HKV_TRY(table_alloc(t, 0, &t->d_scratch, head_bytes + up(keys * 4)));
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((head_bytes / 16 + 255) / 256)), dim3(256), 0, s,
+                       (uint32_t*)t->d_scratch, head_bytes / 4);
+    HKV_HIP(hipGetLastError());
+    t->scratch_buckets = t->view.buckets_num;
+    t->scratch_keys = keys;
   }
-  uint8_t* base = (uint8_t*)t->d_scratch;
-  HitArgs h{};
-  h.absent = base + p.off_absent;
-  dispatch_vec_upl<LaunchHits, OP>(vec, t->view.value_bytes, t->view, a, h, s);
+  c.head = (uint32_t*)t->d_scratch;
+  c.next = (uint32_t*)((uint8_t*)t->d_scratch + head_bytes);
+  return HKV_SUCCESS;
+}
 
-  BinArgs b{};
-  b.keys = a.keys;
-  b.absent = h.absent;
-  b.n = a.n;
-  b.bpb_shift = p.bpb_shift;
-  b.nbins = p.nbins;
-  b.blocks = p.blocks;
-  b.slice = p.slice;
-  b.hist = (uint32_t*)base;
-  b.total = (uint32_t*)(base + p.off_total);
-  b.bin_start = (uint32_t*)(base + p.off_start);
-  b.order = (uint32_t*)(base + p.off_order);
-  const size_t lds = (size_t)p.nbins * 4;
-  hipLaunchKernelGGL(bin_hist_kernel, dim3(p.blocks), dim3(kBinThreads), lds, s, t->view, b);
-  hipLaunchKernelGGL(bin_colscan_kernel, dim3((p.nbins + 255) / 256), dim3(256), 0, s, b);
-  hipLaunchKernelGGL(bin_scatter_kernel, dim3(p.blocks), dim3(kBinThreads), lds, s, t->view, b);
-  GroupArgs g{};
-  g.order = b.order;
-  g.bin_start = b.bin_start;
-  g.bpb_shift = p.bpb_shift;
-  g.locked_rule = locked_rule;
-  dispatch_vec_upl<LaunchMisses, OP>(vec, t->view.value_bytes, t->view, a, g, p.nbins, s);
+/* Caller holds the inserter role on `s`. */
+template <int OP>
+int run_two_phase(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule, hipStream_t s) {
+  ChainArgs c{};
+  HKV_TRY(two_phase_scratch(t, a.n, s, c));
+  c.locked_rule = locked_rule;
+  dispatch_vec_upl<LaunchHits, OP>(vec, t->view.value_bytes, t->view, a, c, s);
+  dispatch_vec_upl<LaunchMisses, OP>(vec, t->view.value_bytes, t->view, a, c, s);
   return HKV_SUCCESS;
 }
 
@@ -687,16 +651,15 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
     HKV_HIP(g.acquire());
     HKV_TRY(settle_locked_count(t, s));
     if (OP == kOpFindOrInsertPtr && a.locked_key_ptrs) t->keys_may_be_locked = true;
-    GroupPlan plan{};
-    if constexpr (OP != kOpFindOrInsertPtr) plan = plan_grouped(t, a.n);
+    bool two_phase = OP != kOpFindOrInsertPtr && two_phase_feasible(t, a.n);
     /* insert_and_evict: the second phase updates the one evicted-counter word once per
-     * wavefront and pass, which serialises at full size (1.14 ms against 0.53 ms per 2^20
-     * keys); only the forced mode of the tests takes it there */
-    if (OP == kOpInsertAndEvict && t->upsert_path != 2) plan.feasible = false;
-    if (vec == 8 || vec == 2) plan.feasible = false; /* units only the slot-lock kernel has */
-    if (plan.feasible) {
+     * wavefront and pass, and updates of one word are served one at a time; only the forced
+     * mode of the tests takes it there */
+    if (OP == kOpInsertAndEvict && t->upsert_path != 2) two_phase = false;
+    if (vec == 8 || vec == 2) two_phase = false; /* units only the slot-lock kernel has */
+    if (two_phase) {
       if constexpr (OP != kOpFindOrInsertPtr)
-        HKV_TRY(run_grouped<OP>(t, a, vec, refuse_equal, plan, s));
+        HKV_TRY(run_two_phase<OP>(t, a, vec, refuse_equal, s));
     } else if (t->keys_may_be_locked) {
       /* slots that lock_keys (or the pointer overload with locked_key_ptrs) left LOCKED must
        * be hidden from the victim scan, which then reads the key words beside the scores; with
@@ -1034,7 +997,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->d_counters = nullptr;
   t->h_values = nullptr;
   t->d_scratch = nullptr;
-  t->scratch_bytes = 0;
+  t->scratch_buckets = t->scratch_keys = 0;
   t->keys_may_be_locked = false;
   t->locked_recount = false;
   t->dual = o->table_mode == 1;

@@ -530,7 +530,7 @@ upsert_kernel(View v, UpsertArgs a) {
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
   s_unsure[lane] = 0;
   __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, s_em, s_unsure, lane);
+  probe_wave<true, kTwoStepWriters>(v, s_meta, s_slot, s_em, s_unsure, lane);
   __syncthreads();
 
   /* ---- state of the key this lane owns ---------------------------------------------- */
@@ -798,7 +798,7 @@ assign_kernel(View v, AssignArgs a) {
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   s_unsure[lane] = 0;
   __syncthreads();
-  probe_wave<true>(v, s_meta, s_slot, nullptr, s_unsure, lane);
+  probe_wave<true, kTwoStepWriters>(v, s_meta, s_slot, nullptr, s_unsure, lane);
   __syncthreads();
   const KeyMeta me = s_meta[lane];
   int64_t hit = s_slot[lane];
