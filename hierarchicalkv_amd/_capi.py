@@ -84,6 +84,7 @@ SIGNATURES = {
     "hkv_table_create_with_allocator": (_i, [C.POINTER(Options), _p, C.POINTER(_T)]),
     "hkv_table_destroy": (_i, [_T]),
     "hkv_insert_or_assign": (_i, [_T, _u64, _p, _p, _p, _p, _i, _i]),
+    "hkv_insert_or_assign_noalloc": (_i, [_T, _u64, _p, _p, _p, _p, _i]),
     "hkv_insert_and_evict": (_i, [_T, _u64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i]),
     "hkv_insert_and_evict_count": (_i, [_T, _u64, _p, _p, _p, _p, _p, _p, _p, _i, _i, C.POINTER(_u64)]),
     "hkv_accum_or_assign": (_i, [_T, _u64, _p, _p, _p, _p, _p, _i]),

@@ -409,6 +409,37 @@ int run_two_phase(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule, 
   return HKV_SUCCESS;
 }
 
+/* ---- the two-phase path on a scratch area that is part of the library image -----------------
+ * hkv_insert_or_assign_noalloc: list heads and links live in a file-scope device array instead
+ * of memory the call may have to allocate.  In host code the array's name is only a handle for
+ * the symbol: its device address is looked up once per device (each device holds its own copy
+ * of the array) and that pointer is what the kernels and the clearing launch get. */
+constexpr uint64_t kNoAllocMaxBuckets = UINT64_C(1) << 20; /* capacity up to 2^27 */
+constexpr uint64_t kNoAllocMaxKeys = UINT64_C(1) << 20;
+
+}  // namespace
+static __device__ __align__(256) uint32_t g_noalloc_scratch[kNoAllocMaxBuckets + kNoAllocMaxKeys];
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_noalloc_mu;
+uint32_t* g_noalloc_ptr[kMaxDevices]; /* device address of g_noalloc_scratch, per device */
+
+/* The device's copy of the scratch array.  The caller has made `device` current. */
+int noalloc_scratch(int device, uint32_t** out) {
+  if (device < 0 || device >= kMaxDevices)
+    return fail(HKV_ERROR_UNSUPPORTED, "device %d: the scratch table holds %d devices", device, kMaxDevices);
+  std::lock_guard<std::mutex> g(g_noalloc_mu);
+  if (!g_noalloc_ptr[device]) {
+    void* p = nullptr;
+    HKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_noalloc_scratch)));
+    if (!p) return fail(HKV_ERROR_HIP, "hipGetSymbolAddress returned a null address");
+    g_noalloc_ptr[device] = (uint32_t*)p;
+  }
+  *out = g_noalloc_ptr[device];
+  return HKV_SUCCESS;
+}
+
 constexpr unsigned kCounterWords = 128;
 
 /* A device word for a call that returns a count.  The word belongs to the call from the
@@ -1195,6 +1226,68 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
   /* with unique_key == false the reference leaves its lock-key kernels for the plain one
    * (merlin_hashtable.cuh:1235-1258), whose rule is "refuse when score < min" */
   return run_upsert<kOpInsertOrAssign>(t, a, vec, unique_key != 0, (hipStream_t)stream);
+}
+
+int hkv_insert_or_assign_noalloc(hkv_table* t, uint64_t n, const uint64_t* keys,
+                                 const void* values, const uint64_t* scores,
+                                 hkv_stream_t stream, int ignore) {
+  if (n == 0) return HKV_SUCCESS;
+  if (n > kNoAllocMaxKeys)
+    return fail(HKV_ERROR_ARGUMENT, "hkv_insert_or_assign_noalloc: %llu keys, the limit is %llu per call",
+                (unsigned long long)n, (unsigned long long)kNoAllocMaxKeys);
+  if (t->view.buckets_num > kNoAllocMaxBuckets)
+    return fail(HKV_ERROR_UNSUPPORTED,
+                "hkv_insert_or_assign_noalloc: the table has %llu buckets, the limit is %llu",
+                (unsigned long long)t->view.buckets_num, (unsigned long long)kNoAllocMaxBuckets);
+  if (t->dual || t->io_by_cpu || !t->opts.api_lock)
+    return fail(HKV_ERROR_UNSUPPORTED,
+                "hkv_insert_or_assign_noalloc needs a single-bucket table with api_lock and without io_by_cpu");
+  if (!t->reach_max_capacity)
+    return fail(HKV_ERROR_UNSUPPORTED,
+                "hkv_insert_or_assign_noalloc: the table can still grow, and growing allocates; "
+                "reserve() it to max_capacity first");
+  const int strategy = ignore ? HKV_CUSTOMIZED : t->opts.evict_strategy;
+  if (!ignore) HKV_TRY(check_scores_arg(t, strategy, scores));
+  hipStream_t s = (hipStream_t)stream;
+  DeviceGuard dev(t->device);
+  if (!dev.ok) return fail(HKV_ERROR_HIP, "cannot make device %d current", t->device);
+  uint32_t* scratch = nullptr;
+  HKV_TRY(noalloc_scratch(t->device, &scratch));
+  UpsertArgs a{};
+  a.keys = keys;
+  a.values_in = (const uint8_t*)values;
+  a.scores = scores;
+  a.n = n;
+  a.strategy = strategy;
+  a.epoch = t->epoch;
+  a.clock = t->clock;
+  a.value_kind = t->opts.value_kind;
+  a.refuse_equal = !t->pure_hbm; /* the lock-key rule of hybrid mode, as hkv_insert_or_assign */
+  const int vec = pick_vec(t->view.value_bytes, {values});
+  {
+    LockGuard g(t, StreamGroupLock::kInserter, s);
+    HKV_HIP(g.acquire());
+    /* slots left LOCKED by lock_keys are invisible to the second phase; whether any are left
+     * after unlock_keys is settled by the next ordinary upsert (it reads a device counter) */
+    if (t->keys_may_be_locked)
+      return fail(HKV_ERROR_UNSUPPORTED,
+                  "hkv_insert_or_assign_noalloc: keys may be locked (lock_keys / find_or_insert with "
+                  "locked_key_ptrs)");
+    ChainArgs c{};
+    c.head = scratch;
+    c.next = scratch + kNoAllocMaxBuckets;
+    c.locked_rule = a.refuse_equal;
+    /* the array keeps what the last call on this device left in it (all zero after a call
+     * that ran to its end, but a call may have failed half way): the heads start at zero */
+    const uint64_t head_words = (t->view.buckets_num + 3) & ~UINT64_C(3);
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((head_words / 4 + 255) / 256)), dim3(256), 0, s,
+                       c.head, head_words);
+    dispatch_vec_upl<LaunchHits, kOpInsertOrAssign>(vec, t->view.value_bytes, t->view, a, c, s);
+    dispatch_vec_upl<LaunchMisses, kOpInsertOrAssign>(vec, t->view.value_bytes, t->view, a, c, s);
+    HKV_HIP(hipGetLastError());
+  }
+  if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
+  return HKV_SUCCESS;
 }
 
 int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,

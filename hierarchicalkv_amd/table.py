@@ -125,6 +125,12 @@ class HashTable:
         _check(lib.hkv_insert_or_assign(self._h, n, _ptr(keys), _ptr(values), _ptr(scores),
                                         _stream(stream), int(unique_key), int(ignore_evict_strategy)))
 
+    def insert_or_assign_noalloc(self, n, keys, values, scores=None, stream=None,
+                                 ignore_evict_strategy=False):
+        """insert_or_assign on the library's static scratch area: allocates nothing."""
+        _check(lib.hkv_insert_or_assign_noalloc(self._h, n, _ptr(keys), _ptr(values), _ptr(scores),
+                                                _stream(stream), int(ignore_evict_strategy)))
+
     def insert_and_evict(self, n, keys, values, scores, evicted_keys, evicted_values,
                          evicted_scores, d_evicted_counter=None, stream=None,
                          unique_key=True, ignore_evict_strategy=False):

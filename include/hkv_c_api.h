@@ -168,6 +168,22 @@ int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
                          hkv_stream_t stream, int unique_key,
                          int ignore_evict_strategy);
 
+/* insert_or_assign for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same results as hkv_insert_or_assign with unique_key = 1, through the two-phase
+ * path: its scratch (one 32-bit list head per bucket, one link per key) lives in a device array
+ * that is part of the library image, 8 MiB per GPU, held until the process ends, instead of
+ * memory allocated by the call; the call itself allocates nothing.
+ * Limits: n <= 2^20 keys per call, tables of up to 2^20 buckets (capacity 2^27), keys unique in
+ * the batch, a table that cannot grow any more (init_capacity * 2 > max_capacity, or grown to the
+ * maximum), api_lock on, no io_by_cpu, no dual-bucket mode, no keys held by lock_keys: anything
+ * else is refused with HKV_ERROR_ARGUMENT / HKV_ERROR_UNSUPPORTED and a message.
+ * All calls on one GPU share that GPU's array (also across tables): calls that overlap in time on
+ * one GPU race on it; calls on one stream, or ordered by the group lock of one table, do not. */
+int hkv_insert_or_assign_noalloc(hkv_table* t, uint64_t n, const uint64_t* keys,
+                                 const void* values, const uint64_t* scores,
+                                 hkv_stream_t stream, int ignore_evict_strategy);
+
 /* HashTable::insert_and_evict (device counter overload),
  * merlin_hashtable.cuh:1351-1473.  The caller zeroes *d_evicted_counter. */
 int hkv_insert_and_evict(hkv_table* t, uint64_t n, const uint64_t* keys,
