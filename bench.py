@@ -71,6 +71,12 @@ def main():
                     help="instead of the one-line benchmark: every entry point at the metric shape "
                          "(capacity 2^26, dim 64, batch 2^20, load factor 1.0), kernel time by HIP "
                          "events and algorithmic GB/s against the 8 TB/s peak, printed as markdown")
+    ap.add_argument("--config", type=int, choices=[2, 3, 4, 5], default=0,
+                    help="instead of the one-line benchmark: the measurement protocol of one of the other "
+                         "workload configurations at its full size (2: dim 8 at load factor 0.50 / 0.75 / 1.00; "
+                         "3: Zipf insert_and_evict + find at 2^27, dim 64; 4: hybrid HBM + pinned host rows at "
+                         "2^28 with HBM and host-link GB/s apart; 5: accum_or_assign / export_batch_if / erase "
+                         "at 2^25, dim 128); a markdown table and one JSON line")
     ap.add_argument("--ceilings", action="store_true",
                     help="instead of the one-line benchmark: what the memory system needs for the access "
                          "patterns of find and insert_or_assign at the same shape with no table logic "
@@ -102,6 +108,9 @@ def main():
         return
     if args.ceilings:
         run_ceilings(args)
+        return
+    if args.config:
+        run_config(args, torch)
         return
     cap = 1 << args.capacity_log2
     dim = args.dim
@@ -460,6 +469,300 @@ def run_ops(args, np, torch, dev, w):
         print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f |" % (name, ms, n / ms / 1e6, bpk, gbs, gbs / HBM_PEAK_GBS),
               flush=True)
     table.close()
+
+
+def run_config(args, torch):
+    """Configurations 2 to 5 at full size: every call is timed by HIP events around it on the
+    stream the library launches on, `reps` isolated calls per figure (a synchronisation before
+    each, fresh keys every time, so nothing of a call's working set is in the caches).
+    Algorithmic bytes per key, VB = row bytes: find hit 145 + 2 VB, miss 137; find* hit 153;
+    upsert of a key that is present 161 + 2 VB (find_or_insert: 169 + 2 VB), of an absent key into
+    a free slot 169 + 2 VB, into a full bucket 1185 + 2 VB; insert_and_evict evicting 1201 + 4 VB;
+    accum_or_assign accumulating 161 + 3 VB; export 16 per scanned slot + (2 VB + 16) per match;
+    erase 165.  Mixes are priced by the outcome fractions the run itself observes."""
+    import workloads_device as wd
+    from hierarchicalkv_amd import EvictStrategy, HashTable, Predicate, default_options
+
+    dev = wd.DEV
+    n = 1 << 20
+    reps = 3
+    rows = []
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b)
+
+    def add(name, ms_list, bpk, keys=n, extra=None):
+        ms = sum(ms_list) / len(ms_list)
+        gbs = bpk * keys / (ms * 1e-3) / 1e9
+        r = {"op": name, "ms": round(ms, 4), "bkvs": round(keys / (ms * 1e-3) / 1e9, 3),
+             "bytes_per_key": round(bpk, 1), "algorithmic_gbs": round(gbs, 1),
+             "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        if extra:
+            r.update(extra)
+        rows.append(r)
+        print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f | %s |" % (
+            name, ms, r["bkvs"], bpk, gbs, gbs / HBM_PEAK_GBS,
+            "; ".join("%s %s" % kv for kv in (extra or {}).items())), flush=True)
+
+    print("| call | ms per call | 10^9 KV/s | algorithmic bytes per key | algorithmic GB/s | fraction of 8 TB/s | notes |")
+    print("|---|---|---|---|---|---|---|")
+    founds = torch.empty(n, dtype=torch.bool, device=dev)
+    info = {}
+
+    if args.config == 2:
+        cap, dim, seed = 1 << 26, 8, 2
+        vb = dim * 4
+        t = HashTable()
+        t.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb, dim=dim,
+                               evict_strategy=EvictStrategy.kLru))
+        out = torch.empty(n, dim, dtype=torch.float32, device=dev)
+        vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
+        pos, fresh, old = 0, 1 << 36, 0
+        for lf in (0.50, 0.75, 1.00):
+            while pos < int(lf * cap) or (lf == 1.0 and t.size() < 0.999 * cap and pos < 3 * cap):
+                t.insert_or_assign(n, wd.dev_keys(seed, pos, n), vals)
+                pos += n
+            size = t.size()
+
+            def resident():  # an old batch: still resident (inserted within the last capacity's worth), cold
+                nonlocal old
+                old += 1
+                return wd.dev_keys(seed, pos - (8 + old % 16) * n, n)
+
+            def mixed():
+                nonlocal fresh
+                k = torch.cat([resident()[: n // 2], wd.dev_keys(seed, fresh, n // 2)])
+                fresh += n // 2
+                return k
+
+            full = size > 0.99 * cap
+            miss = (1185 if full else 169) + 2 * vb
+            ms = []
+            for _ in range(reps):
+                k = resident()
+                ms.append(timed(lambda: t.find(n, k, out, founds)))
+            add("find (100 %% hit), load factor %.2f" % (size / cap), ms, 145 + 2 * vb,
+                extra={"hit_rate": round(float(founds.float().mean().item()), 4)})
+            ms = []
+            for _ in range(reps):
+                k = mixed()
+                ms.append(timed(lambda: t.insert_or_assign(n, k, vals)))
+            add("insert_or_assign (50 %% new), load factor %.2f" % (size / cap), ms,
+                0.5 * (161 + 2 * vb) + 0.5 * miss)
+            ms = []
+            for _ in range(reps):
+                k = mixed()
+                ms.append(timed(lambda: t.find_or_insert(n, k, out)))
+            add("find_or_insert (50 %% new), load factor %.2f" % (size / cap), ms,
+                0.5 * (169 + 2 * vb) + 0.5 * miss, extra={"load_factor_after": round(t.size() / cap, 4)})
+        info = {"workload": "capacity 2^26, dim 8 fp32, LRU, batch 2^20, uniform keys"}
+        t.close()
+
+    elif args.config == 3:
+        cap, dim, seed = 1 << 27, 64, 3
+        vb = dim * 4
+        t = HashTable()
+        t.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb, dim=dim,
+                               evict_strategy=EvictStrategy.kCustomized))
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(0x484B5603)
+        batch = 1
+        # uniform keys up to load factor 1.0 (the lowest scores), then 24 batches of the Zipf
+        # stream so that the timed calls meet the steady state: hot keys resident, tail evicted
+        vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
+        pos = 0
+        while pos < cap or (t.size() < 0.999 * cap and pos < 3 * cap):
+            k = wd.dev_keys(seed, pos, n)
+            t.insert_or_assign(n, k, vals, wd.batch_scores(k, batch))
+            pos += n
+            batch += 1
+        for _ in range(24):
+            k = wd.zipf_keys(gen, n)
+            t.insert_or_assign(n, k, vals, wd.batch_scores(k, batch))
+            batch += 1
+        size0 = t.size()
+        ek = torch.zeros(n, dtype=torch.int64, device=dev)
+        es = torch.zeros(n, dtype=torch.int64, device=dev)
+        ev = torch.zeros(n, dim, dtype=torch.float32, device=dev)
+        out = torch.empty(n, dim, dtype=torch.float32, device=dev)
+        cnt = torch.zeros(1, dtype=torch.int64, device=dev)
+        ms_i, ms_f, hits, evs = [], [], [], []
+        for _ in range(reps + 2):
+            k = wd.zipf_keys(gen, n)
+            sc = wd.batch_scores(k, batch)
+            batch += 1
+            t.contains(n, k, founds)
+            hit = float(founds.float().mean().item())
+            cnt.zero_()
+            ms = timed(lambda: t.insert_and_evict(n, k, vals, sc, ek, ev, es, cnt))
+            evicted = int(cnt.item())
+            msf = timed(lambda: t.find(n, k, out, founds))
+            if _ >= 2:
+                ms_i.append(ms)
+                ms_f.append(msf)
+                hits.append(hit)
+                evs.append(evicted / n)
+        h = sum(hits) / len(hits)
+        e = sum(evs) / len(evs)
+        add("insert_and_evict (Zipf 1.05 over 2^31, load factor 1.0)", ms_i,
+            h * (161 + 2 * vb) + e * (1201 + 4 * vb) + max(0.0, 1.0 - h - e) * (169 + 2 * vb),
+            extra={"present": round(h, 4), "evicting": round(e, 4)})
+        add("find on the same keys (all resident)", ms_f, 145 + 2 * vb,
+            extra={"hit_rate": round(float(founds.float().mean().item()), 4)})
+        info = {"workload": "capacity 2^27, dim 64 fp32 (32 GiB of rows in HBM), Customized scores "
+                            "(batch << 40 | mix), batch 2^20 unique keys with power-law ranks (alpha 1.05) "
+                            "over 2^31; table filled with uniform keys, then 24 batches of the same stream",
+                "size": size0, "fill_batches": batch}
+        t.close()
+
+    elif args.config == 4:
+        cap, dim, seed = 1 << 28, 64, 4
+        vb = dim * 4
+        hbm = 16 << 30
+        t = HashTable()
+        t0 = time.time()
+        t.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=hbm, dim=dim,
+                               evict_strategy=EvictStrategy.kLfu))
+        assert not t.is_pure_hbm()
+        init_s = time.time() - t0
+        # host-link peak: pinned host <-> device copies of 1 GiB, both directions, in this run
+        pin = torch.empty(1 << 28, dtype=torch.float32, pin_memory=True)
+        dbuf = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        h2d = min(timed(lambda: dbuf.copy_(pin, non_blocking=True)) for _ in range(3))
+        d2h = min(timed(lambda: pin.copy_(dbuf, non_blocking=True)) for _ in range(3))
+        link = {"h2d_gbs": round((1 << 30) / (h2d * 1e-3) / 1e9, 1), "d2h_gbs": round((1 << 30) / (d2h * 1e-3) / 1e9, 1)}
+        del pin, dbuf
+        ones = torch.ones(n, dtype=torch.int64, device=dev)
+        vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
+        pos = 0
+        while pos < cap or (t.size() < 0.999 * cap and pos < 3 * cap):
+            t.insert_or_assign(n, wd.dev_keys(seed, pos, n), vals, ones)
+            pos += n
+        size0 = t.size()
+        view = t.view()
+        hbm_lo, hbm_hi = int(view.values), int(view.values) + int(view.hbm_slots) * vb
+        out = torch.empty(n, dim, dtype=torch.float32, device=dev)
+        ptrs = torch.zeros(n, dtype=torch.int64, device=dev)
+        fresh, old = 1 << 40, 0
+
+        def mixed(new_fraction):
+            nonlocal fresh, old
+            m = int(n * new_fraction)
+            old += 1
+            # LFU with every frequency equal: a full bucket gives up its lowest slot, so what
+            # stays resident are the keys that found a free slot, i.e. the early batches of the
+            # fill; the hit rate is measured, and the bytes are priced by it
+            k = torch.cat([wd.dev_keys(seed, (old % 160) * n, n)[: n - m], wd.dev_keys(seed, fresh, m)])
+            fresh += m
+            return k
+
+        def host_rows(k):
+            t.find_ptr(n, k, ptrs, founds)
+            torch.cuda.synchronize()
+            f = founds
+            in_hbm = (ptrs >= hbm_lo) & (ptrs < hbm_hi)
+            return int((f & ~in_hbm).sum().item()), int(f.sum().item())
+
+        ms_f, ms_p, ms_i = [], [], []
+        lf, lp, li, hf = [], [], [], []
+        for _ in range(reps):
+            k = mixed(0.2)
+            hostn, foundn = host_rows(k)
+            ms = timed(lambda: t.find(n, k, out, founds))
+            ms_f.append(ms)
+            lf.append(hostn * vb / (ms * 1e-3) / 1e9)
+            hf.append(foundn / n)
+            k = mixed(0.2)
+            ms_p.append(timed(lambda: t.find_ptr(n, k, ptrs, founds)))
+            k = mixed(0.2)
+            ms = timed(lambda: t.insert_or_assign(n, k, vals, ones))
+            hostn, foundn = host_rows(k)   # where the accepted keys' rows are now
+            ms_i.append(ms)
+            li.append(hostn * vb / (ms * 1e-3) / 1e9)
+        hit = sum(hf) / len(hf)
+        alg_find = hit * (145 + 2 * vb) + (1 - hit) * 137
+        add("find (%.0f %% hit)" % (100 * hit), ms_f, alg_find,
+            extra={"host_link_gbs": round(sum(lf) / len(lf), 1),
+                   "hbm_gbs": round((alg_find * n - sum(lf) / len(lf) * 1e9 * (sum(ms_f) / len(ms_f)) * 1e-3)
+                                    / ((sum(ms_f) / len(ms_f)) * 1e-3) / 1e9, 1)})
+        add("find* (%.0f %% hit)" % (100 * hit), ms_p, hit * 153 + (1 - hit) * 137, extra={"host_link_gbs": 0.0})
+        alg_ins = hit * (169 + 2 * vb) + (1 - hit) * (1185 + 8 + 2 * vb)
+        add("insert_or_assign (%.0f %% new)" % (100 * (1 - hit)), ms_i, alg_ins,
+            extra={"host_link_gbs": round(sum(li) / len(li), 1),
+                   "hbm_gbs": round((alg_ins * n - sum(li) / len(li) * 1e9 * (sum(ms_i) / len(ms_i)) * 1e-3)
+                                    / ((sum(ms_i) / len(ms_i)) * 1e-3) / 1e9, 1)})
+        info = {"workload": "capacity 2^28, dim 64 fp32: 16 GiB of the 64 GiB of rows in HBM, 48 GiB in pinned host "
+                            "memory; LFU; batch 2^20 uniform keys; load factor 1.0",
+                "size": size0, "init_s": round(init_s, 1), "host_link_peak": link}
+        t.close()
+
+    else:
+        cap, dim, seed = 1 << 25, 128, 5
+        vb = dim * 4
+        t = HashTable()
+        t.init(default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb, dim=dim,
+                               evict_strategy=EvictStrategy.kEpochLru))
+        vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-0.01, 0.01)
+        flags = torch.empty(n, dtype=torch.bool, device=dev)
+        out = torch.empty(n, dim, dtype=torch.float32, device=dev)
+        pos, batch = 0, 0
+        while pos < cap or (t.size() < 0.999 * cap and pos < 3 * cap):
+            t.set_global_epoch(batch // 10)
+            t.insert_or_assign(n, wd.dev_keys(seed, pos, n), vals)
+            pos += n
+            batch += 1
+        size0 = t.size()
+        fresh, old = 1 << 40, 0
+        ms, hits = [], []
+        for _ in range(reps):
+            old += 1
+            m = int(0.3 * n)
+            k = torch.cat([wd.dev_keys(seed, pos - (4 + old % 8) * n, n)[: n - m], wd.dev_keys(seed, fresh, m)])
+            fresh += m
+            t.set_global_epoch(batch // 10)
+            batch += 1
+            t.contains(n, k, flags)   # accumulate what is there, assign what is not
+            hits.append(float(flags.float().mean().item()))
+            ms.append(timed(lambda: t.accum_or_assign(n, k, vals, flags)))
+        h = sum(hits) / len(hits)
+        add("accum_or_assign (%.0f %% existing)" % (100 * h), ms, h * (161 + 3 * vb) + (1 - h) * (1185 + 1 + 2 * vb))
+        # threshold that keeps about a quarter of the entries: the 75th percentile of a sample of scores
+        sc = torch.zeros(n, dtype=torch.int64, device=dev)
+        t.find(n, wd.dev_keys(seed, pos - 5 * n, n), out, founds, sc)
+        torch.cuda.synchronize()
+        sample = torch.cat([sc[founds]])
+        for back in (1, 9, 13, 17, 21, 25, 29):
+            t.find(n, wd.dev_keys(seed, pos - back * n, n), out, founds, sc)
+            torch.cuda.synchronize()
+            sample = torch.cat([sample, sc[founds]])
+        thr = int(torch.quantile(sample[:: max(1, sample.numel() // (1 << 20))].to(torch.float64), 0.75).item())
+        window = 1 << 22
+        dk = torch.zeros(window, dtype=torch.int64, device=dev)
+        ds = torch.zeros(window, dtype=torch.int64, device=dev)
+        dv = torch.zeros(window, dim, dtype=torch.float32, device=dev)
+        dc = torch.zeros(1, dtype=torch.int64, device=dev)
+        total_ms, matched = 0.0, 0
+        for off in range(0, cap, window):
+            total_ms += timed(lambda: t.export_batch_if(Predicate.kScoreGe, 0, thr, window, off, dc, dk, dv, ds))
+            matched += int(dc.item())
+        add("export_batch_if (score >= threshold, whole table)", [total_ms],
+            (16 * cap + (2 * vb + 16) * matched) / cap, keys=cap,
+            extra={"kept": round(matched / max(1, size0), 4), "windows": cap // window})
+        ms = []
+        ne = 1 << 18
+        for r in range(reps):
+            k = wd.dev_keys(seed, pos - (2 + r) * n, ne)
+            ms.append(timed(lambda: t.erase(ne, k)))
+        add("erase (2^18 keys)", ms, 165, keys=ne)
+        info = {"workload": "capacity 2^25, dim 128 fp32, EpochLRU (epoch = batch / 10), batch 2^20 uniform keys, "
+                            "deltas in [-0.01, 0.01], load factor 1.0", "size": size0}
+    print(json.dumps({"config": args.config, **info, "ops": rows}))
 
 
 CEILING_PATTERNS = [

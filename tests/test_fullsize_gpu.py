@@ -24,42 +24,7 @@ from hierarchicalkv_amd import EvictStrategy, HashTable, Predicate, ValueKind, d
 
 pytestmark = pytest.mark.gpu
 
-M63 = (1 << 63) - 1
-
-
-def _lsr(x, k):
-    return (x >> k) & ((1 << (64 - k)) - 1)
-
-
-def _s64(c):
-    return c - (1 << 64) if c >= (1 << 63) else c
-
-
-def mix64(x):
-    """splitmix64 finaliser on int64 tensors (bit patterns of uint64): a bijection."""
-    z = x + _s64(0x9E3779B97F4A7C15)
-    z = (z ^ _lsr(z, 30)) * _s64(0xBF58476D1CE4E5B9)
-    z = (z ^ _lsr(z, 27)) * _s64(0x94D049BB133111EB)
-    return z ^ _lsr(z, 31)
-
-
-def dev_keys(seed, start, n):
-    """n unique keys: the mix of the counters start..start+n-1; the four reserved
-    patterns (top 62 bits all ones) are folded away by clearing bit 63."""
-    c = torch.arange(start, start + n, dtype=torch.int64, device=DEV) + (seed << 40)
-    k = mix64(c)
-    reserved = (k | 3) == -1
-    return torch.where(reserved, k & M63, k)
-
-
-def value_of(keys, dim):
-    """fp32 row of a key: float(key & 1023) + d."""
-    return (keys & 1023).to(torch.float32)[:, None] + torch.arange(dim, dtype=torch.float32, device=DEV)[None, :]
-
-
-def score_of(keys):
-    """Customized-strategy score of a key: 63-bit mix, distinct for practical purposes."""
-    return _lsr(mix64(keys ^ 0x5555), 1)
+from workloads_device import M63, _lsr, dev_keys, mix64, score_of, value_of  # noqa: E402,F401
 
 
 def make_table(**kw):
