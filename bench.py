@@ -40,12 +40,21 @@ def upsert_bytes(vb, new_fraction):
     return (1.0 - new_fraction) * (161 + 2 * vb) + new_fraction * (1185 + 2 * vb)
 
 
-# HBM bytes per launch on the default workload, from rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE (KiB per dispatch, each scaled by what the same counter reads for a
-# 1 GiB device-to-device copy: 2.000 and 1.000).  Counters cannot be read from inside
-# this process, so the figures of the committed profile summary are reported; they
-# apply to the default workload and the default (slot-lock) upsert path only.
-MEASURED_TRAFFIC = {"upsert_kernel": 1553.3e6, "lookup_kernel": 868.2e6}
+# HBM bytes per launch on the default workload come from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE runs of this very command (KiB per dispatch, each scaled by what the same
+# counter reads for a 1 GiB device-to-device copy in the same run).  Counters cannot be read
+# from inside this process, so `--profile-summary` writes them to a file beside the profile
+# summaries and the default run reports what that file holds; it applies to the default
+# workload and the default (slot-lock) upsert path only.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic_cap2p26_dim64_batch2p20.json")
+
+
+def measured_traffic(kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)["kernels"][kernel]["traffic_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
@@ -62,7 +71,9 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for "
                          "FETCH_SIZE / WRITE_SIZE when profiling)")
-    ap.add_argument("--cpu-capacity-log2", type=int, default=24)
+    ap.add_argument("--cpu-capacity-log2", type=int, default=26,
+                    help="capacity of the host oracle's table for the CPU baseline (the benchmark's own 2^26 by "
+                         "default: 17 GiB of host memory)")
     ap.add_argument("--matrix", action="store_true",
                     help="instead of the one-line benchmark: the reference's own benchmark table "
                          "(README.md:245-317, benchmark/merlin_hashtable_benchmark.cc.cu), every API "
@@ -77,6 +88,11 @@ def main():
                          "3: Zipf insert_and_evict + find at 2^27, dim 64; 4: hybrid HBM + pinned host rows at "
                          "2^28 with HBM and host-link GB/s apart; 5: accum_or_assign / export_batch_if / erase "
                          "at 2^25, dim 128); a markdown table and one JSON line")
+    ap.add_argument("--profile-summary", metavar="DIR", default=None,
+                    help="no GPU needed: condense rocprofv3 output (DIR/<bench|ops>_<trace|fetch|write|l2|rd|wr|sq|tcp>/"
+                         "out_*.csv, made by the commands the summaries list) into profiles/*.md and "
+                         "profiles/traffic_cap2p26_dim64_batch2p20.json, which the default run reports as "
+                         "roofline.traffic")
     ap.add_argument("--ceilings", action="store_true",
                     help="instead of the one-line benchmark: what the memory system needs for the access "
                          "patterns of find and insert_or_assign at the same shape with no table logic "
@@ -86,6 +102,9 @@ def main():
                     help="with --matrix: the hybrid table of README.md:289-303 (dim 64, capacity "
                          "128M, 16 GB of the rows in HBM, the rest in pinned host memory)")
     args = ap.parse_args()
+    if args.profile_summary:
+        summarize_profiles(args.profile_summary)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path "
               "(one table per device, as in the reference); run with --gpus 1",
@@ -220,8 +239,8 @@ def main():
     default_workload = (args.capacity_log2 == 26 and dim == 64 and args.batch_log2 == 20
                         and not args.warm_keys)
     path = os.environ.get("HKV_UPSERT_PATH", "locked")
-    ups_traffic = MEASURED_TRAFFIC["upsert_kernel"] if default_workload and path == "locked" else None
-    find_traffic = MEASURED_TRAFFIC["lookup_kernel"] if default_workload else None
+    ups_traffic = measured_traffic("upsert_kernel") if default_workload and path == "locked" else None
+    find_traffic = measured_traffic("lookup_kernel") if default_workload else None
     result = {
         "metric": "billion-KV/s for find & insert_or_assign, dim 64, load factor 1.0, 1 GPU",
         "value": round(value, 4),
@@ -469,6 +488,200 @@ def run_ops(args, np, torch, dev, w):
         print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f |" % (name, ms, n / ms / 1e6, bpk, gbs, gbs / HBM_PEAK_GBS),
               flush=True)
     table.close()
+
+
+PROFILE_GROUPS = [
+    ("trace", "--kernel-trace --stats"),
+    ("fetch", "--kernel-trace --pmc FETCH_SIZE TCC_EA0_RDREQ_DRAM_sum"),
+    ("write", "--kernel-trace --pmc WRITE_SIZE TCC_EA0_ATOMIC_sum TCC_ATOMIC_sum"),
+    ("l2", "--kernel-trace --pmc TCC_HIT_sum TCC_MISS_sum TCC_REQ_sum TCC_EA0_RDREQ_32B_sum"),
+    ("rd", "--kernel-trace --pmc TCC_EA0_RDREQ_sum TCC_EA0_RDREQ_64B_sum TCC_EA0_RDREQ_128B_sum TCC_BUBBLE_sum"),
+    ("wr", "--kernel-trace --pmc TCC_EA0_WRREQ_sum TCC_EA0_WRREQ_64B_sum TCC_WRITE_sum TCC_READ_sum"),
+    ("sq", "--kernel-trace --pmc OccupancyPercent SQ_WAVES SQ_LDS_BANK_CONFLICT SQ_INSTS_LDS SQ_WAIT_INST_ANY "
+           "SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR"),
+    ("tcp", "--kernel-trace --pmc TCP_TCC_READ_REQ_sum TCP_TCC_WRITE_REQ_sum TCP_TCC_ATOMIC_WITH_RET_REQ_sum "
+            "TCP_UTCL1_TRANSLATION_MISS_sum"),
+]
+# kernels of bench.py --ops, in the order of its table: (substring of the kernel name, call, algorithmic bytes per key)
+OPS_KERNELS = [
+    ("lookup_kernel<0, 16", "find (100 % hit)", 657),
+    ("lookup_kernel<1, 16", "find* (100 % hit)", 153),
+    ("lookup_kernel<2, 16", "contains (100 % hit)", 145),
+    ("assign_kernel<16, 2, true>", "assign (100 % hit)", 673),
+    ("upsert_kernel<0, 16, 2, false>", "insert_or_assign (50 % new)", 1185),
+    ("upsert_kernel<2, 16, 2, false>", "find_or_insert (50 % new)", 1189),
+    ("upsert_kernel<4, 16, 1, false>", "find_or_insert* (50 % new)", 689),
+    ("upsert_kernel<1, 16, 2, false>", "insert_and_evict (50 % new)", 1449),
+    ("upsert_kernel<3, 16, 2, false>", "accum_or_assign (50 % new)", 1314),
+    ("export_if_kernel", "export_batch_if (2^20 slots, all match)", 544),
+    ("erase_kernel<true>", "erase (100 % hit)", 165),
+]
+
+
+def summarize_profiles(root):
+    """rocprofv3 CSVs -> profiles/*.md + the traffic file.  Per kernel: the average over its last
+    dispatches (the timed calls: the launches of the table fill come first), durations from the
+    --kernel-trace --stats run, counters from the --pmc runs, FETCH_SIZE / WRITE_SIZE scaled by what
+    they read for the 1 GiB device copy of the same run (--calibrate)."""
+    import collections
+    import csv
+    import glob
+
+    def csv_of(tag, group, kind):
+        hits = glob.glob(os.path.join(root, "%s_%s" % (tag, group), "**", "*%s.csv" % kind), recursive=True)
+        return hits[0] if hits else None
+
+    def counters(tag, group):
+        by = collections.defaultdict(lambda: collections.defaultdict(list))
+        meta = {}
+        f = csv_of(tag, group, "counter_collection")
+        if not f:
+            return by, meta
+        for r in csv.DictReader(open(f)):
+            by[r["Kernel_Name"]][r["Counter_Name"]].append(float(r["Counter_Value"]))
+            meta[r["Kernel_Name"]] = (int(r["VGPR_Count"]), int(r["Accum_VGPR_Count"]), int(r["LDS_Block_Size"]),
+                                      int(r["Scratch_Size"]), int(r["Workgroup_Size"]), int(r["Grid_Size"]))
+        return by, meta
+
+    def durations(tag):
+        by = collections.defaultdict(list)
+        f = csv_of(tag, "trace", "kernel_trace")
+        if f:
+            for r in csv.DictReader(open(f)):
+                by[r["Kernel_Name"]].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+        return by
+
+    def pick(table, needle):
+        for name in table:
+            if needle in name:
+                return name
+        return None
+
+    # bench.py --ops launches lookup_kernel<values> twice: 8 times for its find row (the first 8
+    # dispatches, 2 of them warm-up) and again, at a 50 % hit rate, to make accum_or_assign's flags
+    first_eight = {"find (100 % hit)"}
+
+    def last(values, k, call=None):
+        v = values[2:8] if call in first_eight and k == 6 else values[-k:]
+        return sum(v) / len(v) if v else float("nan")
+
+    n = 1 << 20
+    traffic = {"workload": "capacity 2^26, dim 64 fp32, batch 2^20, LRU, load factor 1.0", "kernels": {}}
+    for tag, cmd, take, kernels, fname, title in [
+        ("bench", "python3 bench.py --steps 4 --warmup 1 --no-cpu-baseline --calibrate", 3,
+         [("lookup_kernel<0, 16", "find (100 % hit)", 657), ("upsert_kernel<0, 16, 2, false>", "insert_or_assign (50 % new)", 1185)],
+         "lookup_kernel_upsert_kernel_cap2p26_dim64_batch2p20.md",
+         "lookup_kernel (find) and upsert_kernel (insert_or_assign) on the benchmark's workload"),
+        ("ops", "python3 bench.py --ops", 6, OPS_KERNELS, "all_entry_points_cap2p26_dim64_batch2p20.md",
+         "every entry point at the benchmark's shape (bench.py --ops)"),
+    ]:
+        dur = durations(tag)
+        if not dur:
+            continue
+        groups = {g: counters(tag, g) for g, _ in PROFILE_GROUPS if g != "trace"}
+        fe, _ = groups["fetch"]
+        wr, _ = groups["write"]
+        copyk = pick(fe, "copyBuffer")
+        cal_f = cal_w = None
+        if copyk and tag == "bench":
+            cal_f = (1 << 20) / max(fe[copyk]["FETCH_SIZE"])      # KiB of a 1 GiB copy / counter
+            cal_w = (1 << 20) / max(wr[pick(wr, "copyBuffer")]["WRITE_SIZE"])
+            traffic["calibration"] = {"fetch_factor": round(cal_f, 4), "write_factor": round(cal_w, 4),
+                                      "by": "1 GiB device-to-device copy in the same rocprofv3 run"}
+        else:
+            cal = traffic.get("calibration", {"fetch_factor": 2.0, "write_factor": 1.0})
+            cal_f, cal_w = cal["fetch_factor"], cal["write_factor"]
+        o = ["# rocprofv3: %s\n" % title,
+             "Workload: capacity 2^26, dim 64 fp32 (16 GiB of rows in HBM), batch 2^20 unique keys, LRU, load factor 1.0.",
+             "One MI355X.  Commands, from the repository root after `cd /tmp && export TMPDIR=/tmp && cd -`, one run each:\n"]
+        bench_cmd = "python3 bench.py --steps 10 --warmup 3 --no-cpu-baseline" if tag == "bench" else cmd
+        for g, pargs in PROFILE_GROUPS:
+            o.append("    rocprofv3 %s --output-format csv -d gpurun_out/prof/%s_%s -o out -- %s" % (
+                pargs, tag, g, bench_cmd if g == "trace" else cmd))
+        o.append("    python3 bench.py --profile-summary gpurun_out/prof\n")
+        o.append("Every figure is the average over the last %d dispatches of the kernel in its run (the timed calls; the "
+                 "launches that fill the table come first).  FETCH_SIZE and WRITE_SIZE are scaled by what they read for a "
+                 "plain 1 GiB device copy (factors %.3f and %.3f).  Counter runs serialise the kernels and slow them "
+                 "down; durations are those of the trace run.\n" % (take, cal_f, cal_w))
+        o.append("## Time and HBM traffic\n")
+        o.append("| call | kernel | avg us | algorithmic MB | FETCH MB | WRITE MB | traffic / algorithmic | algorithmic GB/s | "
+                 "fraction of 8 TB/s | traffic GB/s |\n|---|---|---|---|---|---|---|---|---|---|")
+        detail = []
+        for needle, call, bpk in kernels:
+            k = pick(dur, needle)
+            if not k:
+                continue
+            us = last(dur[k], take, call)
+            alg = bpk * n / 1e6
+            kf, kw = pick(fe, needle), pick(wr, needle)
+            fmb = last(fe[kf]["FETCH_SIZE"], take, call) * cal_f * 1024 / 1e6 if kf else float("nan")
+            wmb = last(wr[kw]["WRITE_SIZE"], take, call) * cal_w * 1024 / 1e6 if kw else float("nan")
+            short = k.split("(")[0].replace("void ", "").replace("hkv::", "")
+            o.append("| %s | `%s` | %.1f | %.1f | %.1f | %.1f | %.2f | %.0f | %.3f | %.0f |" % (
+                call, short, us, alg, fmb, wmb, (fmb + wmb) / alg, alg / us * 1e3, alg / us * 1e3 / HBM_PEAK_GBS,
+                (fmb + wmb) / us * 1e3))
+            if tag == "bench":
+                key = "lookup_kernel" if "lookup" in needle else "upsert_kernel"
+                traffic["kernels"][key] = {"kernel": short, "traffic_bytes": round((fmb + wmb) * 1e6),
+                                           "fetch_bytes": round(fmb * 1e6), "write_bytes": round(wmb * 1e6),
+                                           "avg_us": round(us, 1), "algorithmic_bytes": round(alg * 1e6)}
+            row = {"call": call}
+            for g in ("write", "l2", "rd", "wr", "sq", "tcp"):
+                by, meta = groups[g]
+                kk = pick(by, needle)
+                if kk:
+                    for c, v in by[kk].items():
+                        row[c] = last(v, take, call)
+                    row["meta"] = meta[kk]
+            detail.append(row)
+
+        def col(r, c, scale=1.0, fmt="%.2f"):
+            return fmt % (r[c] * scale) if c in r else "-"
+
+        o.append("\n## L2 (TCC) and its requests to memory, millions per launch\n")
+        o.append("| call | L2 requests | L2 hit rate | reads to memory | of them 128 B | 64 B | 32 B | writes to memory | of them full 64 B | "
+                 "partial (below 64 B: read-modify-write at the memory side) | atomics to memory |\n|---|---|---|---|---|---|---|---|---|---|---|")
+        for r in detail:
+            hit = "%.3f" % (r["TCC_HIT_sum"] / max(1.0, r["TCC_REQ_sum"])) if "TCC_HIT_sum" in r else "-"
+            part = "%.2f" % ((r["TCC_EA0_WRREQ_sum"] - r["TCC_EA0_WRREQ_64B_sum"]) / 1e6) if "TCC_EA0_WRREQ_sum" in r else "-"
+            o.append("| %s | %s | %s | %s | %s | %s | %s | %s | %s | %s | %s |" % (
+                r["call"], col(r, "TCC_REQ_sum", 1e-6), hit, col(r, "TCC_EA0_RDREQ_sum", 1e-6),
+                col(r, "TCC_EA0_RDREQ_128B_sum", 1e-6), col(r, "TCC_EA0_RDREQ_64B_sum", 1e-6, "%.3f"),
+                col(r, "TCC_EA0_RDREQ_32B_sum", 1e-6, "%.3f"), col(r, "TCC_EA0_WRREQ_sum", 1e-6),
+                col(r, "TCC_EA0_WRREQ_64B_sum", 1e-6), part, col(r, "TCC_EA0_ATOMIC_sum", 1e-6)))
+        o.append("\n## Wavefronts, LDS, vector memory, address translation\n")
+        o.append("Registers per lane: twice rocprofv3's VGPR_Count field, which counts register pairs on this part (the "
+                 "compiler's resource report for the same kernels reads 114 and 182 registers, allocated as 120 and 184).\n")
+        o.append("| call | wavefronts | vector registers per lane | LDS bytes per workgroup | scratch | occupancy % of the maximum | vector memory reads "
+                 "/ writes (M instructions) | L1 -> L2 read / write requests (M) | returning atomics (M) | L1 TLB misses (M) | "
+                 "LDS instructions (M) | LDS bank-conflict cycles (M) |\n|---|---|---|---|---|---|---|---|---|---|---|---|")
+        for r in detail:
+            m = r.get("meta", (0, 0, 0, 0, 0, 0))
+            o.append("| %s | %s | %d | %d | %d | %s | %s / %s | %s / %s | %s | %s | %s | %s |" % (
+                r["call"], col(r, "SQ_WAVES", 1.0, "%.0f"), 2 * (m[0] + m[1]), m[2], m[3], col(r, "OccupancyPercent", 1.0, "%.1f"),
+                col(r, "SQ_INSTS_VMEM_RD", 1e-6), col(r, "SQ_INSTS_VMEM_WR", 1e-6), col(r, "TCP_TCC_READ_REQ_sum", 1e-6),
+                col(r, "TCP_TCC_WRITE_REQ_sum", 1e-6), col(r, "TCP_TCC_ATOMIC_WITH_RET_REQ_sum", 1e-6),
+                col(r, "TCP_UTCL1_TRANSLATION_MISS_sum", 1e-6), col(r, "SQ_INSTS_LDS", 1e-6),
+                col(r, "SQ_LDS_BANK_CONFLICT", 1e-6)))
+        if tag == "bench":
+            stats = csv_of(tag, "trace", "kernel_stats")
+            if stats:
+                o.append("\n## `--stats` of the trace run (whole process, table fill included)\n")
+                o.append("| kernel | calls | avg us | min us | max us | % of GPU time |\n|---|---|---|---|---|---|")
+                for r in csv.DictReader(open(stats)):
+                    if "hkv::" in r["Name"]:
+                        o.append("| `%s` | %s | %.1f | %.1f | %.1f | %s |" % (
+                            r["Name"].split("(")[0].replace("void ", "").replace("hkv::", ""), r["Calls"],
+                            float(r["AverageNs"]) / 1e3, float(r["MinNs"]) / 1e3, float(r["MaxNs"]) / 1e3, r["Percentage"]))
+        path = os.path.join(ROOT, "profiles", fname)
+        with open(path, "w") as f:
+            f.write("\n".join(o) + "\n")
+        print("wrote", path)
+    if traffic["kernels"]:
+        with open(TRAFFIC_FILE, "w") as f:
+            json.dump(traffic, f, indent=1)
+            f.write("\n")
+        print("wrote", TRAFFIC_FILE)
 
 
 def run_config(args, torch):
