@@ -88,6 +88,10 @@ def main():
                          "3: Zipf insert_and_evict + find at 2^27, dim 64; 4: hybrid HBM + pinned host rows at "
                          "2^28 with HBM and host-link GB/s apart; 5: accum_or_assign / export_batch_if / erase "
                          "at 2^25, dim 128); a markdown table and one JSON line")
+    ap.add_argument("--group-lock", action="store_true",
+                    help="instead of the one-line benchmark: what the API-level group lock costs the host per call, "
+                         "as built (stream events, never blocks) against a host-blocking acquisition as the "
+                         "reference does it (a one-thread kernel on a side stream plus a stream synchronisation)")
     ap.add_argument("--profile-summary", metavar="DIR", default=None,
                     help="no GPU needed: condense rocprofv3 output (DIR/<bench|ops>_<trace|fetch|write|l2|rd|wr|sq|tcp>/"
                          "out_*.csv, made by the commands the summaries list) into profiles/*.md and "
@@ -130,6 +134,9 @@ def main():
         return
     if args.config:
         run_config(args, torch)
+        return
+    if args.group_lock:
+        run_group_lock(torch)
         return
     cap = 1 << args.capacity_log2
     dim = args.dim
@@ -488,6 +495,75 @@ def run_ops(args, np, torch, dev, w):
         print("| %s | %.4f | %.2f | %.0f | %.0f | %.3f |" % (name, ms, n / ms / 1e6, bpk, gbs, gbs / HBM_PEAK_GBS),
               flush=True)
     table.close()
+
+
+def run_group_lock(torch):
+    """Host time per API call, small batches so that the GPU work is negligible (1024 keys, dim 8):
+    api_lock off / on with one stream (nothing to wait for, nothing recorded) / on with readers and
+    an inserter alternating on two streams (every call records one event and waits for one) / a
+    host-blocking acquisition in front of every call, which is what group_lock.cuh:130-166 costs
+    (lock kernel <<<1,1>>> on a side stream, then cudaStreamSynchronize)."""
+    import workloads_device as wd
+    from hierarchicalkv_amd import EvictStrategy, HashTable, default_options
+
+    dev = wd.DEV
+    n, dim, calls = 1024, 8, 2000
+    keys = wd.dev_keys(7, 0, n)
+    vals = torch.zeros(n, dim, dtype=torch.float32, device=dev)
+    out = torch.zeros(n, dim, dtype=torch.float32, device=dev)
+    founds = torch.zeros(n, dtype=torch.bool, device=dev)
+    side = torch.cuda.Stream()
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    rows = []
+
+    def table(api_lock):
+        t = HashTable()
+        t.init(default_options(init_capacity=1 << 16, max_capacity=1 << 16, dim=dim, max_hbm_for_vectors=1 << 30,
+                               api_lock=api_lock, evict_strategy=EvictStrategy.kLru))
+        t.insert_or_assign(n, keys, vals)
+        torch.cuda.synchronize()
+        return t
+
+    def per_call(fn):
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        host = (time.perf_counter() - t0) / calls
+        torch.cuda.synchronize()
+        total = (time.perf_counter() - t0) / calls
+        return host * 1e6, total * 1e6
+
+    t = table(False)
+    rows.append(("api_lock off, one stream", *per_call(lambda: t.find(n, keys, out, founds))))
+    t.close()
+    t = table(True)
+    rows.append(("group lock as built, one stream", *per_call(lambda: t.find(n, keys, out, founds))))
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    state = [0]
+
+    def two_streams():
+        state[0] ^= 1
+        if state[0]:
+            t.find(n, keys, out, founds, stream=s1)
+        else:
+            t.insert_or_assign(n, keys, vals, stream=s2)
+    rows.append(("group lock as built, find on one stream and insert_or_assign on another in turn", *per_call(two_streams)))
+
+    def blocking():
+        with torch.cuda.stream(side):
+            flag.add_(1)          # stands for the lock kernel <<<1,1>>>
+        side.synchronize()        # the host waits for it, as group_lock.cuh:146-166 does
+        t.find(n, keys, out, founds)
+    rows.append(("host-blocking acquisition before every call (as the reference)", *per_call(blocking)))
+    t.close()
+    print("| lock | host time per call, us | wall time per call incl. the GPU work, us |")
+    print("|---|---|---|")
+    for name, host, total in rows:
+        print("| %s | %.1f | %.1f |" % (name, host, total), flush=True)
+    print(json.dumps({"group_lock": [{"lock": r[0], "host_us": round(r[1], 2), "wall_us": round(r[2], 2)} for r in rows]}))
 
 
 PROFILE_GROUPS = [

@@ -69,9 +69,16 @@ bool ispow2(uint64_t x) { return x && !(x & (x - 1)); }
  * The reference blocks the host on a one-thread kernel per call; here the
  * exclusion is expressed between streams with events, so a call never waits on
  * the host: begin() makes `stream` wait for the conflicting work already
- * enqueued on other streams, end() remembers that `stream` now carries work of
- * this role.  Work on one stream is ordered by the stream itself, so a table
- * that is only ever used from one stream records and waits on nothing.
+ * enqueued on other streams, end() publishes what the call has just enqueued.
+ *
+ * A stream is only ever touched inside a call that was made on it (the caller
+ * may destroy it right afterwards).  While the table has seen one stream, the
+ * stream's own order is all that is needed and nothing is recorded.  When a
+ * second stream turns up, the device is synchronised once (the first stream may
+ * be gone by then); from then on every call records one event on its own
+ * stream in end(), and begin() waits for the events of the conflicting roles.
+ * Entries whose event has completed are dropped, so streams that come and go
+ * leave nothing behind.
  */
 class StreamGroupLock {
  public:
@@ -79,24 +86,35 @@ class StreamGroupLock {
 
   ~StreamGroupLock() {
     for (auto& r : roles_)
-      for (auto& kv : r) (void)hipEventDestroy(kv.second.ev);
+      for (auto& kv : r) (void)hipEventDestroy(kv.second);
+    for (hipEvent_t e : spare_) (void)hipEventDestroy(e);
   }
 
   hipError_t begin(Role role, hipStream_t s) {
     mu_.lock();
     hipError_t e = hipSuccess;
-    for (int other = 0; other < 3 && e == hipSuccess; other++) {
-      if (!conflicts(role, (Role)other)) continue;
-      for (auto& kv : roles_[other]) {
-        if (kv.first == s) continue;
-        Entry& en = kv.second;
-        if (en.dirty) {
-          e = hipEventRecord(en.ev, kv.first);
-          if (e != hipSuccess) break;
-          en.dirty = false;
+    if (!multi_) {
+      if (!seen_one_) {
+        seen_one_ = true;
+        only_ = s;
+      } else if (s != only_) {
+        /* everything the first stream carries is complete after this, whether or not the
+         * stream still exists */
+        e = hipDeviceSynchronize();
+        multi_ = true;
+      }
+    } else {
+      for (int other = 0; other < 3 && e == hipSuccess; other++) {
+        const bool clash = conflicts(role, (Role)other);
+        for (auto it = roles_[other].begin(); it != roles_[other].end() && e == hipSuccess;) {
+          if (hipEventQuery(it->second) == hipSuccess) { /* done: nobody needs to wait for it */
+            spare_.push_back(it->second);
+            it = roles_[other].erase(it);
+            continue;
+          }
+          if (clash && it->first != s) e = hipStreamWaitEvent(s, it->second, 0);
+          ++it;
         }
-        e = hipStreamWaitEvent(s, en.ev, 0);
-        if (e != hipSuccess) break;
       }
     }
     if (e != hipSuccess) mu_.unlock();
@@ -105,34 +123,25 @@ class StreamGroupLock {
 
   hipError_t end(Role role, hipStream_t s) {
     hipError_t e = hipSuccess;
-    auto it = roles_[role].find(s);
-    if (it == roles_[role].end()) {
-      Entry en;
-      e = hipEventCreateWithFlags(&en.ev, hipEventDisableTiming);
-      if (e == hipSuccess) {
-        en.dirty = true;
-        roles_[role].emplace(s, en);
+    if (multi_) {
+      auto it = roles_[role].find(s);
+      if (it == roles_[role].end()) {
+        hipEvent_t ev = nullptr;
+        if (!spare_.empty()) {
+          ev = spare_.back();
+          spare_.pop_back();
+        } else {
+          e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+        }
+        if (e == hipSuccess) it = roles_[role].emplace(s, ev).first;
       }
-    } else {
-      it->second.dirty = true;
+      if (e == hipSuccess) e = hipEventRecord(it->second, s);
     }
     mu_.unlock();
     return e;
   }
 
-  /* counts of streams carrying unpublished work per role (tests) */
-  int pending(Role role) {
-    std::lock_guard<std::mutex> g(mu_);
-    int c = 0;
-    for (auto& kv : roles_[role]) c += kv.second.dirty;
-    return c;
-  }
-
  private:
-  struct Entry {
-    hipEvent_t ev;
-    bool dirty;
-  };
   /* Updaters on different streams are ordered among themselves as well (the reference
    * lets them overlap and pays a slot lock per key for it): an updater that is alone on
    * the table needs no slot locks. */
@@ -142,7 +151,10 @@ class StreamGroupLock {
     return a != b;
   }
   std::mutex mu_;
-  std::map<hipStream_t, Entry> roles_[3];
+  bool seen_one_ = false, multi_ = false;
+  hipStream_t only_ = nullptr;
+  std::map<hipStream_t, hipEvent_t> roles_[3]; /* last event of each stream in each role */
+  std::vector<hipEvent_t> spare_;
 };
 
 }  // namespace

@@ -10,6 +10,8 @@
 #include <random>
 #include <set>
 #include <unordered_set>
+#include <thread>
+#include <atomic>
 #include <vector>
 
 #include "merlin_hashtable.cuh"
@@ -60,6 +62,15 @@ struct EraseIfPredFunctor {
   }
 };
 
+
+template <class Kt, class St>
+struct MatchNothing {
+  __forceinline__ __device__ bool operator()(const Kt&, St&, const Kt&, const St&) { return false; }
+};
+template <class Kt, class St>
+struct MatchEverything {
+  __forceinline__ __device__ bool operator()(const Kt&, St&, const Kt&, const St&) { return true; }
+};
 
 /* Functors of the tile-cooperative forms, shaped like the ones the reference's tests
  * hand to erase_if_v2 / export_batch_if_v2 / for_each
@@ -592,6 +603,75 @@ static void test_growth_and_key_locks() {
 }
 
 
+/* The calls whose kernels are compiled in the caller's translation unit (size_if, erase_if,
+ * export_batch_if) take the table's layout while they hold their role in the group lock: other
+ * host threads that make the table grow meanwhile (which frees the old arrays) must not pull
+ * the arrays away under a kernel that is about to be launched.  Four threads insert into a
+ * table that grows 64-fold, two keep counting and erasing (a predicate that matches nothing)
+ * on streams of their own. */
+static void test_header_templates_beside_growth() {
+  constexpr size_t DIM = 8, INIT = 1 << 12, MAX = 1 << 18, N = 1024, ROUNDS = 40, WRITERS = 4;
+  HashTableOptions o;
+  o.init_capacity = INIT;
+  o.max_capacity = MAX;
+  o.dim = DIM;
+  o.max_load_factor = 0.5f;
+  o.max_hbm_for_vectors = GB(1);
+  using Table = HashTable<K, V, S, EvictStrategy::kLru>;
+  Table table;
+  table.init(o);
+  std::atomic<int> writers_left{(int)WRITERS};
+  std::atomic<int> failures{0};
+  std::atomic<long> counted{0};
+  auto writer = [&](int tid) {
+    try {
+      hipStream_t st;
+      HIP(hipStreamCreate(&st));
+      DevBuf<K> dk(N);
+      DevBuf<V> dv(N * DIM);
+      for (size_t r = 0; r < ROUNDS; r++) {
+        std::vector<K> keys(N);
+        for (size_t i = 0; i < N; i++) keys[i] = (K)((((uint64_t)tid * ROUNDS + r) * N + i) * 2654435761ull + 17);
+        dk.up(keys);
+        dv.up(values_of(keys, DIM));
+        table.insert_or_assign(N, dk.p, dv.p, nullptr, st);
+        HIP(hipStreamSynchronize(st));
+      }
+      HIP(hipStreamDestroy(st));
+    } catch (const std::exception& e) {
+      std::printf("writer %d: %s\n", tid, e.what());
+      failures++;
+    }
+    writers_left--;
+  };
+  auto counter = [&](int tid) {
+    try {
+      hipStream_t st;
+      HIP(hipStreamCreate(&st));
+      size_t before = 0;
+      while (writers_left.load() > 0) {
+        const size_t now = table.template size_if<MatchEverything>(0, 0, st);
+        if (now < before || now > WRITERS * ROUNDS * N) failures++;  // keys are never lost or invented
+        before = now;
+        if (table.template erase_if<MatchNothing>(0, 0, st) != 0) failures++;
+        counted++;
+      }
+      HIP(hipStreamDestroy(st));
+    } catch (const std::exception& e) {
+      std::printf("counter %d: %s\n", tid, e.what());
+      failures++;
+    }
+  };
+  std::vector<std::thread> th;
+  for (size_t w = 0; w < WRITERS; w++) th.emplace_back(writer, (int)w);
+  for (int c = 0; c < 2; c++) th.emplace_back(counter, c);
+  for (auto& x : th) x.join();
+  CHECK(failures.load() == 0);
+  CHECK(counted.load() > 0);
+  CHECK(table.capacity() > INIT);
+  CHECK(table.size() == WRITERS * ROUNDS * N);
+}
+
 template <size_t DIM>
 static void run_functor_forms() {
   constexpr size_t CAP = 1 << 14, N = 6000;
@@ -1075,6 +1155,7 @@ int main() {
     test_allocator_hybrid_and_checkpoint();
     test_option_checks();
     test_growth_and_key_locks();
+    test_header_templates_beside_growth();
     test_functor_forms();
     test_dual_bucket_mode();
     test_uint32_scores();
