@@ -338,6 +338,60 @@ def test_hybrid_mode(oracle):
     t.close()
 
 
+def test_hybrid_batch_is_some_serial_order(oracle):
+    """Where hybrid mode differs from the reference.  The reference's hybrid upsert holds every
+    slot lock of a batch from its lock kernel to its write kernel (upsert.cuh:1350-1595), so an
+    absent key never takes the slot of another key of its own batch: each takes the lowest-scored
+    resident that is still visible.  The fused kernel here releases a slot as soon as its key is
+    in, so a later key of the batch may evict an earlier one, exactly as if the keys had been
+    handed over one call at a time.  On a one-bucket table with a batch whose scores interleave
+    with the lowest resident scores: the GPU's result must be what the oracle gives for some
+    order of one-key calls (all 120 orders are tried), and it is not what the reference's batch
+    model gives (there the key with score 105 stays, because its slot is invisible to the scans
+    of the later keys of the batch; one key at a time it always loses the slot again)."""
+    import itertools
+    dim = 4
+    opts = default_options(init_capacity=128, max_capacity=128, dim=dim, max_hbm_for_vectors=0,
+                           evict_strategy=EvictStrategy.kCustomized)
+    keys = w.unique_keys(311, 0, 128)
+    vals = w.values_from_keys(keys, dim)
+    sc = np.arange(100, 100 + 10 * 128, 10, dtype=np.uint64)
+    batch = w.unique_keys(312, 0, 5)
+    bvals = w.values_from_keys(batch, dim)
+    bsc = np.array([105, 200, 115, 125, 99], np.uint64)
+
+    def resident_map(table):
+        ek, _, es = table.export_all()
+        return frozenset(zip(ek.tolist(), es.tolist()))
+
+    serial = set()
+    for order in itertools.permutations(range(5)):
+        o = oracle.OracleTable(opts, hybrid=True)
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+        for i in order:
+            o.insert_or_assign(batch[i:i + 1], bytes_of(bvals[i:i + 1]), bsc[i:i + 1])
+        serial.add(resident_map(o))
+        o.close()
+    ref = oracle.OracleTable(opts, hybrid=True)
+    ref.insert_or_assign(keys, bytes_of(vals), sc)
+    ref.insert_or_assign(batch, bytes_of(bvals), bsc)
+    batch_model = resident_map(ref)
+    ref.close()
+    assert batch_model not in serial
+
+    t = HashTable()
+    t.init(opts)
+    assert not t.is_pure_hbm()
+    t.insert_or_assign(128, dev(keys), dev(vals), dev(sc))
+    t.insert_or_assign(5, dev(batch), dev(bvals), dev(bsc))
+    gk, gv, gs = export_table(t, dim * 4)
+    assert frozenset(zip(gk.tolist(), gs.tolist())) in serial
+    allv = {int(k): v for k, v in zip(np.concatenate([keys, batch]), np.concatenate([bytes_of(vals), bytes_of(bvals)]))}
+    assert all((gv[i] == allv[int(k)]).all() for i, k in enumerate(gk))  # every resident carries its own row
+    assert t.size() == 128
+    t.close()
+
+
 def test_io_by_cpu(oracle):
     """io_by_cpu (merlin_hashtable.cuh:1275-1292, 1820-1841, 2175-2192, 2414-2431): all rows in
     pinned host memory, host threads move the rows of insert_or_assign, find_or_insert, assign
