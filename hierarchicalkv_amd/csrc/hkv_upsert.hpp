@@ -21,8 +21,10 @@
  *            lanes: the digest probe (hkv_lookup.hpp), the min-score scan of a
  *            full bucket (16 scores per lane, 8 coalesced 128-byte lines per
  *            tile, reduce inside the lane and then over the tile) and the
- *            value-row copies, each issued for several keys before the first
- *            result is awaited.
+ *            value-row copies, issued for several keys before the first result
+ *            is awaited.  How much is in flight per wavefront is weighed
+ *            against registers: at 118 registers four wavefronts share a SIMD,
+ *            and that is worth more here than deeper batches per wavefront.
  *
  * Lock discipline on a SIMD machine: every lock taken in a trip of the retry
  * loop is released at the end of the same trip, and the loop's exit test is a
@@ -278,8 +280,7 @@ __device__ __forceinline__ uint32_t first_from(uint64_t lo, uint64_t hi, uint32_
 }
 
 /*
- * Min-score scan of a bucket by the 8 lanes of a tile, split in two so that
- * the loads of two buckets can be in flight before either is reduced.
+ * Min-score scan of a bucket by the 8 lanes of a tile: the loads, then the reduction.
  * Lane j holds scores {16 it + 2j, 16 it + 2j + 1 : it = 0..7}: each `it` is
  * one coalesced 128-byte line per tile.  LOCKED_RULE hides slots whose key is
  * LOCKED or EMPTY (find_ptr_or_insert.cuh:170-180).
@@ -349,6 +350,12 @@ __device__ __forceinline__ void scan_reduce(const View& v, const uint64_t* sc, c
   }
 }
 
+/* 16-byte units of value rows a lane holds in registers at a time in the bulk copies.  Fewer
+ * means fewer row loads in flight per wavefront but also fewer registers, i.e. more wavefronts
+ * per SIMD; measured on insert_or_assign (rows of 256 bytes): 16 units 0.323 ms, 8 units
+ * 0.306 ms per 2^20 keys. */
+constexpr int kRowUnits = 8;
+
 /*
  * Bulk row traffic of one trip.  Round q of a tile is the key owned by lane q
  * of the tile: `move` says what to do with it, `tab` is its table row, `usr`
@@ -362,7 +369,7 @@ template <int VEC, int UPL, bool CAN_READ_TABLE, bool CAN_ACCUM>
 __device__ __forceinline__ void bulk_rows(int move, uint8_t* tab, uint8_t* usr,
                                           uint32_t units, int value_kind, int lane) {
   using T = typename VecType<VEC>::type;
-  constexpr int kGroup = (16 / UPL) < kTile ? (16 / UPL) : kTile;
+  constexpr int kGroup = kRowUnits / UPL < 1 ? 1 : (kRowUnits / UPL < kTile ? kRowUnits / UPL : kTile);
   const int j = lane & (kTile - 1);
   const int lane_base = lane & ~(kTile - 1);
   for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
@@ -420,7 +427,7 @@ template <int VEC, int UPL>
 __device__ __forceinline__ void bulk_evicted(int kind, const uint8_t* src, uint8_t* dst,
                                              uint32_t units, int lane) {
   using T = typename VecType<VEC>::type;
-  constexpr int kGroup = (16 / UPL) < kTile ? (16 / UPL) : kTile;
+  constexpr int kGroup = kRowUnits / UPL < 1 ? 1 : (kRowUnits / UPL < kTile ? kRowUnits / UPL : kTile);
   const int j = lane & (kTile - 1);
   const int lane_base = lane & ~(kTile - 1);
   for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
@@ -600,7 +607,9 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
-    /* ---- step 2: full buckets: min-score scan by the tile, two buckets in flight ------------ */
+    /* ---- step 2: full buckets: min-score scan by the tile, one bucket after the other ------------
+     * (two buckets in flight per tile took 32 more registers and with them a wavefront per
+     * SIMD: 0.308 against 0.323 ms per 2^20 keys) */
     uint64_t best = kMaxScore;
     uint32_t bpos = 0;
     {
@@ -610,25 +619,16 @@ upsert_kernel(View v, UpsertArgs a) {
         if (need) {
           const int r0 = __ffs(need) - 1;
           need &= need - 1;
-          const int r1 = need ? __ffs(need) - 1 : r0;
-          need &= need - 1; /* no-op when need is already 0 */
           const uint64_t bs0 = __shfl((unsigned long long)bslot, lane_base + r0);
-          const uint64_t bs1 = __shfl((unsigned long long)bslot, lane_base + r1);
-          uint64_t sc0[2 * kTile], sc1[2 * kTile];
-          uint64_t kc0[LOCKED_RULE ? 2 * kTile : 1], kc1[LOCKED_RULE ? 2 * kTile : 1];
+          uint64_t sc0[2 * kTile];
+          uint64_t kc0[LOCKED_RULE ? 2 * kTile : 1];
           scan_load<LOCKED_RULE>(v, bs0, j, sc0, kc0);
-          if (r1 != r0) scan_load<LOCKED_RULE>(v, bs1, j, sc1, kc1);
-          uint64_t b0, b1 = kMaxScore;
-          uint32_t p0, p1 = 0;
+          uint64_t b0;
+          uint32_t p0;
           scan_reduce<LOCKED_RULE>(v, sc0, kc0, j, b0, p0);
-          if (r1 != r0) scan_reduce<LOCKED_RULE>(v, sc1, kc1, j, b1, p1);
           if (j == r0) {
             best = b0;
             bpos = p0;
-          }
-          if (r1 != r0 && j == r1) {
-            best = b1;
-            bpos = p1;
           }
         }
       }
