@@ -152,8 +152,8 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
   }
 }
 
-/* the writers' probes (upsert and assign families) */
-constexpr bool kTwoStepWriters = false;
+/* the writers' probes (upsert and assign families): they move rows, like find */
+constexpr bool kTwoStepWriters = true;
 
 /* the 16 digest bytes of lane j of a tile, read past the caches */
 __device__ __forceinline__ uint4 ld_digests16(const View& v, uint32_t bkt, int j) {
