@@ -277,7 +277,7 @@ def main():
         "insert_or_assign": {"ms": round(ups_avg, 4), "bkvs": round(n / (ups_avg * 1e-3) / 1e9, 4),
                              "bkvs_2p30": round(n / (ups_avg * 1e-3) / 2**30, 4)},
         "roofline": {"kernel": "upsert_kernel<insert_or_assign>" if path == "locked" else
-                     "two-phase upsert: upsert_hits_kernel + bin_* + grouped_miss_kernel", "bound": "hbm",
+                     "two-phase upsert: upsert_hits_kernel + chained_miss_kernel", "bound": "hbm",
                      "achieved": round(ups_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": ups_traffic,
                      "bytes_per_key": upsert_bytes(vb, 0.5)},
@@ -727,7 +727,7 @@ def summarize_profiles(root):
                 col(r, "TCC_EA0_WRREQ_64B_sum", 1e-6), part, col(r, "TCC_EA0_ATOMIC_sum", 1e-6)))
         o.append("\n## Wavefronts, LDS, vector memory, address translation\n")
         o.append("Registers per lane: twice rocprofv3's VGPR_Count field, which counts register pairs on this part (the "
-                 "compiler's resource report for the same kernels reads 114 and 182 registers, allocated as 120 and 184).\n")
+                 "compiler's resource report for the same kernels reads 114 and 118 registers, both allocated as 120).\n")
         o.append("| call | wavefronts | vector registers per lane | LDS bytes per workgroup | scratch | occupancy % of the maximum | vector memory reads "
                  "/ writes (M instructions) | L1 -> L2 read / write requests (M) | returning atomics (M) | L1 TLB misses (M) | "
                  "LDS instructions (M) | LDS bank-conflict cycles (M) |\n|---|---|---|---|---|---|---|---|---|---|---|---|")
