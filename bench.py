@@ -1064,6 +1064,9 @@ CEILING_PATTERNS = [
     ("find_pattern_1line", "find's accesses, one key line per key, no logic (algorithmic bytes)", "GB/s"),
     ("find_pattern", "find's accesses, 1.44 key lines per key (false digest matches), no logic "
                      "(algorithmic bytes)", "GB/s"),
+    ("find_pattern_chained", "find's accesses, 1.1 key lines per key, each group of addresses known only when the "
+                             "group before has arrived (batch key -> digest line -> key word -> row), no logic "
+                             "(algorithmic bytes)", "GB/s"),
     ("upsert_pattern", "insert_or_assign's accesses, 50 % absent keys into full buckets, no locks, no logic "
                        "(algorithmic bytes)", "GB/s"),
     ("upsert_pattern_locks", "the same plus the slot-lock protocol's atomics, re-reads and unlock stores "

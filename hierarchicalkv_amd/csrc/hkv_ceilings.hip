@@ -2,7 +2,8 @@
  * Memory-system ceilings for the table kernels: kernels that issue the access pattern of
  * find and of insert_or_assign at a given table shape with no table logic in them (no
  * hashing of real keys, no comparisons, no dependent loads: every address is a function of
- * the thread index and a salt), plus the plain streaming, gather, scatter and small-access
+ * the thread index and a salt; one variant of find's pattern chains its four groups of loads
+ * as the real kernel has to), plus the plain streaming, gather, scatter and small-access
  * rates the patterns are made of.  What such a kernel takes is what the memory system
  * needs for the bytes alone; the distance of a real kernel from it is what its logic and its
  * dependent round trips cost.
@@ -111,11 +112,23 @@ __global__ void k_row_scatter(Shape sh, Buffers b, uint64_t salt) {
  * digest line (8 lanes x 16 bytes), one 8-byte key word of the table (a whole line of
  * traffic), a second one for `extra_pm` keys in 1000 (false digest matches), the row (row_bytes)
  * gathered and written to the dense output, one found flag. */
+/* zero, but only known once `x` has arrived: makes an address depend on a load */
+__device__ __forceinline__ uint32_t zero_after(uint32_t x) {
+  uint32_t z;
+  asm volatile("v_and_b32 %0, 0, %1" : "=v"(z) : "v"(x));
+  return z;
+}
+
+/* CHAIN: the same accesses, but each group of addresses is only known when the group before
+ * it has arrived, as in the real kernel (key of the batch -> digest line -> key word of the
+ * table -> row): four round trips in a row instead of one. */
+template <bool CHAIN>
 __global__ void __launch_bounds__(64)
 k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
   const int lane = threadIdx.x, tile = lane >> 3, j = lane & 7;
   const uint64_t base = (uint64_t)blockIdx.x * 64;
   uint64_t acc = b.in_keys[base + lane];
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   /* digest lines: tile t reads the lines of keys 8t..8t+7 */
   uint4 dg[8];
 #pragma unroll
@@ -125,6 +138,7 @@ k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
   }
 #pragma unroll
   for (int r = 0; r < 8; r++) acc += dg[r].x ^ dg[r].w;
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   /* key words: lane L verifies key L */
   {
     const uint64_t h = mix(base + lane + salt);
@@ -135,6 +149,7 @@ k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
   }
   if (acc == 0x123456789ULL) *b.sink = 1;
   b.flags[base + lane] = 1;
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   /* rows: 64 rows x units spread over the 64 lanes, loads before stores */
   const uint32_t upr = sh.row_bytes / 16;
   const uint32_t total = upr * 64;
@@ -410,7 +425,11 @@ int hkv_ceilings_run(const char* name, int reps, double* ms, double* bytes) {
       /* 0.44 extra key lines per key: 127 other slots / 256 digest values, 7 of 8 of them in
        * another 128-byte key line; "_1line": exactly one key line per key */
       const uint32_t extra = !strcmp(name, "find_pattern") ? 440 : 0;
-      hipLaunchKernelGGL(k_find_pattern, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, extra);
+      hipLaunchKernelGGL(k_find_pattern<false>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, extra);
+      moved = (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1);
+    } else if (!strcmp(name, "find_pattern_chained")) {
+      /* 1.1 key lines per key, what the two-step verification fetches */
+      hipLaunchKernelGGL(k_find_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u);
       moved = (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1);
     } else if (!strcmp(name, "upsert_pattern") || !strcmp(name, "upsert_pattern_locks")) {
       const int locks = !strcmp(name, "upsert_pattern_locks");

@@ -24,6 +24,8 @@
 #ifndef HKV_LOOKUP_HPP_
 #define HKV_LOOKUP_HPP_
 
+#include <type_traits>
+
 #include "hkv_common.hpp"
 
 namespace hkv {
@@ -72,11 +74,12 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
   /* TWO_STEP: candidates are verified in two steps.  An 8-byte key load costs a whole
    * 128-byte line of memory traffic, a key that is present has one true candidate, and a
    * false 8-bit match turns up in every second bucket: so step 1 fetches only the
-   * candidates of the first lane of the tile that has any (a lane's 16 slots share one key
-   * line), and the other lanes' candidates are fetched in step 2 only for the keys step 1
-   * did not find: 1.27 key lines per key that is present instead of 1.44.  It pays where the
-   * kernel is bound by bytes (find with its rows); a kernel that moves little besides the
-   * probe is bound by its dependent round trips and takes all candidates at once. */
+   * candidates of one lane of the tile (a lane's 16 slots share one key line), the one
+   * where the key most likely is, and the other lanes' candidates are fetched in step 2
+   * only for the keys step 1 did not find: 1.03 to 1.27 key lines per key that is present
+   * (keys that went into a free slot / into a victim's slot) instead of 1.44.  The lookups
+   * and the kernels that move rows use it; erase and lock_keys, which move little besides
+   * the probe and are bound by their dependent round trips, take all candidates at once. */
   uint32_t cm[kTile];    /* this lane's digest matches, bw order */
   uint32_t later[kTile]; /* lanes of the tile whose candidates wait for step 2 */
   uint64_t k0[kTile], k1[kTile];
@@ -89,7 +92,13 @@ __device__ __forceinline__ void probe_wave(const View& v, const KeyMeta* s_meta,
       s_em[tile * kTile + r][j] =
           (uint16_t)(valid ? match16_natural(dg[r], v.empty_digest * 0x01010101u) : 0u);
     const uint32_t lanes = TWO_STEP ? tile_ballot(cm[r] != 0, tile) : 0u;
-    later[r] = lanes & (lanes - 1);
+    /* step 1 takes the first lane with a candidate at or after the lane of the key's start
+     * slot, going round: an insert takes the first free slot from there (the reference's
+     * probe order, kernel_utils.cuh:636-643), so that is where the key most likely is */
+    const uint32_t sl = inf[r] >> 20; /* start slot / 16 */
+    const uint32_t turned = ((lanes >> sl) | (lanes << (kTile - sl))) & 0xFFu;
+    const uint32_t first = (uint32_t)(__ffs(turned) - 1 + sl) & (kTile - 1);
+    later[r] = lanes & ~(1u << first);
     const uint64_t* kb = v.keys + (uint64_t)bkt[r] * kBucketSize + j * 16;
     k0[r] = v.empty_key;
     k1[r] = v.empty_key;
@@ -272,12 +281,12 @@ lookup_kernel(View v, FindArgs a) {
   if (DUAL) restage_first_bucket(v, s_meta, lane);
   if (WAVES > 1 && threadIdx.x == 0) s_missed[0] = 0;
   __syncthreads();
-  probe_wave<false, MODE == kLookupValues>(v, s_meta, s_slot, nullptr, nullptr, lane);
+  probe_wave<false, true>(v, s_meta, s_slot, nullptr, nullptr, lane);
   __syncthreads();
   if (DUAL) {
     restage_second_bucket(v, s_meta, s_slot, lane);
     __syncthreads();
-    probe_wave<false, MODE == kLookupValues>(v, s_meta, s_slot, nullptr, nullptr, lane);
+    probe_wave<false, true>(v, s_meta, s_slot, nullptr, nullptr, lane);
     __syncthreads();
   }
 
@@ -323,6 +332,64 @@ lookup_kernel(View v, FindArgs a) {
   const uint32_t total = units * kWave;
   const bool pow2 = (units & (units - 1)) == 0;
   const uint32_t sh = 31 - __clz(units);
+  if constexpr (VEC == 16) {
+    /* Rows of 16 to 1024 bytes whose size is a power of two, all in HBM, slot numbers below
+     * 2^32 (every decision here is the same for the whole wavefront): lane L then always
+     * moves unit L mod units of a row, and in pass b the row of key (L / units) + b * (64 /
+     * units), so the slot numbers are read from LDS in one go and an address costs one
+     * multiply-add.  The general form below spends more instructions on addresses than
+     * the memory system needs time for the rows. */
+    if (pow2 && units <= kWave && v.hbm_slots >= v.capacity && v.capacity <= 0xFFFFFFFFull) {
+      constexpr int kB = 16;
+      const uint32_t c = lane & (units - 1);
+      const uint32_t kk0 = lane >> sh;
+      const uint32_t kstep = kWave >> sh;
+      const uint8_t* const src0 = v.values + c * 16;
+      uint8_t* const dst0 = a.out_values + (base + kk0) * v.value_bytes + c * 16;
+      const uint64_t dstep = (uint64_t)kstep * v.value_bytes;
+      /* with all 64 keys found nothing below is conditional, and the stores start as the
+       * first rows arrive instead of after the last one */
+      const bool all = __ballot(my_slot >= 0) == ~0ull;
+      auto move = [&](auto all_found) {
+        constexpr bool ALL = decltype(all_found)::value;
+        for (uint32_t b0 = 0; b0 < units; b0 += kB) {
+          int64_t sl[kB];
+          u32x4_t buf[kB];
+          if (ALL && units >= kB) {
+#pragma unroll
+            for (int b = 0; b < kB; b++) sl[b] = s_slot[kk0 + (b0 + b) * kstep];
+#pragma unroll
+            for (int b = 0; b < kB; b++)
+              buf[b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
+                  src0 + (uint64_t)(uint32_t)sl[b] * v.value_bytes));
+#pragma unroll
+            for (int b = 0; b < kB; b++)
+              __builtin_nontemporal_store(buf[b],
+                                          reinterpret_cast<u32x4_t*>(dst0 + (b0 + b) * dstep));
+          } else {
+#pragma unroll
+            for (int b = 0; b < kB; b++)
+              sl[b] = b0 + b < units ? s_slot[kk0 + (b0 + b) * kstep] : -1;
+#pragma unroll
+            for (int b = 0; b < kB; b++)
+              if (sl[b] >= 0)
+                buf[b] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
+                    src0 + (uint64_t)(uint32_t)sl[b] * v.value_bytes));
+#pragma unroll
+            for (int b = 0; b < kB; b++)
+              if (sl[b] >= 0)
+                __builtin_nontemporal_store(buf[b],
+                                            reinterpret_cast<u32x4_t*>(dst0 + (b0 + b) * dstep));
+          }
+        }
+      };
+      if (all)
+        move(std::true_type{});
+      else
+        move(std::false_type{});
+      return;
+    }
+  }
   constexpr int kBatch = VEC == 16 ? 16 : 4;
   for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
     T buf[kBatch];
