@@ -577,7 +577,29 @@ PROFILE_GROUPS = [
            "SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR"),
     ("tcp", "--kernel-trace --pmc TCP_TCC_READ_REQ_sum TCP_TCC_WRITE_REQ_sum TCP_TCC_ATOMIC_WITH_RET_REQ_sum "
             "TCP_UTCL1_TRANSLATION_MISS_sum"),
+    ("lat", "--kernel-trace --pmc TCP_TCC_READ_REQ_LATENCY_sum TCP_TCC_READ_REQ_sum TCP_PENDING_STALL_CYCLES_sum "
+            "SQ_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_SALU SQ_WAVE_CYCLES SQ_WAIT_ANY"),
 ]
+
+# the part these figures are taken on: SQ_BUSY_CYCLES is summed over the shader engines
+N_SHADER_ENGINES = 32
+N_CUS = 256
+
+
+def in_flight_row(label, c):
+    """Row of the requests-in-flight table from one kernel's counters of the `lat` group."""
+    busy = c["SQ_BUSY_CYCLES"] / N_SHADER_ENGINES
+    reqs = max(1.0, c["TCP_TCC_READ_REQ_sum"])
+    lat = c["TCP_TCC_READ_REQ_LATENCY_sum"]
+    return "| %s | %.2f | %.0f | %.1f | %.2f | %.1f | %.1f | %.2f |" % (
+        label, reqs / 1e6, lat / reqs, lat / busy / N_CUS, c["TCP_PENDING_STALL_CYCLES_sum"] / N_CUS / busy,
+        c["SQ_INSTS_VALU"] / 1e6, c["SQ_INSTS_SALU"] / 1e6, c["SQ_WAIT_ANY"] / max(1.0, c["SQ_WAVE_CYCLES"]))
+
+
+IN_FLIGHT_HEAD = (
+    "| kernel | L1 -> L2 read requests (M) | average latency of one (cycles) | of them in flight per CU | share of the run "
+    "in which a CU's L1 has its pending-request queue full | vector instructions (M) | scalar instructions (M) | "
+    "share of wavefront time spent waiting |\n|---|---|---|---|---|---|---|---|")
 # kernels of bench.py --ops, in the order of its table: (substring of the kernel name, call, algorithmic bytes per key)
 OPS_KERNELS = [
     ("lookup_kernel<0, 16", "find (100 % hit)", 657),
@@ -739,6 +761,17 @@ def summarize_profiles(root):
                 col(r, "TCP_TCC_WRITE_REQ_sum", 1e-6), col(r, "TCP_TCC_ATOMIC_WITH_RET_REQ_sum", 1e-6),
                 col(r, "TCP_UTCL1_TRANSLATION_MISS_sum", 1e-6), col(r, "SQ_INSTS_LDS", 1e-6),
                 col(r, "SQ_LDS_BANK_CONFLICT", 1e-6)))
+        lat_by, _ = groups["lat"]
+        if lat_by:
+            o.append("\n## Read requests in flight\n")
+            o.append("What bounds these kernels is the number of read requests a CU keeps in flight and how long one "
+                     "takes: latency sum / busy cycles (SQ_BUSY_CYCLES is summed over the %d shader engines of the "
+                     "part, %d CUs).\n" % (N_SHADER_ENGINES, N_CUS))
+            o.append(IN_FLIGHT_HEAD)
+            for needle, call, _ in kernels:
+                kk = pick(lat_by, needle)
+                if kk:
+                    o.append(in_flight_row(call, {c: last(v, take, call) for c, v in lat_by[kk].items()}))
         if tag == "bench":
             stats = csv_of(tag, "trace", "kernel_stats")
             if stats:
@@ -750,6 +783,44 @@ def summarize_profiles(root):
                             r["Name"].split("(")[0].replace("void ", "").replace("hkv::", ""), r["Calls"],
                             float(r["AverageNs"]) / 1e3, float(r["MinNs"]) / 1e3, float(r["MaxNs"]) / 1e3, r["Percentage"]))
         path = os.path.join(ROOT, "profiles", fname)
+        with open(path, "w") as f:
+            f.write("\n".join(o) + "\n")
+        print("wrote", path)
+    dur = durations("ceil")
+    lat_by, _ = counters("ceil", "lat")
+    if dur and lat_by:
+        reps = 21  # launches per pattern: one untimed, twenty timed
+        # kernel, which of its launches (patterns run in the order of CEILING_PATTERNS), label
+        rows = [("k_stream_read", (1, reps), "stream_read"),
+                ("k_row_gather", (1, reps), "row_gather"),
+                ("k_find_pattern<false>", (reps + 1, 2 * reps), "find_pattern (1.44 key lines)"),
+                ("k_find_pattern<true>", (1, reps), "find_pattern_chained, launched behind itself"),
+                ("k_find_pattern<true>", (2 * reps + 1, 3 * reps), "the same in the step (step_find)"),
+                ("k_upsert_pattern<false>", (reps + 1, 2 * reps), "upsert_pattern_locks"),
+                ("k_upsert_pattern<true>", (1, reps), "upsert_pattern_chained, launched behind itself"),
+                ("k_upsert_pattern<true>", (3 * reps + 1, 4 * reps), "the same in the step (step_upsert)")]
+        o = ["# rocprofv3: the no-logic pattern kernels of bench.py --ceilings\n",
+             "Workload: capacity 2^26, dim 64 fp32, batch 2^20; one MI355X.  Commands, from the repository root after "
+             "`cd /tmp && export TMPDIR=/tmp && cd -`:\n",
+             "    rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof/ceil_trace -o out -- python3 bench.py --ceilings",
+             "    rocprofv3 %s --output-format csv -d gpurun_out/prof/ceil_lat -o out -- python3 bench.py --ceilings" % dict(PROFILE_GROUPS)["lat"],
+             "    python3 bench.py --profile-summary gpurun_out/prof\n",
+             "Averages over the named launches of each kernel (the counter run serialises kernels: its durations are "
+             "not used).  Compare with the same table for the product kernels in "
+             "lookup_kernel_upsert_kernel_cap2p26_dim64_batch2p20.md.\n",
+             "| kernel | avg us (trace) | L1 -> L2 read requests (M) | average latency of one (cycles) | of them in flight per CU | "
+             "share of the run in which a CU's L1 has its pending-request queue full | vector instructions (M) | scalar "
+             "instructions (M) | share of wavefront time spent waiting |\n|---|---|---|---|---|---|---|---|---|"]
+        for needle, (lo, hi), label in rows:
+            kd, kl = pick(dur, needle), pick(lat_by, needle)
+            if not kd or not kl:
+                continue
+            us = dur[kd][lo:hi]
+            c = {name: sum(v[lo:hi]) / max(1, len(v[lo:hi])) for name, v in lat_by[kl].items()}
+            if not us or not c.get("SQ_BUSY_CYCLES"):
+                continue
+            o.append(in_flight_row("%s | %.1f" % (label, sum(us) / len(us)), c))
+        path = os.path.join(ROOT, "profiles", "ceiling_kernels_cap2p26_dim64_batch2p20.md")
         with open(path, "w") as f:
             f.write("\n".join(o) + "\n")
         print("wrote", path)
@@ -1071,6 +1142,13 @@ CEILING_PATTERNS = [
                        "(algorithmic bytes)", "GB/s"),
     ("upsert_pattern_locks", "the same plus the slot-lock protocol's atomics, re-reads and unlock stores "
                              "(algorithmic bytes)", "GB/s"),
+    ("upsert_pattern_chained", "upsert_pattern_locks with 1.1 key lines per key and every group of addresses known "
+                               "only when the group before has arrived (batch key -> digest line -> key word and "
+                               "compare-and-swap -> score scan -> exchange and score re-read -> stores -> unlock)", "GB/s"),
+    ("step_pattern", "find_pattern_chained, then upsert_pattern_chained on other keys: the benchmark's step "
+                     "(algorithmic bytes of both)", "GB/s"),
+    ("step_find", "the find half of step_pattern, timed launch by launch", "GB/s"),
+    ("step_upsert", "the insert_or_assign half of step_pattern, timed launch by launch", "GB/s"),
     ("small_load8", "8-byte loads, one per random 128-byte line", "G ops/s"),
     ("small_store8", "8-byte write-through stores, one per random line", "G ops/s"),
     ("small_store1", "1-byte write-through stores, one per random line", "G ops/s"),

@@ -183,11 +183,16 @@ k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
  * `locks` adds what the slot-lock protocol spends: a compare-and-swap and an unlock store per
  * present key, an exchange and a score re-read per absent key (the key store of an absent
  * key doubles as its unlock). */
+template <bool CHAIN>
 __global__ void __launch_bounds__(64)
 k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int locks) {
   const int lane = threadIdx.x, tile = lane >> 3, j = lane & 7;
   const uint64_t base = (uint64_t)blockIdx.x * 64;
   uint64_t acc = b.in_keys[base + lane];
+  /* CHAIN: as in k_find_pattern, every group of addresses waits for the group before it:
+   * batch key -> digest line -> key word (and compare-and-swap) -> score scan -> exchange
+   * and score re-read -> stores -> unlock */
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   uint4 dg[8];
 #pragma unroll
   for (int r = 0; r < 8; r++) {
@@ -196,10 +201,11 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
   }
 #pragma unroll
   for (int r = 0; r < 8; r++) acc += dg[r].x ^ dg[r].w;
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   const uint64_t h = mix(base + lane + salt);
   const uint64_t bk = h & (sh.buckets - 1);
   const uint32_t p = (uint32_t)(h >> 40) & 127u;
-  const uint64_t slot = bk * 128 + p;
+  uint64_t slot = bk * 128 + p;
   const bool absent = lane & 1;
   acc += b.keys[slot];
   if ((uint32_t)((h >> 48) % 1000) < extra_pm) acc += b.keys[bk * 128 + ((p + 64) & 127u)];
@@ -211,6 +217,7 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
       acc += expect;
     }
   }
+  if (CHAIN) salt += zero_after((uint32_t)acc);
   /* score scans of the absent keys: keys 8t+1, 8t+3, 8t+5, 8t+7 of each tile, two in flight */
 #pragma unroll
   for (int r = 1; r < 8; r += 4) {
@@ -227,9 +234,16 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
 #pragma unroll
       for (int it = 0; it < 8; it++) acc += sc[w][it].x ^ sc[w][it].z;
   }
+  if (CHAIN) slot += zero_after((uint32_t)acc);
   if (locks && absent) {
     acc += __hip_atomic_exchange(b.keys + slot, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (CHAIN) slot += zero_after((uint32_t)acc);
     acc += __hip_atomic_load(b.scores + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (CHAIN) {
+    const uint32_t z = zero_after((uint32_t)acc);
+    slot += z;
+    salt += z;
   }
   if (acc == 0x123456789ULL) *b.sink = 1;
   /* metadata stores */
@@ -401,6 +415,39 @@ int hkv_ceilings_run(const char* name, int reps, double* ms, double* bytes) {
   CK(hipEventCreate(&e0));
   CK(hipEventCreate(&e1));
   double moved = 0;
+  /* "step_find" / "step_upsert": the two halves of the benchmark's step, launched in turn,
+   * one of them timed launch by launch */
+  const bool step_find = !strcmp(name, "step_find"), step_upsert = !strcmp(name, "step_upsert");
+  if (step_find || step_upsert) {
+    /* three events per step and no synchronisation inside the run, as the benchmark times
+     * its own steps */
+    hipEvent_t* ev = new hipEvent_t[3 * (reps + 1)];
+    for (int q = 0; q < 3 * (reps + 1); q++) CK(hipEventCreate(&ev[q]));
+    for (int rep = 0; rep <= reps; rep++) {
+      const uint64_t salt = (uint64_t)rep * 0x9E3779B97F4A7C15ULL + 12345;
+      CK(hipEventRecord(ev[3 * rep], 0));
+      hipLaunchKernelGGL(k_find_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u);
+      CK(hipEventRecord(ev[3 * rep + 1], 0));
+      hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, ~salt, 100u, 1);
+      CK(hipEventRecord(ev[3 * rep + 2], 0));
+      CK(hipGetLastError());
+    }
+    CK(hipDeviceSynchronize());
+    double sum = 0;
+    for (int rep = 1; rep <= reps; rep++) {
+      float t = 0;
+      CK(hipEventElapsedTime(&t, ev[3 * rep + (step_find ? 0 : 1)], ev[3 * rep + (step_find ? 1 : 2)]));
+      sum += t;
+    }
+    for (int q = 0; q < 3 * (reps + 1); q++) CK(hipEventDestroy(ev[q]));
+    delete[] ev;
+    CK(hipEventDestroy(e0));
+    CK(hipEventDestroy(e1));
+    *ms = sum / reps;
+    *bytes = step_find ? (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1)
+                       : (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
+    return 0;
+  }
   for (int rep = 0; rep <= reps; rep++) {
     const uint64_t salt = (uint64_t)rep * 0x9E3779B97F4A7C15ULL + 12345;
     if (rep == 1) CK(hipEventRecord(e0, 0));
@@ -431,9 +478,19 @@ int hkv_ceilings_run(const char* name, int reps, double* ms, double* bytes) {
       /* 1.1 key lines per key, what the two-step verification fetches */
       hipLaunchKernelGGL(k_find_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u);
       moved = (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1);
+    } else if (!strcmp(name, "upsert_pattern_chained")) {
+      hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 1);
+      moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
+    } else if (!strcmp(name, "step_pattern")) {
+      /* the benchmark's step: a find and an insert_or_assign on other keys, one after the
+       * other, so that each finds the caches as the other left them */
+      hipLaunchKernelGGL(k_find_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u);
+      hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, ~salt, 100u, 1);
+      moved = (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1) +
+              (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
     } else if (!strcmp(name, "upsert_pattern") || !strcmp(name, "upsert_pattern_locks")) {
       const int locks = !strcmp(name, "upsert_pattern_locks");
-      hipLaunchKernelGGL(k_upsert_pattern, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 440u,
+      hipLaunchKernelGGL(k_upsert_pattern<false>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 440u,
                          locks);
       /* half present (161 + 2 row), half absent into a full bucket (1185 + 2 row) */
       moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
