@@ -1131,3 +1131,70 @@ def test_every_row_moving_call_with_odd_and_long_rows(oracle, row_bytes):
     for i in np.flatnonzero(of)[:: 53]:
         assert np.array_equal(read_device(int(gp[i]), row_bytes), ov[i])
     t.close()
+
+
+def test_one_digest_for_a_whole_bucket(oracle):
+    """Every key of a bucket carries the same digest byte, so every probe sees 128 candidates,
+    16 per lane of its tile: the candidate order (the lane of the key's start slot first), the
+    second step, the second candidate of a lane and the loop over the rest are all taken, by
+    readers and writers alike.  Two buckets, 300 such keys: fill, find (present and absent),
+    find*, contains, erase and insert again, insert_and_evict, all against the oracle."""
+    dim = 4
+    t, o, _ = make_pair(oracle, init_capacity=256, max_capacity=256, dim=dim,
+                        evict_strategy=EvictStrategy.kCustomized)
+    cand = w.unique_keys(901, 0, 1 << 17)
+    dig = np.array([oracle.locate(int(k), 2)[2] for k in cand[:1 << 17]], np.uint8)
+    same = cand[dig == dig[0]][:300]
+    assert len(same) == 300
+    vals = w.values_from_keys(same, dim)
+    sc = np.arange(1000, 1300, dtype=np.uint64)
+
+    def check_lookups(q):
+        n = len(q)
+        out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        f = torch.zeros(n, dtype=torch.bool, device=DEV)
+        s = torch.zeros(n, dtype=torch.int64, device=DEV)
+        t.find(n, dev(q), out, f, s)
+        p = torch.zeros(n, dtype=torch.int64, device=DEV)
+        f2 = torch.zeros(n, dtype=torch.bool, device=DEV)
+        t.find_ptr(n, dev(q), p, f2)
+        c = torch.zeros(n, dtype=torch.bool, device=DEV)
+        t.contains(n, dev(q), c)
+        torch.cuda.synchronize()
+        ov, of, osc = o.find(q)
+        gf = f.cpu().numpy()
+        assert (gf == of).all() and (f2.cpu().numpy() == of).all() and (c.cpu().numpy() == of).all()
+        assert (bytes_of(out.cpu().numpy())[of] == ov[of]).all()
+        assert (host_u64(s)[of] == osc[of]).all()
+        return int(of.sum())
+
+    # 200 keys into 256 slots (free slots everywhere), then 100 more: the buckets fill up and evict
+    t.insert_or_assign(200, dev(same[:200]), dev(vals[:200]), dev(sc[:200]))
+    o.insert_or_assign(same[:200], bytes_of(vals[:200]), sc[:200])
+    assert check_lookups(same) == 200
+    assert_same_table(t, o, dim * 4)
+    t.insert_or_assign(100, dev(same[200:]), dev(vals[200:]), dev(sc[200:]))
+    o.insert_or_assign(same[200:], bytes_of(vals[200:]), sc[200:])
+    assert t.size() == o.size() == 256
+    assert check_lookups(same) == 256
+    assert_same_table(t, o, dim * 4)
+    # erase every third resident key, look again, put some back with new rows
+    gone = np.ascontiguousarray(same[44::3][:60])
+    t.erase(len(gone), dev(gone))
+    o.erase(gone)
+    assert t.size() == o.size()
+    check_lookups(same)
+    back = np.concatenate([gone[:30], same[:10]])
+    bv = w.uniform_values(902, 0, len(back), dim)
+    bs_ = np.arange(2000, 2000 + len(back), dtype=np.uint64)
+    t.insert_or_assign(len(back), dev(back), dev(bv), dev(bs_))
+    o.insert_or_assign(back, bytes_of(bv), bs_)
+    check_lookups(same)
+    assert_same_table(t, o, dim * 4)
+    # assign on present and absent keys of the same digest
+    av = w.uniform_values(903, 0, 300, dim)
+    as_ = np.arange(3000, 3300, dtype=np.uint64)
+    t.assign(300, dev(same), dev(av), dev(as_))
+    o.assign(same, bytes_of(av), as_)
+    assert_same_table(t, o, dim * 4)
+    t.close()
