@@ -606,11 +606,11 @@ OPS_KERNELS = [
     ("lookup_kernel<1, 16", "find* (100 % hit)", 153),
     ("lookup_kernel<2, 16", "contains (100 % hit)", 145),
     ("assign_kernel<16, 2, true>", "assign (100 % hit)", 673),
-    ("upsert_kernel<0, 16, 2, false>", "insert_or_assign (50 % new)", 1185),
-    ("upsert_kernel<2, 16, 2, false>", "find_or_insert (50 % new)", 1189),
-    ("upsert_kernel<4, 16, 1, false>", "find_or_insert* (50 % new)", 689),
-    ("upsert_kernel<1, 16, 2, false>", "insert_and_evict (50 % new)", 1449),
-    ("upsert_kernel<3, 16, 2, false>", "accum_or_assign (50 % new)", 1314),
+    ("upsert_kernel<0, 16, 2, false", "insert_or_assign (50 % new)", 1185),
+    ("upsert_kernel<2, 16, 2, false", "find_or_insert (50 % new)", 1189),
+    ("upsert_kernel<4, 16, 1, false", "find_or_insert* (50 % new)", 689),
+    ("upsert_kernel<1, 16, 2, false", "insert_and_evict (50 % new)", 1449),
+    ("upsert_kernel<3, 16, 2, false", "accum_or_assign (50 % new)", 1314),
     ("export_if_kernel", "export_batch_if (2^20 slots, all match)", 544),
     ("erase_kernel<true>", "erase (100 % hit)", 165),
 ]
@@ -667,7 +667,7 @@ def summarize_profiles(root):
     traffic = {"workload": "capacity 2^26, dim 64 fp32, batch 2^20, LRU, load factor 1.0", "kernels": {}}
     for tag, cmd, take, kernels, fname, title in [
         ("bench", "python3 bench.py --steps 4 --warmup 1 --no-cpu-baseline --calibrate", 3,
-         [("lookup_kernel<0, 16", "find (100 % hit)", 657), ("upsert_kernel<0, 16, 2, false>", "insert_or_assign (50 % new)", 1185)],
+         [("lookup_kernel<0, 16", "find (100 % hit)", 657), ("upsert_kernel<0, 16, 2, false", "insert_or_assign (50 % new)", 1185)],
          "lookup_kernel_upsert_kernel_cap2p26_dim64_batch2p20.md",
          "lookup_kernel (find) and upsert_kernel (insert_or_assign) on the benchmark's workload"),
         ("ops", "python3 bench.py --ops", 6, OPS_KERNELS, "all_entry_points_cap2p26_dim64_batch2p20.md",
@@ -798,7 +798,8 @@ def summarize_profiles(root):
                 ("k_find_pattern<true>", (2 * reps + 1, 3 * reps), "the same in the step (step_find)"),
                 ("k_upsert_pattern<false>", (reps + 1, 2 * reps), "upsert_pattern_locks"),
                 ("k_upsert_pattern<true>", (1, reps), "upsert_pattern_chained, launched behind itself"),
-                ("k_upsert_pattern<true>", (3 * reps + 1, 4 * reps), "the same in the step (step_upsert)")]
+                ("k_upsert_pattern<true>", (reps + 1, 2 * reps), "upsert_pattern_bounds, launched behind itself"),
+                ("k_upsert_pattern<true>", (4 * reps + 1, 5 * reps), "upsert_pattern_chained in the step (step_upsert)")]
         o = ["# rocprofv3: the no-logic pattern kernels of bench.py --ceilings\n",
              "Workload: capacity 2^26, dim 64 fp32, batch 2^20; one MI355X.  Commands, from the repository root after "
              "`cd /tmp && export TMPDIR=/tmp && cd -`:\n",
@@ -1145,6 +1146,8 @@ CEILING_PATTERNS = [
     ("upsert_pattern_chained", "upsert_pattern_locks with 1.1 key lines per key and every group of addresses known "
                                "only when the group before has arrived (batch key -> digest line -> key word and "
                                "compare-and-swap -> score scan -> exchange and score re-read -> stores -> unlock)", "GB/s"),
+    ("upsert_pattern_bounds", "upsert_pattern_chained with the bucket's 8 score bounds (64 bytes) and one score line "
+                              "read per absent key instead of all 8 lines, and one more 8-byte store", "GB/s"),
     ("step_pattern", "find_pattern_chained, then upsert_pattern_chained on other keys: the benchmark's step "
                      "(algorithmic bytes of both)", "GB/s"),
     ("step_find", "the find half of step_pattern, timed launch by launch", "GB/s"),

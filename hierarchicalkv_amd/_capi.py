@@ -67,6 +67,7 @@ class TableView(C.Structure):
         ("pow2_buckets", C.c_uint8),
         ("dual_bucket", C.c_uint8),
         ("pad_", C.c_uint8 * 4),
+        ("bounds", C.c_void_p),
     ]
 
 
@@ -121,6 +122,7 @@ SIGNATURES = {
     "hkv_lock_begin": (_i, [_T, _i, _p]),
     "hkv_lock_end": (_i, [_T, _i, _p]),
     "hkv_set_clock": (_i, [_T, _i, _u64]),
+    "hkv_scores_changed": (_i, [_T]),
 }
 
 

@@ -218,7 +218,28 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
     }
   }
   if (CHAIN) salt += zero_after((uint32_t)acc);
-  /* score scans of the absent keys: keys 8t+1, 8t+3, 8t+5, 8t+7 of each tile, two in flight */
+  /* score scans of the absent keys: keys 8t+1, 8t+3, 8t+5, 8t+7 of each tile, two in flight;
+   * with score bounds (locks == 2): the bucket's 8 bounds (64 bytes), then one score line */
+  if (locks == 2) {
+    uint64_t bd[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const uint64_t bk2 = mix(base + tile * 8 + 2 * w + 1 + salt) & (sh.buckets - 1);
+      bd[w] = reinterpret_cast<const uint64_t*>(b.digests)[bk2 * 8 + j];
+    }
+#pragma unroll
+    for (int w = 0; w < 4; w++) acc += bd[w];
+    if (CHAIN) salt += zero_after((uint32_t)acc);
+    uint4 ln[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const uint64_t h2 = mix(base + tile * 8 + 2 * w + 1 + salt);
+      const uint64_t bk2 = h2 & (sh.buckets - 1);
+      ln[w] = *reinterpret_cast<const uint4*>(b.scores + bk2 * 128 + ((h2 >> 40) & 7) * 16 + j * 2);
+    }
+#pragma unroll
+    for (int w = 0; w < 4; w++) acc += ln[w].x ^ ln[w].z;
+  } else
 #pragma unroll
   for (int r = 1; r < 8; r += 4) {
     uint4 sc[2][8];
@@ -251,6 +272,7 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
   if (absent) {
     st1_wt(b.digests + slot, (uint8_t)acc);
     st8_wt(b.keys + slot, acc);
+    if (locks == 2) st8_wt(reinterpret_cast<uint64_t*>(b.digests) + (slot >> 4), acc);
   }
   /* rows: dense input -> table rows, 64 rows x units over the 64 lanes */
   const uint32_t upr = sh.row_bytes / 16;
@@ -480,6 +502,9 @@ int hkv_ceilings_run(const char* name, int reps, double* ms, double* bytes) {
       moved = (double)n * (8 + 128 + 8 + 2.0 * sh.row_bytes + 1);
     } else if (!strcmp(name, "upsert_pattern_chained")) {
       hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 1);
+      moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
+    } else if (!strcmp(name, "upsert_pattern_bounds")) {
+      hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 2);
       moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
     } else if (!strcmp(name, "step_pattern")) {
       /* the benchmark's step: a find and an insert_or_assign on other keys, one after the

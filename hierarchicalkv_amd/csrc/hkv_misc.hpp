@@ -10,8 +10,8 @@
 namespace hkv {
 
 /* initialize_buckets (core_kernels.cuh:169-292) and clear_kernel (:656-676) in
- * one grid-wide fill: key = EMPTY, digest = EMPTY marker, size = 0; scores are
- * zeroed only at creation (clear leaves scores and values as they are).
+ * one grid-wide fill: key = EMPTY, digest = EMPTY marker, size = 0, score bounds = 0; scores
+ * are zeroed only at creation (clear leaves scores and values as they are).
  * One thread per 16 slots. */
 __global__ void __launch_bounds__(256)
 fill_kernel(View v, int zero_scores) {
@@ -28,6 +28,7 @@ fill_kernel(View v, int zero_scores) {
 #pragma unroll
       for (int q = 0; q < 16; q++) s[q] = 0;
     }
+    v.bounds[t] = 0; /* one per 16 slots */
   }
   if (t < v.buckets_num) v.sizes[t] = 0;
 }
@@ -73,6 +74,7 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
     if (erased) {
       v.digests[slot] = v.reclaim_digest;
       v.scores[slot] = 0;
+      v.bounds[slot >> 4] = 0; /* the one place where a score goes down: its line's bound follows */
     }
   }
   const uint32_t bkt = erased ? (uint32_t)(slot >> 7) : 0xFFFFFFFFu;

@@ -166,7 +166,9 @@ struct hkv_table {
   bool pure_hbm;
   bool own_alloc;
   hkv_allocator alloc;
-  void* d_meta;          /* digests + keys + scores + sizes in one arena */
+  void* d_meta;          /* digests + keys + scores + sizes + score bounds in one arena */
+  bool score_bounds;     /* LRU upserts search victims through the score bounds (HKV_SCORE_BOUNDS=0: off) */
+  std::atomic<bool> bounds_stale{false}; /* a call may have written scores below the bounds */
   uint64_t meta_bytes;
   void* d_values;        /* value rows in HBM */
   void* h_values;        /* host address of the pinned value rows (hybrid) */
@@ -186,6 +188,8 @@ struct hkv_table {
   bool keys_may_be_locked; /* LOCKED key words may sit in the table (lock_keys, the pointer
                               overload with locked_key_ptrs), until the count below reads 0 */
   bool locked_recount;     /* unlock_keys has run since the count was last read */
+  unsigned long long* d_bound_caps; /* two device words: clock readings of the last calls that used the score bounds, used in turn */
+  unsigned bound_cap_turn = 0;
   unsigned long long* d_locked; /* device word: slots left LOCKED by those calls, less the unlocked */
   bool dual;               /* TableMode::kMemory: two candidate buckets per key */
   bool io_by_cpu;          /* value rows of the writers are moved by host threads */
@@ -313,10 +317,13 @@ int accum_unit(uint32_t value_bytes, const void* p, int kind) {
   return unit >= (int)elem[kind] ? unit : 0;
 }
 
-template <int OP, bool LOCKED_RULE>
+/* BOUNDS: the victim search reads the bucket's score bounds and one or two of its score lines
+ * instead of all eight (hkv_upsert.hpp); for 16-byte units, which is what tables with rows of a
+ * multiple of 16 bytes use. */
+template <int OP, bool LOCKED_RULE, bool BOUNDS = false>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
-  if constexpr (OP == kOpAccumOrAssign) {
+  if constexpr (OP == kOpAccumOrAssign && !BOUNDS) {
     /* the two units that only the element-wise add needs */
     if (vec == 8) {
       hipLaunchKernelGGL((upsert_kernel<OP, 8, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
@@ -328,20 +335,21 @@ void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
     }
   }
   if (OP == kOpFindOrInsertPtr) {
-    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE>), grid, block, 0, s, v, a);
+    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a);
     return;
   }
   if (vec == 16) {
     switch (pick_upl(v.value_bytes, 16)) {
-      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE>), grid, block, 0, s, v, a); break;
-      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE>), grid, block, 0, s, v, a); break;
-      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE>), grid, block, 0, s, v, a); break;
-      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE>), grid, block, 0, s, v, a); break;
+      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
+      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
+      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
+      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
     }
-  } else if (vec == 4) {
-    hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
-  } else {
-    hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+  } else if constexpr (!BOUNDS) {
+    if (vec == 4)
+      hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+    else
+      hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
   }
 }
 
@@ -518,7 +526,7 @@ int sync_clock(hkv_table* t) {
       t->clock.offset = t0 + (t1 - t0) / 2 - (uint64_t)ticks * t->clock.ns_per_tick;
     }
   }
-  HKV_HIP(hipMemset(d, 0, (kCounterWords + 1) * sizeof(unsigned long long)));
+  HKV_HIP(hipMemset(d, 0, (kCounterWords + 3) * sizeof(unsigned long long)));
   return HKV_SUCCESS;
 }
 
@@ -544,18 +552,20 @@ int alloc_arenas(hkv_table* t, uint64_t buckets_num, View& v, TableMem& m) {
   v.buckets_num = buckets_num;
   v.capacity = buckets_num * kBucketSize;
   v.pow2_buckets = ispow2(buckets_num);
-  /* metadata arena: digests | keys | scores | sizes, each 256-byte aligned */
+  /* metadata arena: digests | keys | scores | sizes | score bounds, each 256-byte aligned */
   auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
   const uint64_t off_keys = up(v.capacity);
   const uint64_t off_scores = off_keys + up(v.capacity * 8);
   const uint64_t off_sizes = off_scores + up(v.capacity * 8);
-  m.meta_bytes = off_sizes + up(v.buckets_num * 4);
+  const uint64_t off_bounds = off_sizes + up(v.buckets_num * 4);
+  m.meta_bytes = off_bounds + up(v.buckets_num * 8 * sizeof(uint64_t));
   HKV_TRY(table_alloc(t, 0, &m.d_meta, m.meta_bytes));
   uint8_t* base = (uint8_t*)m.d_meta;
   v.digests = base;
   v.keys = (uint64_t*)(base + off_keys);
   v.scores = (uint64_t*)(base + off_scores);
   v.sizes = (int32_t*)(base + off_sizes);
+  v.bounds = (uint64_t*)(base + off_bounds);
   /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
    * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
   const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
@@ -689,6 +699,8 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   a.value_kind = t->opts.value_kind;
   const bool refuse_equal = OP == kOpFindOrInsertPtr || (hybrid_rule && !t->pure_hbm);
   a.refuse_equal = refuse_equal;
+  /* scores that do not come from the table's clock may be lower than what the bounds say */
+  if (a.strategy != t->opts.evict_strategy) t->bounds_stale = true;
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
@@ -709,6 +721,24 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
        * no such slot the plain scan finds the same victims (a slot locked by another key of
        * the batch is retried instead of skipped) */
       launch_upsert<OP, true>(vec, t->view, a, s);
+    } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr)) {
+      /* LRU scores only grow, which is what keeps the score bounds right by themselves */
+      if (t->bounds_stale.exchange(false)) {
+        const uint64_t words = t->view.buckets_num * 8 * 2;
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((words / 4 + 255) / 256)), dim3(256), 0, s,
+                           (uint32_t*)t->view.bounds, words);
+      }
+      /* No bound may be above a score that this call writes.  Deterministic clock: the call's
+       * scores start at its base.  Hardware clock: they are later than the start of the last
+       * call of this kind, which that call left in a device word (this one leaves its own in
+       * the other word). */
+      a.bound_cap = t->clock.base;
+      if (t->clock.mode == 0) {
+        a.bound_cap_in = t->d_bound_caps + (t->bound_cap_turn & 1);
+        a.bound_cap_out = t->d_bound_caps + ((t->bound_cap_turn + 1) & 1);
+        t->bound_cap_turn++;
+      }
+      launch_upsert<OP, false, true>(vec, t->view, a, s);
     } else {
       launch_upsert<OP, false>(vec, t->view, a, s);
     }
@@ -1051,6 +1081,10 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
    * one per find + insert_or_assign step), "auto" = two-phase for large batches,
    * "grouped" = two-phase whenever it is possible (tests) */
   t->upsert_path = 1;
+  {
+    const char* b = getenv("HKV_SCORE_BOUNDS");
+    t->score_bounds = !(b && !strcmp(b, "0"));
+  }
   if (const char* e = getenv("HKV_UPSERT_PATH")) {
     if (!strcmp(e, "auto")) t->upsert_path = 0;
     if (!strcmp(e, "locked")) t->upsert_path = 1;
@@ -1137,12 +1171,13 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->pure_hbm = v.hbm_slots == v.capacity;
   void* cnt = nullptr;
   {
-    int rc = table_alloc(t, 0, &cnt, (kCounterWords + 1) * sizeof(unsigned long long));
+    int rc = table_alloc(t, 0, &cnt, (kCounterWords + 3) * sizeof(unsigned long long));
     if (rc) return bail(rc);
   }
   t->d_counters = (unsigned long long*)cnt;
   for (unsigned w = 0; w < kCounterWords; w++) t->counter_free.push_back(w);
   t->d_locked = t->d_counters + kCounterWords;
+  t->d_bound_caps = t->d_counters + kCounterWords + 1;
   {
     int rc = sync_clock(t);
     if (rc) return bail(rc);
@@ -1275,6 +1310,7 @@ int hkv_insert_or_assign_noalloc(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.clock = t->clock;
   a.value_kind = t->opts.value_kind;
   a.refuse_equal = !t->pure_hbm; /* the lock-key rule of hybrid mode, as hkv_insert_or_assign */
+  if (a.strategy != t->opts.evict_strategy) t->bounds_stale = true;
   const int vec = pick_vec(t->view.value_bytes, {values});
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
@@ -1861,6 +1897,12 @@ int hkv_set_clock(hkv_table* t, int mode, uint64_t base) {
   if (mode != 0 && mode != 1) return fail(HKV_ERROR_ARGUMENT, "bad clock mode %d", mode);
   t->clock.mode = (uint32_t)mode;
   t->clock.base = base;
+  t->bounds_stale = true; /* the new clock may be behind the old one */
+  return HKV_SUCCESS;
+}
+
+int hkv_scores_changed(hkv_table* t) {
+  t->bounds_stale = true;
   return HKV_SUCCESS;
 }
 

@@ -68,6 +68,11 @@ struct UpsertArgs {
   int32_t strategy; /* hkv_evict_strategy; uniform, so a scalar branch */
   int32_t refuse_equal; /* refuse when score <= min instead of < (hybrid and
                            pointer kernels, upsert.cuh:1524, find_or_insert.cuh:1593) */
+  /* score bounds (BOUNDS kernels): no bound is set above `bound_cap`, or above *bound_cap_in
+   * when that is given; the kernel leaves a clock reading in *bound_cap_out for the next call */
+  uint64_t bound_cap;
+  const unsigned long long* bound_cap_in;
+  unsigned long long* bound_cap_out;
 };
 
 /* ScoreFunctor<Strategy>::desired_when_missed, kernel_utils.cuh:275-279,
@@ -350,6 +355,83 @@ __device__ __forceinline__ void scan_reduce(const View& v, const uint64_t* sc, c
   }
 }
 
+/* ---- min-score search with per-line lower bounds (LRU) -------------------------------------------
+ * v.bounds holds, for every line of 16 scores, a value that is not above any score in the line.
+ * Under LRU a score only ever grows (a touched or new key gets the current time), so a bound
+ * that was right once stays right without anybody maintaining it, and 0 is always right.  The
+ * tile reads the bucket's 8 bounds (64 bytes), then only the score line with the lowest bound:
+ * if that line's minimum is not above any other line's bound it is the bucket's minimum, found
+ * with 2 line reads instead of 8.  Otherwise the lines whose bound is below the best score so
+ * far are opened one by one (and their bounds set to what they hold).  The result is the slot a
+ * scan of all 128 scores returns (ties to the lowest slot).
+ * "Only grows" holds from call to call, not inside one: keys of one batch get their scores in no
+ * particular order.  So no bound is ever set above `cap`, a value no score of the running call
+ * is below (the base of the deterministic clock, or a clock reading from before the call). */
+
+/* the two scores of lane j in line g of the bucket at slot `bs` */
+__device__ __forceinline__ uint4 line_load(const View& v, uint64_t bs, uint32_t g, int j) {
+  const uint64_t at = bs + g * 16 + j * 2;
+  if (v.capacity < (UINT64_C(1) << 29)) return ld_u128_at(v.scores, v.capacity * 8, at * 8);
+  const uint64_t a = ld_u64(v.scores + at), b = ld_u64(v.scores + at + 1);
+  return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
+}
+/* minimum of line g over the tile: score and slot position in the bucket */
+__device__ __forceinline__ void line_min(const uint4& x, uint32_t g, int j, uint64_t& m, uint32_t& pos) {
+  const uint64_t s0 = x.x | ((uint64_t)x.y << 32), s1 = x.z | ((uint64_t)x.w << 32);
+  const uint32_t p0 = g * 16 + j * 2;
+  m = s1 < s0 ? s1 : s0;
+  pos = s1 < s0 ? p0 + 1 : p0;
+#pragma unroll
+  for (int off = 1; off < kTile; off <<= 1) {
+    const uint64_t om = __shfl_xor(m, off);
+    const uint32_t op = __shfl_xor(pos, off);
+    if (om < m || (om == m && op < pos)) {
+      m = om;
+      pos = op;
+    }
+  }
+}
+/* `bd`: this lane's bound (line j); `g`, `x`: the line with the lowest bound and this lane's
+ * part of it.  All 8 lanes of the tile call this together.  `nb`: what line bpos / 16 is bounded
+ * by once slot bpos has been given a score that is above everything else in it. */
+__device__ __forceinline__ void bounded_min(const View& v, uint64_t bs, int tile, int j, uint64_t bd,
+                                            uint32_t g, uint4 x, uint64_t cap, uint64_t& best,
+                                            uint32_t& bpos, uint64_t& nb) {
+  uint64_t* const bounds = v.bounds + (bs >> 4);
+  line_min(x, g, j, best, bpos);
+  uint32_t opened = 1u << g;
+  for (;;) {
+    const bool lower = !((opened >> j) & 1u) && (bd < best || (bd == best && (uint32_t)j < (bpos >> 4)));
+    const uint32_t cand = tile_ballot(lower, tile);
+    if (!cand) break;
+    const uint32_t c = (uint32_t)__ffs(cand) - 1;
+    opened |= 1u << c;
+    const uint4 y = line_load(v, bs, c, j);
+    uint64_t m;
+    uint32_t pos;
+    line_min(y, c, j, m, pos);
+    if (m < best || (m == best && pos < bpos)) {
+      /* the line that held the best so far is bounded by exactly that */
+      if ((uint32_t)j == (bpos >> 4)) st_u64(bounds + j, best < cap ? best : cap);
+      best = m;
+      bpos = pos;
+      x = y;
+    } else if ((uint32_t)j == c) {
+      st_u64(bounds + c, m < cap ? m : cap);
+    }
+  }
+  /* the smallest score of the chosen line apart from the chosen slot */
+  const uint64_t s0 = x.x | ((uint64_t)x.y << 32), s1 = x.z | ((uint64_t)x.w << 32);
+  const uint32_t p0 = (bpos & ~15u) + j * 2;
+  const uint64_t r0 = p0 == bpos ? kMaxScore : s0, r1 = p0 + 1 == bpos ? kMaxScore : s1;
+  nb = r1 < r0 ? r1 : r0;
+#pragma unroll
+  for (int off = 1; off < kTile; off <<= 1) {
+    const uint64_t o = __shfl_xor(nb, off);
+    if (o < nb) nb = o;
+  }
+}
+
 /* 16-byte units of value rows a lane holds in registers at a time in the bulk copies.  Fewer
  * means fewer row loads in flight per wavefront but also fewer registers, i.e. more wavefronts
  * per SIMD; measured on insert_or_assign (rows of 256 bytes): 16 units 0.323 ms, 8 units
@@ -520,9 +602,11 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * the plain scan would pick and wait for without end.  Whether a key is
  * refused at score == min is a separate switch (UpsertArgs::refuse_equal).
  */
-template <int OP, int VEC, int UPL, bool LOCKED_RULE>
+template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false>
 __global__ void __launch_bounds__(kWave)
+    __attribute__((amdgpu_waves_per_eu(BOUNDS && OP != kOpAccumOrAssign ? 4 : 1)))
 upsert_kernel(View v, UpsertArgs a) {
+  static_assert(!(BOUNDS && LOCKED_RULE), "the bounded search does not look at key words");
   __shared__ KeyMeta s_meta[kWave];
   __shared__ int64_t s_slot[kWave];
   __shared__ __attribute__((aligned(16))) uint16_t s_em[kWave][kTile];
@@ -533,6 +617,11 @@ upsert_kernel(View v, UpsertArgs a) {
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
 
+  uint64_t bound_cap = 0;
+  if constexpr (BOUNDS) {
+    bound_cap = a.bound_cap_in ? *a.bound_cap_in : a.bound_cap;
+    if (a.bound_cap_out && blockIdx.x == 0 && lane == 0) *a.bound_cap_out = now_ns(a.clock, 0);
+  }
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
   s_unsure[lane] = 0;
@@ -612,7 +701,55 @@ upsert_kernel(View v, UpsertArgs a) {
      * SIMD: 0.308 against 0.323 ms per 2^20 keys) */
     uint64_t best = kMaxScore;
     uint32_t bpos = 0;
-    {
+    uint64_t new_bound = 0;
+    if constexpr (BOUNDS) {
+      /* the bounds of four buckets, then the most promising score line of each, in flight */
+      const uint32_t need = tile_ballot(want_scan, tile);
+      const int lane_base = lane & ~(kTile - 1);
+#pragma unroll
+      for (int h = 0; h < kTile; h += 4) {
+        if (!__ballot(((need >> h) & 0xFu) != 0)) continue;
+        uint64_t bs[4], bd[4];
+        uint32_t g[4];
+        uint4 x[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          bs[q] = __shfl((unsigned long long)bslot, lane_base + h + q);
+          bd[q] = kMaxScore;
+          if ((need >> (h + q)) & 1u) bd[q] = ld_u64(v.bounds + (bs[q] >> 4) + j);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          uint64_t b = bd[q];
+          uint32_t gi = (uint32_t)j;
+#pragma unroll
+          for (int off = 1; off < kTile; off <<= 1) {
+            const uint64_t ob = __shfl_xor(b, off);
+            const uint32_t og = __shfl_xor(gi, off);
+            if (ob < b || (ob == b && og < gi)) {
+              b = ob;
+              gi = og;
+            }
+          }
+          g[q] = gi;
+          x[q] = make_uint4(0, 0, 0, 0);
+          if ((need >> (h + q)) & 1u) x[q] = line_load(v, bs[q], g[q], j);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          if ((need >> (h + q)) & 1u) {
+            uint64_t b0, nb0;
+            uint32_t p0;
+            bounded_min(v, bs[q], tile, j, bd[q], g[q], x[q], bound_cap, b0, p0, nb0);
+            if (j == h + q) {
+              best = b0;
+              bpos = p0;
+              new_bound = nb0;
+            }
+          }
+        }
+      }
+    } else {
       uint32_t need = tile_ballot(want_scan, tile);
       const int lane_base = lane & ~(kTile - 1);
       for (unsigned long long more = __ballot(need != 0); more; more = __ballot(need != 0)) {
@@ -701,6 +838,10 @@ upsert_kernel(View v, UpsertArgs a) {
       if (a.locked_key_ptrs) a.locked_key_ptrs[i] = locked ? v.keys + slot : nullptr;
     }
     if (commit) {
+      /* a victim's slot gets a score of this call: what bounds its line now is the lowest of
+       * the line's other scores */
+      if (BOUNDS && (got == kStEvict || got == kStReclaimed))
+        st_u64(v.bounds + (slot >> 4), new_bound < bound_cap ? new_bound : bound_cap);
       write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
       if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
     }

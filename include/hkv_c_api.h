@@ -124,6 +124,10 @@ typedef struct hkv_table_view {
   uint8_t pow2_buckets; /* buckets_num is a power of two */
   uint8_t dual_bucket;  /* TableMode::kMemory: a key lives in one of two buckets */
   uint8_t pad_[4];
+  uint64_t* bounds;     /* [buckets_num][8]: for each run of 16 slots a value that is not above
+                           any score in it (0 is always right); kept tight by the LRU upserts,
+                           which with it read one or two of a bucket's eight score lines
+                           instead of all of them, and only meaningful for the LRU strategy */
 } hkv_table_view;
 
 /* BaseAllocator (include/merlin/allocator.cuh:27-58) as a table of callbacks.
@@ -341,6 +345,12 @@ int hkv_lock_end(const hkv_table* t, int role, hkv_stream_t stream);
  *           reference's own tests can only bound them (no counterpart there).
  */
 int hkv_set_clock(hkv_table* t, int mode, uint64_t base);
+
+/* Scores may have been changed by code outside the library: a functor handed to for_each gets
+ * a writable score (merlin_hashtable.cuh:3372-3412).  The table then drops what it knows about
+ * the scores (hkv_table_view::bounds) before it relies on it again.  No counterpart in the
+ * reference, which keeps no such knowledge. */
+int hkv_scores_changed(hkv_table* t);
 
 #ifdef __cplusplus
 }

@@ -841,6 +841,7 @@ class HashTable : public HashTableBase<K, V, S> {
     hkv_table_view v;
     throw_on_error_(hkv_table_get_view(table_, &v));
     if (first >= v.capacity || last > v.capacity || first >= last) return;
+    throw_on_error_(hkv_scores_changed(table_)); /* the functor may write scores */
     const uint64_t n = last - first;
     const unsigned blocks = static_cast<unsigned>(std::min<uint64_t>((n + 127) / 128, 16384));
     const uint64_t dim = options_.dim;

@@ -792,6 +792,107 @@ static void test_functor_forms() {
 }
 
 
+/* for_each body that pushes the scores of odd keys down to 1..N: what a caller may do with the
+ * writable score it is handed */
+template <class Kt, class Vt, class St>
+struct SinkOddKeys {
+  template <int GroupSize>
+  __forceinline__ __device__ void operator()(const Kt& key, Vt* value, St* score,
+                                             cg::thread_block_tile<GroupSize>& g) {
+    if (live_key(key) && (key & 1u)) *score = 1 + (static_cast<uint64_t>(key) >> 40);
+  }
+};
+
+/* An LRU table finds eviction victims through per-line lower bounds of the scores
+ * (hkv_table_view::bounds).  The calls of the header that lower scores behind the library's back
+ * - erase_if, erase_if_v2 (tombstones have score 0) and for_each with a functor that writes
+ * scores - must leave them right: after each, and after upserts that evict, no bound is above a
+ * score of its line, and the keys whose scores were pushed down are the ones that go. */
+static void test_score_bounds_after_header_calls() {
+  constexpr size_t DIM = 8, CAP = 1 << 14, N = 1 << 13;
+  HashTableOptions o;
+  o.init_capacity = o.max_capacity = CAP;
+  o.dim = DIM;
+  o.max_hbm_for_vectors = GB(1);
+  using Table = HashTable<K, V, S, EvictStrategy::kLru>;
+  Table table;
+  table.init(o);
+  auto bounds_hold = [&]() {
+    HIP(hipDeviceSynchronize());
+    hkv_table_view v;
+    if (hkv_table_get_view(table.native_handle(), &v)) return false;
+    std::vector<uint64_t> sc(v.capacity), bd(v.capacity / 16);
+    HIP(hipMemcpy(sc.data(), v.scores, sc.size() * 8, hipMemcpyDeviceToHost));
+    HIP(hipMemcpy(bd.data(), v.bounds, bd.size() * 8, hipMemcpyDeviceToHost));
+    for (size_t l = 0; l < bd.size(); l++)
+      for (size_t q = 0; q < 16; q++)
+        if (bd[l] > sc[l * 16 + q]) return false;
+    return true;
+  };
+  DevBuf<K> dk(N);
+  DevBuf<V> dv(N * DIM);
+  auto put = [&](uint64_t seed) {
+    auto keys = random_keys(N, seed);
+    dk.up(keys);
+    dv.up(values_of(keys, DIM));
+    table.insert_or_assign(N, dk.p, dv.p);
+    return keys;
+  };
+  for (uint64_t b = 0; b < 5; b++) put(4000 + b);  // 2.5 x capacity: every bucket has evicted
+  CHECK(table.size() > CAP * 95 / 100);
+  CHECK(bounds_hold());
+  // tombstones from both erase_if forms, in lines whose bounds are tight
+  const size_t before = table.size();
+  const size_t odd = table.template erase_if<EraseIfPredFunctor>(0, S(0));  // odd keys, any score
+  CHECK(odd > before / 3 && table.size() == before - odd);
+  CHECK(bounds_hold());
+  put(4010);
+  CHECK(bounds_hold());
+  ScoreBelowV2<K, V, S> all{~S(0)};
+  const size_t rest = table.template erase_if_v2<ScoreBelowV2<K, V, S>>(all);
+  CHECK(rest > 0 && table.size() == 0);
+  CHECK(bounds_hold());
+  // refill, then push the scores of the odd keys far down through for_each: they go first
+  std::vector<K> resident;
+  for (uint64_t b = 0; b < 4; b++) {
+    auto k = put(4020 + b);
+    resident.insert(resident.end(), k.begin(), k.end());
+  }
+  SinkOddKeys<K, V, S> sink;
+  table.template for_each<SinkOddKeys<K, V, S>>(0, table.capacity(), sink);
+  HIP(hipDeviceSynchronize());
+  CHECK(table.template size_if<EraseIfPredFunctor>(0, S(0)) > CAP / 3);
+  hkv_table_view v;
+  CHECK(hkv_table_get_view(table.native_handle(), &v) == 0);
+  std::vector<uint64_t> keys0(v.capacity), keys1(v.capacity), sc1(v.capacity);
+  HIP(hipMemcpy(keys0.data(), v.keys, keys0.size() * 8, hipMemcpyDeviceToHost));
+  put(4030);  // a table's worth of new keys: every eviction takes its bucket's lowest score
+  put(4031);
+  CHECK(bounds_hold());
+  HIP(hipMemcpy(keys1.data(), v.keys, keys1.size() * 8, hipMemcpyDeviceToHost));
+  HIP(hipMemcpy(sc1.data(), v.scores, sc1.size() * 8, hipMemcpyDeviceToHost));
+  /* bucket by bucket: while a sunk score is left in a bucket, no key that was not sunk can have
+   * been evicted from it */
+  size_t wrong = 0, sunk_gone = 0;
+  for (size_t b = 0; b < v.buckets_num; b++) {
+    std::unordered_set<uint64_t> after(keys1.begin() + b * 128, keys1.begin() + (b + 1) * 128);
+    bool sunk_left = false, even_lost = false;
+    for (size_t q = 0; q < 128; q++) {
+      const uint64_t k1 = keys1[b * 128 + q], k0 = keys0[b * 128 + q];
+      if (k1 < 0xFFFFFFFFFFFFFFFCull && (k1 & 1u) && sc1[b * 128 + q] < (1ull << 30)) sunk_left = true;
+      if (k0 < 0xFFFFFFFFFFFFFFFCull && !after.count(k0)) {
+        if (k0 & 1u)
+          sunk_gone++;
+        else
+          even_lost = true;
+      }
+    }
+    if (sunk_left && even_lost) wrong++;
+  }
+  CHECK(wrong == 0);
+  CHECK(sunk_gone > CAP / 4);
+}
+
 // TableMode::kMemory through the header: init checks, insert_or_assign + find, guards
 // (tests/dual_bucket_test.cc.cu:74-158, 471-515, 641-661, 1051-1107)
 static void test_dual_bucket_mode() {
@@ -1157,6 +1258,7 @@ int main() {
     test_growth_and_key_locks();
     test_header_templates_beside_growth();
     test_functor_forms();
+    test_score_bounds_after_header_calls();
     test_dual_bucket_mode();
     test_uint32_scores();
     test_basic_for_cpu_io();
