@@ -28,7 +28,7 @@ fill_kernel(View v, int zero_scores) {
 #pragma unroll
       for (int q = 0; q < 16; q++) s[q] = 0;
     }
-    v.bounds[t] = 0; /* one per 16 slots */
+    if (v.bounds) v.bounds[t] = 0; /* one per 16 slots */
   }
   if (t < v.buckets_num) v.sizes[t] = 0;
 }
@@ -74,7 +74,8 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
     if (erased) {
       v.digests[slot] = v.reclaim_digest;
       v.scores[slot] = 0;
-      v.bounds[slot >> 4] = 0; /* the one place where a score goes down: its line's bound follows */
+      /* the one place where a score goes down: its line's bound follows */
+      if (v.bounds) v.bounds[slot >> 4] = 0;
     }
   }
   const uint32_t bkt = erased ? (uint32_t)(slot >> 7) : 0xFFFFFFFFu;

@@ -558,14 +558,14 @@ int alloc_arenas(hkv_table* t, uint64_t buckets_num, View& v, TableMem& m) {
   const uint64_t off_scores = off_keys + up(v.capacity * 8);
   const uint64_t off_sizes = off_scores + up(v.capacity * 8);
   const uint64_t off_bounds = off_sizes + up(v.buckets_num * 4);
-  m.meta_bytes = off_bounds + up(v.buckets_num * 8 * sizeof(uint64_t));
+  m.meta_bytes = off_bounds + (t->score_bounds ? up(v.buckets_num * 8 * sizeof(uint64_t)) : 0);
   HKV_TRY(table_alloc(t, 0, &m.d_meta, m.meta_bytes));
   uint8_t* base = (uint8_t*)m.d_meta;
   v.digests = base;
   v.keys = (uint64_t*)(base + off_keys);
   v.scores = (uint64_t*)(base + off_scores);
   v.sizes = (int32_t*)(base + off_sizes);
-  v.bounds = (uint64_t*)(base + off_bounds);
+  v.bounds = t->score_bounds ? (uint64_t*)(base + off_bounds) : nullptr;
   /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
    * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
   const uint64_t bucket_bytes = (uint64_t)kBucketSize * v.value_bytes;
@@ -1083,7 +1083,8 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->upsert_path = 1;
   {
     const char* b = getenv("HKV_SCORE_BOUNDS");
-    t->score_bounds = !(b && !strcmp(b, "0"));
+    /* only LRU keeps them right by itself (hkv_upsert.hpp); other tables carry none */
+    t->score_bounds = !(b && !strcmp(b, "0")) && t->opts.evict_strategy == HKV_LRU && !t->dual;
   }
   if (const char* e = getenv("HKV_UPSERT_PATH")) {
     if (!strcmp(e, "auto")) t->upsert_path = 0;

@@ -124,10 +124,11 @@ typedef struct hkv_table_view {
   uint8_t pow2_buckets; /* buckets_num is a power of two */
   uint8_t dual_bucket;  /* TableMode::kMemory: a key lives in one of two buckets */
   uint8_t pad_[4];
-  uint64_t* bounds;     /* [buckets_num][8]: for each run of 16 slots a value that is not above
-                           any score in it (0 is always right); kept tight by the LRU upserts,
-                           which with it read one or two of a bucket's eight score lines
-                           instead of all of them, and only meaningful for the LRU strategy */
+  uint64_t* bounds;     /* LRU tables, else NULL.  [buckets_num][8]: for each run of 16 slots a
+                           value that is not above any score in it (0 is always right); kept
+                           tight by the upserts, which with it read one or two of a bucket's
+                           eight score lines instead of all of them.  Whoever lowers a score
+                           (a tombstone gets score 0) sets the bound of its run to 0 */
 } hkv_table_view;
 
 /* BaseAllocator (include/merlin/allocator.cuh:27-58) as a table of callbacks.

@@ -260,7 +260,7 @@ erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshol
       v.keys[s] = v.reclaim_key;
       v.digests[s] = v.reclaim_digest;
       v.scores[s] = 0;
-      v.bounds[s >> 4] = 0;
+      if (v.bounds) v.bounds[s >> 4] = 0;
       atomicSub(v.sizes + (s >> 7), 1);
       local++;
     }
@@ -422,7 +422,7 @@ erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* 
       v.digests[slot] = v.reclaim_digest;
       v.keys[slot] = v.reclaim_key;
       v.scores[slot] = 0;
-      v.bounds[slot >> 4] = 0;
+      if (v.bounds) v.bounds[slot >> 4] = 0;
       atomicSub(v.sizes + (slot >> 7), 1);
       local++;
     }
