@@ -188,6 +188,37 @@ zero_words_kernel(uint32_t* p, uint64_t n) {
   if (q * 4 < n) reinterpret_cast<uint4*>(p)[q] = make_uint4(0, 0, 0, 0);
 }
 
+/* The score bounds of an LRU table from scratch: for every line of 16 slots the lowest score of
+ * its keys, but nothing above a value that no score written from now on is below (as
+ * UpsertArgs::bound_cap), and 0 for a line without keys.  A free slot does not count: what it gets later
+ * is a score of that time.  Eight lanes per line, one wavefront per 8 lines; the caller has
+ * the table to itself. */
+__global__ void __launch_bounds__(256)
+rebuild_bounds_kernel(View v, Clock clock) {
+  const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint64_t line = t >> 3;
+  const int j = (int)(t & 7);
+  if (line >= v.capacity / 16) return; /* whole tiles leave together: lines are a multiple of 8 */
+  /* deterministic clock: the base of the call that is about to run; hardware clock: now, which
+   * is before anything that call writes */
+  const uint64_t cap = clock.mode == 1 ? clock.base : now_ns(clock, 0);
+  const uint4 k = *reinterpret_cast<const uint4*>(v.keys + line * 16 + j * 2);
+  const uint4 s = *reinterpret_cast<const uint4*>(v.scores + line * 16 + j * 2);
+  const uint64_t k0 = k.x | ((uint64_t)k.y << 32), k1 = k.z | ((uint64_t)k.w << 32);
+  const uint64_t s0 = s.x | ((uint64_t)s.y << 32), s1 = s.z | ((uint64_t)s.w << 32);
+  /* a tombstone holds score 0 and is what a search should find first; LOCKED slots (lock_keys)
+   * hold a key with its score */
+  uint64_t m = kMaxScore;
+  if (k0 != v.empty_key) m = s0;
+  if (k1 != v.empty_key && s1 < m) m = s1;
+#pragma unroll
+  for (int off = 1; off < kTile; off <<= 1) {
+    const uint64_t o = __shfl_xor(m, off);
+    m = o < m ? o : m;
+  }
+  if (j == 0) v.bounds[line] = m == kMaxScore ? 0 : (m < cap ? m : cap);
+}
+
 /* ---- built-in predicates (hkv_predicate) -------------------------------------- */
 
 struct PredAlways {

@@ -167,8 +167,9 @@ struct hkv_table {
   bool own_alloc;
   hkv_allocator alloc;
   void* d_meta;          /* digests + keys + scores + sizes + score bounds in one arena */
+  std::atomic<uint64_t> keys_offered{0}; /* keys handed to upserts since creation or clear: above the size */
   bool score_bounds;     /* LRU upserts search victims through the score bounds (HKV_SCORE_BOUNDS=0: off) */
-  std::atomic<bool> bounds_stale{false}; /* a call may have written scores below the bounds */
+  std::atomic<bool> bounds_stale{true}; /* a call may have written scores below the bounds */
   uint64_t meta_bytes;
   void* d_values;        /* value rows in HBM */
   void* h_values;        /* host address of the pinned value rows (hybrid) */
@@ -622,6 +623,7 @@ int double_table(hkv_table* t, hipStream_t s) {
   t->h_values = mem.h_values;
   t->view = nv;
   t->pure_hbm = nv.hbm_slots == nv.capacity;
+  t->bounds_stale = true; /* the new arenas have none yet */
   free_arenas(t, old);
   return HKV_SUCCESS;
 }
@@ -701,6 +703,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   a.refuse_equal = refuse_equal;
   /* scores that do not come from the table's clock may be lower than what the bounds say */
   if (a.strategy != t->opts.evict_strategy) t->bounds_stale = true;
+  t->keys_offered += a.n;
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
@@ -721,13 +724,12 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
        * no such slot the plain scan finds the same victims (a slot locked by another key of
        * the batch is retried instead of skipped) */
       launch_upsert<OP, true>(vec, t->view, a, s);
-    } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr)) {
-      /* LRU scores only grow, which is what keeps the score bounds right by themselves */
-      if (t->bounds_stale.exchange(false)) {
-        const uint64_t words = t->view.buckets_num * 8 * 2;
-        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((words / 4 + 255) / 256)), dim3(256), 0, s,
-                           (uint32_t*)t->view.bounds, words);
-      }
+    } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr) &&
+               t->keys_offered * 10 >= t->view.capacity * 9) {
+      /* LRU scores only grow, which is what keeps the score bounds right by themselves.  The
+       * bounded search pays once buckets are full; a table that cannot be nine tenths full yet
+       * (it has not been offered that many keys since it was created or cleared) takes the plain
+       * kernel, whose few evictions leave the bounds as they are, which is as right as before. */
       /* No bound may be above a score that this call writes.  Deterministic clock: the call's
        * scores start at its base.  Hardware clock: they are later than the start of the last
        * call of this kind, which that call left in a device word (this one leaves its own in
@@ -737,6 +739,13 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
         a.bound_cap_in = t->d_bound_caps + (t->bound_cap_turn & 1);
         a.bound_cap_out = t->d_bound_caps + ((t->bound_cap_turn + 1) & 1);
         t->bound_cap_turn++;
+      }
+      /* bounds that were never set (a new or cleared table reaching this point) or that may be
+       * above a score (scores from outside the clock) are made from the scores as they are */
+      if (t->bounds_stale.exchange(false)) {
+        const uint64_t threads = t->view.capacity / 16 * 8;
+        hipLaunchKernelGGL(rebuild_bounds_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                           t->view, t->clock);
       }
       launch_upsert<OP, false, true>(vec, t->view, a, s);
     } else {
@@ -1756,6 +1765,8 @@ int hkv_clear(hkv_table* t, hkv_stream_t stream) {
   /* every key word becomes EMPTY, the LOCKED ones included */
   t->keys_may_be_locked = false;
   t->locked_recount = false;
+  t->keys_offered = 0;
+  t->bounds_stale = true;
   hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, t->d_locked);
   const uint64_t groups = t->view.capacity / 16;
   hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s,

@@ -24,12 +24,15 @@ def bytes_of(a):
 
 
 def bounds_hold(t):
-    """bound[line] <= every score of the line, for all lines of the table."""
+    """bound[line] <= the score of every key (or tombstone) of the line, for all lines of the table.
+    A free slot does not count: it gets a score of the time when it is taken."""
     torch.cuda.synchronize()
     v = t.view()
     cap = v.capacity
-    scores = read_device(v.scores, cap * 8).view(np.uint64).reshape(cap // 16, 16)
+    scores = read_device(v.scores, cap * 8).view(np.uint64).reshape(cap // 16, 16).copy()
+    keys = read_device(v.keys, cap * 8).view(np.uint64).reshape(cap // 16, 16)
     bounds = read_device(v.bounds, cap // 16 * 8).view(np.uint64)
+    scores[keys == np.uint64(v.empty_key)] = np.uint64((1 << 64) - 1)
     bad = np.flatnonzero(bounds > scores.min(axis=1))
     return len(bad) == 0, bad[:5], int((bounds > 0).sum())
 
