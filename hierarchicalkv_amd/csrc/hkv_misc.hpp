@@ -36,7 +36,7 @@ fill_kernel(View v, int zero_scores) {
 /* one sample of the constant-rate device counter (table creation: see Clock) */
 __global__ void clock_sample_kernel(unsigned long long* out) { *out = wall_clock64(); }
 
-/* remove_kernel (core_kernels.cuh:679-741): tombstone the slot.
+/* remove_kernel (core_kernels.cuh:679-741): free the slot.
  * EXCLUSIVE: the call is the only one on the table while it runs (it holds the inserter role
  * of the group lock), so the key word is overwritten with a plain store as in the reference
  * (core_kernels.cuh:723-737; like there, a batch that names a key twice in different
@@ -64,18 +64,23 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
   }
   bool erased = false;
   if (mine) {
+    /* The slot becomes a free slot outright: EMPTY key, EMPTY digest.  The reference leaves a
+     * tombstone (RECLAIM key, score 0, core_kernels.cuh:723-737) because its probes stop at the
+     * first EMPTY key; here every probe looks at all 128 digests, a free slot in the middle of a
+     * bucket hides nothing, and the next insert takes it through the free-slot path instead of
+     * finding it as the bucket's lowest score.  Which slot a key lands in shows in no result;
+     * one store and one score write less per key. */
     if (EXCLUSIVE) {
       erased = true;
-      v.keys[slot] = v.reclaim_key;
+      v.keys[slot] = v.empty_key;
     } else {
       uint64_t seen = key;
-      erased = cas_lock(v.keys + slot, seen, v.reclaim_key);
+      erased = cas_lock(v.keys + slot, seen, v.locked_key);
     }
     if (erased) {
-      v.digests[slot] = v.reclaim_digest;
-      v.scores[slot] = 0;
-      /* the one place where a score goes down: its line's bound follows */
-      if (v.bounds) v.bounds[slot >> 4] = 0;
+      v.digests[slot] = v.empty_digest;
+      /* without the group lock an inserter may be looking: the key word opens last */
+      if (!EXCLUSIVE) st_u64(v.keys + slot, v.empty_key);
     }
   }
   const uint32_t bkt = erased ? (uint32_t)(slot >> 7) : 0xFFFFFFFFu;

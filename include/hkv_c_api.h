@@ -128,7 +128,8 @@ typedef struct hkv_table_view {
                            value that is not above any score in it (0 is always right); kept
                            tight by the upserts, which with it read one or two of a bucket's
                            eight score lines instead of all of them.  Whoever lowers a score
-                           (a tombstone gets score 0) sets the bound of its run to 0 */
+                           in place sets the bound of its run to 0 or calls
+                           hkv_scores_changed */
 } hkv_table_view;
 
 /* BaseAllocator (include/merlin/allocator.cuh:27-58) as a table of callbacks.

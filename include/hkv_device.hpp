@@ -257,10 +257,9 @@ erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshol
     uint64_t key = v.keys[s];
     uint64_t score = v.scores[s];
     if (!is_reserved_key(v, key) && pred(key, score, pattern, threshold)) {
-      v.keys[s] = v.reclaim_key;
-      v.digests[s] = v.reclaim_digest;
-      v.scores[s] = 0;
-      if (v.bounds) v.bounds[s >> 4] = 0;
+      /* a free slot again, not a tombstone: see erase_kernel */
+      v.keys[s] = v.empty_key;
+      v.digests[s] = v.empty_digest;
       atomicSub(v.sizes + (s >> 7), 1);
       local++;
     }
@@ -419,10 +418,8 @@ erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* 
     bool match = pred.template operator()<GroupSize>(key, value, score, g);
     if (is_reserved_key(v, raw)) match = false;
     if (match) {
-      v.digests[slot] = v.reclaim_digest;
-      v.keys[slot] = v.reclaim_key;
-      v.scores[slot] = 0;
-      if (v.bounds) v.bounds[slot >> 4] = 0;
+      v.digests[slot] = v.empty_digest;
+      v.keys[slot] = v.empty_key;
       atomicSub(v.sizes + (slot >> 7), 1);
       local++;
     }

@@ -804,9 +804,9 @@ struct SinkOddKeys {
 };
 
 /* An LRU table finds eviction victims through per-line lower bounds of the scores
- * (hkv_table_view::bounds).  The calls of the header that lower scores behind the library's back
- * - erase_if, erase_if_v2 (tombstones have score 0) and for_each with a functor that writes
- * scores - must leave them right: after each, and after upserts that evict, no bound is above a
+ * (hkv_table_view::bounds).  The calls of the header that change slots or scores behind the
+ * library's back - erase_if, erase_if_v2 and for_each with a functor that writes scores - must
+ * leave them right: after each, and after upserts that evict, no bound is above a
  * score of its line, and the keys whose scores were pushed down are the ones that go. */
 static void test_score_bounds_after_header_calls() {
   constexpr size_t DIM = 8, CAP = 1 << 14, N = 1 << 13;
@@ -842,7 +842,7 @@ static void test_score_bounds_after_header_calls() {
   for (uint64_t b = 0; b < 5; b++) put(4000 + b);  // 2.5 x capacity: every bucket has evicted
   CHECK(table.size() > CAP * 95 / 100);
   CHECK(bounds_hold());
-  // tombstones from both erase_if forms, in lines whose bounds are tight
+  // slots freed by both erase_if forms, in lines whose bounds are tight
   const size_t before = table.size();
   const size_t odd = table.template erase_if<EraseIfPredFunctor>(0, S(0));  // odd keys, any score
   CHECK(odd > before / 3 && table.size() == before - odd);

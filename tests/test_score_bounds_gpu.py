@@ -4,8 +4,8 @@ one or two of its eight score lines.  Checked here:
   * the invariant itself, read back from device memory after mixed call sequences, on the
     deterministic and on the hardware clock (a bound above a score would send an eviction to the
     wrong slot sooner or later);
-  * that the calls which may lower scores (erase, upserts with ignore_evict_strategy, set_clock)
-    leave the bounds right;
+  * that erase and the calls which may lower scores (upserts with ignore_evict_strategy,
+    set_clock) leave the bounds right;
   * parity with the oracle through all of this (deterministic clock), which is the parity of the
     bounded search with the full scan: the oracle scans all 128 scores."""
 import numpy as np
