@@ -199,8 +199,11 @@ zero_words_kernel(uint32_t* p, uint64_t n) {
  * is a score of that time.  Eight lanes per line, one wavefront per 8 lines; the caller has
  * the table to itself. */
 __global__ void __launch_bounds__(256)
-rebuild_bounds_kernel(View v, Clock clock) {
+rebuild_bounds_kernel(View v, Clock clock, unsigned long long* cap_word) {
   const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  /* hardware clock: the upsert that follows takes its own limit for bounds from this word
+   * (UpsertArgs::bound_cap_in), which has no reading yet the first time */
+  if (t == 0 && cap_word) *cap_word = now_ns(clock, 0);
   const uint64_t line = t >> 3;
   const int j = (int)(t & 7);
   if (line >= v.capacity / 16) return; /* whole tiles leave together: lines are a multiple of 8 */

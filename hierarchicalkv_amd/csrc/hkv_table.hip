@@ -745,7 +745,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
       if (t->bounds_stale.exchange(false)) {
         const uint64_t threads = t->view.capacity / 16 * 8;
         hipLaunchKernelGGL(rebuild_bounds_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           t->view, t->clock);
+                           t->view, t->clock, const_cast<unsigned long long*>(a.bound_cap_in));
       }
       launch_upsert<OP, false, true>(vec, t->view, a, s);
     } else {
