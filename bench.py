@@ -1,7 +1,7 @@
 #!/usr/bin/env python
 """Benchmark of the hot path on one MI355X.
 
-Workload (BASELINE.json metric shape): capacity 2^26 keys, uint64 keys, fp32
+Workload (the shape the headline metric is quoted on): capacity 2^26 keys, uint64 keys, fp32
 values dim 64 (16 GiB of value rows, all in HBM), uint64 scores, LRU, batch
 2^20, table pre-filled to load factor 1.0.  One step = find on 2^20 resident
 keys (100 % hits) followed by insert_or_assign of 2^20 keys, half resident and

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes.
+"""The benchmark configurations 2 to 5 at their full sizes.
 
 No host oracle finishes at these sizes, so the checks are properties that do
 not depend on size: every row that comes back (found, evicted or exported)
