@@ -690,6 +690,17 @@ int settle_locked_count(hkv_table* t, hipStream_t s) {
   return HKV_SUCCESS;
 }
 
+/* A call recorded into a HIP graph runs again with every replay: the pass that builds the score
+ * bounds does not belong into one (the plain kernel is recorded instead while the bounds are stale). */
+bool capturing(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st == hipStreamCaptureStatusActive;
+}
+
 /* `hybrid_rule`: the operation follows the lock-key kernels of hybrid mode when
  * the table is not pure HBM (insert_or_assign, find_or_insert); the pointer
  * overload always does. */
@@ -725,7 +736,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
        * the batch is retried instead of skipped) */
       launch_upsert<OP, true>(vec, t->view, a, s);
     } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr) &&
-               t->keys_offered * 10 >= t->view.capacity * 9) {
+               t->keys_offered * 10 >= t->view.capacity * 9 && !(t->bounds_stale && capturing(s))) {
       /* LRU scores only grow, which is what keeps the score bounds right by themselves.  The
        * bounded search pays once buckets are full; a table that cannot be nine tenths full yet
        * (it has not been offered that many keys since it was created or cleared) takes the plain
