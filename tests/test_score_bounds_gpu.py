@@ -16,7 +16,10 @@ import workloads as w
 from gpu_util import DEV, assert_same_table, dev, read_device
 from hierarchicalkv_amd import EvictStrategy, HashTable, default_options
 
-pytestmark = [pytest.mark.gpu]
+import os
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("HKV_SCORE_BOUNDS") == "0", reason="score bounds switched off")]
 
 
 def bytes_of(a):
