@@ -132,6 +132,47 @@ __device__ __forceinline__ uint32_t tile_ballot(bool pred, int tile) {
   return (uint32_t)(__ballot(pred) >> (tile * kTile)) & 0xFFu;
 }
 
+/* Value of lane (lane ^ OFF) of the same 8-lane tile, OFF = 1, 2 or 4, by data-parallel moves
+ * inside the vector unit: no trip through the LDS permute network as with __shfl_xor, whose
+ * latency adds up in the reductions that sit in dependent chains.  Every lane of the tile must
+ * be active.  lane ^ 4 is the mirror image of the 8 lanes followed by the mirror image of each
+ * quad. */
+template <int OFF>
+__device__ __forceinline__ uint32_t tile_xor(uint32_t x) {
+  static_assert(OFF == 1 || OFF == 2 || OFF == 4, "inside a tile");
+  if constexpr (OFF == 1) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, true); /* quad_perm [1,0,3,2] */
+  if constexpr (OFF == 2) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, true); /* quad_perm [2,3,0,1] */
+  const int h = __builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, true); /* row_half_mirror */
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, h, 0x1B, 0xF, 0xF, true);     /* quad_perm [3,2,1,0] */
+}
+template <int OFF>
+__device__ __forceinline__ uint64_t tile_xor(uint64_t x) {
+  return tile_xor<OFF>((uint32_t)x) | ((uint64_t)tile_xor<OFF>((uint32_t)(x >> 32)) << 32);
+}
+/* Minimum of a 64-bit value over the tile, and of (value, position) pairs ordered by value, then
+ * position; selects, no branches. */
+__device__ __forceinline__ uint64_t tile_min(uint64_t m) {
+  uint64_t o = tile_xor<1>(m);
+  m = o < m ? o : m;
+  o = tile_xor<2>(m);
+  m = o < m ? o : m;
+  o = tile_xor<4>(m);
+  return o < m ? o : m;
+}
+template <int OFF>
+__device__ __forceinline__ void tile_min_pair_step(uint64_t& m, uint32_t& pos) {
+  const uint64_t om = tile_xor<OFF>(m);
+  const uint32_t op = tile_xor<OFF>(pos);
+  const bool take = om < m || (om == m && op < pos);
+  m = take ? om : m;
+  pos = take ? op : pos;
+}
+__device__ __forceinline__ void tile_min_pair(uint64_t& m, uint32_t& pos) {
+  tile_min_pair_step<1>(m, pos);
+  tile_min_pair_step<2>(m, pos);
+  tile_min_pair_step<4>(m, pos);
+}
+
 /* ---- coherent access to words other wavefronts may be changing -----------
  *
  * An MI355X has one L2 per XCD (8 of them); ordinary cached loads and stores

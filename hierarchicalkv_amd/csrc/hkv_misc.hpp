@@ -219,11 +219,7 @@ rebuild_bounds_kernel(View v, Clock clock, unsigned long long* cap_word) {
   uint64_t m = kMaxScore;
   if (k0 != v.empty_key) m = s0;
   if (k1 != v.empty_key && s1 < m) m = s1;
-#pragma unroll
-  for (int off = 1; off < kTile; off <<= 1) {
-    const uint64_t o = __shfl_xor(m, off);
-    m = o < m ? o : m;
-  }
+  m = tile_min(m);
   if (j == 0) v.bounds[line] = m == kMaxScore ? 0 : (m < cap ? m : cap);
 }
 

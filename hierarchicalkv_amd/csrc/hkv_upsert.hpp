@@ -344,15 +344,7 @@ __device__ __forceinline__ void scan_reduce(const View& v, const uint64_t* sc, c
       bpos = p;
     }
   }
-#pragma unroll
-  for (int off = 1; off < kTile; off <<= 1) {
-    const uint64_t ob = __shfl_xor(best, off);
-    const uint32_t op = __shfl_xor(bpos, off);
-    if (ob < best || (ob == best && op < bpos)) {
-      best = ob;
-      bpos = op;
-    }
-  }
+  tile_min_pair(best, bpos);
 }
 
 /* ---- min-score search with per-line lower bounds (LRU) -------------------------------------------
@@ -381,15 +373,7 @@ __device__ __forceinline__ void line_min(const uint4& x, uint32_t g, int j, uint
   const uint32_t p0 = g * 16 + j * 2;
   m = s1 < s0 ? s1 : s0;
   pos = s1 < s0 ? p0 + 1 : p0;
-#pragma unroll
-  for (int off = 1; off < kTile; off <<= 1) {
-    const uint64_t om = __shfl_xor(m, off);
-    const uint32_t op = __shfl_xor(pos, off);
-    if (om < m || (om == m && op < pos)) {
-      m = om;
-      pos = op;
-    }
-  }
+  tile_min_pair(m, pos);
 }
 /* `bd`: this lane's bound (line j); `g`, `x`: the line with the lowest bound and this lane's
  * part of it.  All 8 lanes of the tile call this together.  `nb`: what line bpos / 16 is bounded
@@ -424,12 +408,7 @@ __device__ __forceinline__ void bounded_min(const View& v, uint64_t bs, int tile
   const uint64_t s0 = x.x | ((uint64_t)x.y << 32), s1 = x.z | ((uint64_t)x.w << 32);
   const uint32_t p0 = (bpos & ~15u) + j * 2;
   const uint64_t r0 = p0 == bpos ? kMaxScore : s0, r1 = p0 + 1 == bpos ? kMaxScore : s1;
-  nb = r1 < r0 ? r1 : r0;
-#pragma unroll
-  for (int off = 1; off < kTile; off <<= 1) {
-    const uint64_t o = __shfl_xor(nb, off);
-    if (o < nb) nb = o;
-  }
+  nb = tile_min(r1 < r0 ? r1 : r0);
 }
 
 /* 16-byte units of value rows a lane holds in registers at a time in the bulk copies.  Fewer
@@ -722,15 +701,7 @@ upsert_kernel(View v, UpsertArgs a) {
         for (int q = 0; q < 4; q++) {
           uint64_t b = bd[q];
           uint32_t gi = (uint32_t)j;
-#pragma unroll
-          for (int off = 1; off < kTile; off <<= 1) {
-            const uint64_t ob = __shfl_xor(b, off);
-            const uint32_t og = __shfl_xor(gi, off);
-            if (ob < b || (ob == b && og < gi)) {
-              b = ob;
-              gi = og;
-            }
-          }
+          tile_min_pair(b, gi);
           g[q] = gi;
           x[q] = make_uint4(0, 0, 0, 0);
           if ((need >> (h + q)) & 1u) x[q] = line_load(v, bs[q], g[q], j);
