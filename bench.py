@@ -49,6 +49,46 @@ def upsert_bytes(vb, new_fraction):
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic_cap2p26_dim64_batch2p20.json")
 
 
+class HipEvent:
+    """A HIP event for timing only, created with hipEventDisableSystemFence: recording it does not
+    write the caches back and invalidate them, as the events torch creates do, so the kernel after
+    it starts as it would with no event there (hip_runtime_api.h says as much of the flag).  The
+    timed region ends with a device synchronisation, after which the time stamps are read."""
+    _hip = None
+
+    def __init__(self, torch):
+        import ctypes as C
+        if HipEvent._hip is None:
+            HipEvent._hip = C.CDLL("libamdhip64.so")
+            HipEvent._hip.hipEventCreateWithFlags.argtypes = [C.POINTER(C.c_void_p), C.c_uint]
+            HipEvent._hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+            HipEvent._hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+            HipEvent._hip.hipEventDestroy.argtypes = [C.c_void_p]
+        self._C = C
+        self._torch = torch
+        self._e = C.c_void_p()
+        rc = HipEvent._hip.hipEventCreateWithFlags(C.byref(self._e), 0x20000000)  # hipEventDisableSystemFence
+        if rc:
+            raise RuntimeError("hipEventCreateWithFlags: %d" % rc)
+
+    def record(self):
+        rc = HipEvent._hip.hipEventRecord(self._e, self._C.c_void_p(self._torch.cuda.current_stream().cuda_stream))
+        if rc:
+            raise RuntimeError("hipEventRecord: %d" % rc)
+
+    def elapsed_time(self, later):
+        ms = self._C.c_float()
+        rc = HipEvent._hip.hipEventElapsedTime(self._C.byref(ms), self._e, later._e)
+        if rc:
+            raise RuntimeError("hipEventElapsedTime: %d" % rc)
+        return ms.value
+
+    def __del__(self):
+        if self._e:
+            HipEvent._hip.hipEventDestroy(self._e)
+            self._e = None
+
+
 def measured_traffic(kernel):
     try:
         with open(TRAFFIC_FILE) as f:
@@ -205,7 +245,7 @@ def main():
     out_vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
     founds = torch.empty(n, dtype=torch.bool, device=dev)
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    ev = [[HipEvent(torch) for _ in range(3)] for _ in range(steps)]
 
     def step(s):
         ev[s][0].record()
