@@ -323,7 +323,8 @@ int accum_unit(uint32_t value_bytes, const void* p, int kind) {
  * multiple of 16 bytes use. */
 template <int OP, bool LOCKED_RULE, bool BOUNDS = false>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
-  const dim3 grid(grid_for(a.n)), block(kWave);
+  constexpr int waves = upsert_waves(OP);
+  const dim3 grid(grid_for((a.n + waves - 1) / waves)), block(kWave * waves);
   if constexpr (OP == kOpAccumOrAssign && !BOUNDS) {
     /* the two units that only the element-wise add needs */
     if (vec == 8) {

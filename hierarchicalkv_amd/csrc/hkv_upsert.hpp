@@ -581,25 +581,42 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * the plain scan would pick and wait for without end.  Whether a key is
  * refused at score == min is a separate switch (UpsertArgs::refuse_equal).
  */
+/* Wavefronts per workgroup, each with its own 64 keys and its own staging area.  One everywhere
+ * except insert_and_evict, whose wavefronts claim their part of the evicted-keys output together:
+ * updates of one word are served one at a time, about 15 ns each, and one per wavefront and trip
+ * (some 24 thousand for 2^20 keys into full buckets) took 0.07 ms of the call's 0.46. */
+constexpr int upsert_waves(int op) { return op == kOpInsertAndEvict ? 2 : 1; }
+
 template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kWave * upsert_waves(OP))
     __attribute__((amdgpu_waves_per_eu(BOUNDS && OP != kOpAccumOrAssign ? 4 : 1)))
 upsert_kernel(View v, UpsertArgs a) {
   static_assert(!(BOUNDS && LOCKED_RULE), "the bounded search does not look at key words");
-  __shared__ KeyMeta s_meta[kWave];
-  __shared__ int64_t s_slot[kWave];
-  __shared__ __attribute__((aligned(16))) uint16_t s_em[kWave][kTile];
-  __shared__ uint8_t s_unsure[kWave];
+  constexpr int WAVES = upsert_waves(OP);
+  __shared__ KeyMeta s_meta_all[WAVES][kWave];
+  __shared__ int64_t s_slot_all[WAVES][kWave];
+  __shared__ __attribute__((aligned(16))) uint16_t s_em_all[WAVES][kWave][kTile];
+  __shared__ uint8_t s_unsure_all[WAVES][kWave];
+  /* what the wavefronts of a workgroup tell each other in a trip (two sets, used in turn):
+   * entries for the evicted-keys output and whether any key is still pending; then where the
+   * workgroup's entries start */
+  __shared__ uint32_t s_trip[2][WAVES];
+  __shared__ unsigned long long s_claim[2];
 
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  KeyMeta* const s_meta = s_meta_all[wave];
+  int64_t* const s_slot = s_slot_all[wave];
+  uint16_t (*const s_em)[kTile] = s_em_all[wave];
+  uint8_t* const s_unsure = s_unsure_all[wave];
   const int tile = lane >> 3, j = lane & 7;
-  const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
+  const uint64_t i = ((uint64_t)blockIdx.x * WAVES + wave) * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
 
   uint64_t bound_cap = 0;
   if constexpr (BOUNDS) {
     bound_cap = a.bound_cap_in ? *a.bound_cap_in : a.bound_cap;
-    if (a.bound_cap_out && blockIdx.x == 0 && lane == 0) *a.bound_cap_out = now_ns(a.clock, 0);
+    if (a.bound_cap_out && blockIdx.x == 0 && threadIdx.x == 0) *a.bound_cap_out = now_ns(a.clock, 0);
   }
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
@@ -628,7 +645,11 @@ upsert_kernel(View v, UpsertArgs a) {
    * lanes take part in every trip (the tile-cooperative steps read registers
    * of lanes whose own key is already done), until no lane is pending. */
   unsigned long long pend_mask = __ballot(pending);
-  while (pend_mask) {
+  /* with several wavefronts per workgroup all of them make as many trips as the slowest, so
+   * that every one arrives at the workgroup's barriers */
+  bool more = pend_mask != 0;
+  if constexpr (WAVES > 1) more = __syncthreads_or(more);
+  for (int trip = 0; more; trip++) {
     if (__ballot(pending && reprobe))
       settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, waited, lane);
 
@@ -781,27 +802,29 @@ upsert_kernel(View v, UpsertArgs a) {
       commit = is_accum == (got == kStDuplicate);
     }
 
+    /* upsert_and_evict.cuh:188-194, 218-224, 236-245: an evicted key leaves with its old row
+     * and the scanned minimum, a refused key with its input.  One counter update per workgroup
+     * and trip: every wavefront posts its number of entries (and whether it has keys left for
+     * another trip, which is known by now), the first wavefront claims the sum, and the
+     * bookkeeping stores of the trip go out while that update is under way. */
+    const bool emit = OP == kOpInsertAndEvict && (refused_now || (commit && got == kStEvict));
+    unsigned long long votes = 0, claimed = 0;
+    uint32_t before = 0, total = 0;
+    const int set = trip & 1;
     if (OP == kOpInsertAndEvict) {
-      /* upsert_and_evict.cuh:188-194, 218-224, 236-245: an evicted key leaves with
-       * its old row and the scanned minimum, a refused key with its input; one
-       * counter update per wavefront */
-      const bool emit = refused_now || (commit && got == kStEvict);
-      const unsigned long long votes = __ballot(emit);
-      if (votes) {
-        const int leader = (int)__ffsll(votes) - 1;
-        unsigned long long base_idx = 0;
-        if (lane == leader)
-          base_idx = atomicAdd(a.evicted_counter, (unsigned long long)__popcll(votes));
-        base_idx = __shfl(base_idx, leader);
-        const unsigned long long idx = base_idx + __popcll(votes & ((1ull << lane) - 1));
-        if (emit) {
-          a.evicted_keys[idx] = refused_now ? key : victim;
-          if (a.evicted_scores) a.evicted_scores[idx] = refused_now ? desired : best;
-        }
-        bulk_evicted<VEC, UPL>(emit ? (refused_now ? 1 : 2) : 0,
-                               refused_now ? a.values_in + i * v.value_bytes : row,
-                               a.evicted_values + idx * v.value_bytes, units, lane);
+      votes = __ballot(emit);
+      const bool stay = __ballot(pending && got == kStNone) != 0;
+      if (lane == 0) s_trip[set][wave] = (uint32_t)__popcll(votes) | (stay ? 0x100u : 0u);
+      __syncthreads();
+      more = false;
+#pragma unroll
+      for (int w = 0; w < WAVES; w++) {
+        const uint32_t t = s_trip[set][w];
+        if (w < wave) before += t & 0xFFu;
+        total += t & 0xFFu; /* the same in every wavefront of the workgroup */
+        more |= (t & 0x100u) != 0;
       }
+      if (total && threadIdx.x == 0) claimed = atomicAdd(a.evicted_counter, (unsigned long long)total);
     }
     if (OP == kOpFindOrInsertPtr && (locked || refused_now)) {
       a.out_ptrs[i] = locked ? row : nullptr;
@@ -815,6 +838,20 @@ upsert_kernel(View v, UpsertArgs a) {
         st_u64(v.bounds + (slot >> 4), new_bound < bound_cap ? new_bound : bound_cap);
       write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
       if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
+    }
+    if (OP == kOpInsertAndEvict && total) {
+      if (threadIdx.x == 0) s_claim[set] = claimed;
+      __syncthreads();
+      if (votes) {
+        const unsigned long long idx = s_claim[set] + before + __popcll(votes & ((1ull << lane) - 1));
+        if (emit) {
+          a.evicted_keys[idx] = refused_now ? key : victim;
+          if (a.evicted_scores) a.evicted_scores[idx] = refused_now ? desired : best;
+        }
+        bulk_evicted<VEC, UPL>(emit ? (refused_now ? 1 : 2) : 0,
+                               refused_now ? a.values_in + i * v.value_bytes : row,
+                               a.evicted_values + idx * v.value_bytes, units, lane);
+      }
     }
     if (OP != kOpFindOrInsertPtr) {
       int move = kMoveNone;
@@ -847,6 +884,7 @@ upsert_kernel(View v, UpsertArgs a) {
     }
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
+    if constexpr (WAVES == 1) more = pend_mask != 0;
     if (pend_mask) __builtin_amdgcn_s_sleep(1);
   }
 }
