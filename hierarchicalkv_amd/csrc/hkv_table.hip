@@ -321,38 +321,50 @@ int accum_unit(uint32_t value_bytes, const void* p, int kind) {
 /* BOUNDS: the victim search reads the bucket's score bounds and one or two of its score lines
  * instead of all eight (hkv_upsert.hpp); for 16-byte units, which is what tables with rows of a
  * multiple of 16 bytes use. */
-template <int OP, bool LOCKED_RULE, bool BOUNDS = false>
+template <int OP, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
-  constexpr int waves = upsert_waves(OP);
-  const dim3 grid(grid_for((a.n + waves - 1) / waves)), block(kWave * waves);
+  const dim3 grid(grid_for((a.n + WAVES - 1) / WAVES)), block(kWave * WAVES);
   if constexpr (OP == kOpAccumOrAssign && !BOUNDS) {
     /* the two units that only the element-wise add needs */
     if (vec == 8) {
-      hipLaunchKernelGGL((upsert_kernel<OP, 8, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      hipLaunchKernelGGL((upsert_kernel<OP, 8, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
       return;
     }
     if (vec == 2) {
-      hipLaunchKernelGGL((upsert_kernel<OP, 2, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      hipLaunchKernelGGL((upsert_kernel<OP, 2, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
       return;
     }
   }
   if (OP == kOpFindOrInsertPtr) {
-    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a);
+    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a);
     return;
   }
   if (vec == 16) {
     switch (pick_upl(v.value_bytes, 16)) {
-      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
-      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
-      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
-      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS>), grid, block, 0, s, v, a); break;
+      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
+      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
+      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
+      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
     }
   } else if constexpr (!BOUNDS) {
     if (vec == 4)
-      hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
     else
-      hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE>), grid, block, 0, s, v, a);
+      hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
   }
+}
+
+/* insert_and_evict with `pair`: two wavefronts per workgroup share the claims on the
+ * evicted-keys output (hkv_upsert.hpp) */
+template <int OP, bool LOCKED_RULE, bool BOUNDS = false>
+void launch_upsert_for(bool pair, int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
+  if constexpr (OP == kOpInsertAndEvict) {
+    if (pair) {
+      launch_upsert<OP, LOCKED_RULE, BOUNDS, 2>(vec, v, a, s);
+      return;
+    }
+  }
+  launch_upsert<OP, LOCKED_RULE, BOUNDS, 1>(vec, v, a, s);
 }
 
 /* Whether a batch goes through the two-phase path (hkv_grouped.hpp). */
@@ -727,6 +739,8 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
      * mode of the tests takes it there */
     if (OP == kOpInsertAndEvict && t->upsert_path != 2) two_phase = false;
     if (vec == 8 || vec == 2) two_phase = false; /* units only the slot-lock kernel has */
+    /* a table that has been offered fewer keys than nine tenths of its slots evicts next to nothing */
+    const bool pair = OP == kOpInsertAndEvict && t->keys_offered * 10 >= t->view.capacity * 9;
     if (two_phase) {
       if constexpr (OP != kOpFindOrInsertPtr)
         HKV_TRY(run_two_phase<OP>(t, a, vec, refuse_equal, s));
@@ -735,7 +749,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
        * be hidden from the victim scan, which then reads the key words beside the scores; with
        * no such slot the plain scan finds the same victims (a slot locked by another key of
        * the batch is retried instead of skipped) */
-      launch_upsert<OP, true>(vec, t->view, a, s);
+      launch_upsert_for<OP, true>(pair, vec, t->view, a, s);
     } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr) &&
                t->keys_offered * 10 >= t->view.capacity * 9 && !(t->bounds_stale && capturing(s))) {
       /* LRU scores only grow, which is what keeps the score bounds right by themselves.  The
@@ -759,9 +773,9 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
         hipLaunchKernelGGL(rebuild_bounds_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
                            t->view, t->clock, const_cast<unsigned long long*>(a.bound_cap_in));
       }
-      launch_upsert<OP, false, true>(vec, t->view, a, s);
+      launch_upsert_for<OP, false, true>(pair, vec, t->view, a, s);
     } else {
-      launch_upsert<OP, false>(vec, t->view, a, s);
+      launch_upsert_for<OP, false>(pair, vec, t->view, a, s);
     }
     HKV_HIP(hipGetLastError());
   }

@@ -581,18 +581,18 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * the plain scan would pick and wait for without end.  Whether a key is
  * refused at score == min is a separate switch (UpsertArgs::refuse_equal).
  */
-/* Wavefronts per workgroup, each with its own 64 keys and its own staging area.  One everywhere
- * except insert_and_evict, whose wavefronts claim their part of the evicted-keys output together:
- * updates of one word are served one at a time, about 15 ns each, and one per wavefront and trip
- * (some 24 thousand for 2^20 keys into full buckets) took 0.07 ms of the call's 0.46. */
-constexpr int upsert_waves(int op) { return op == kOpInsertAndEvict ? 2 : 1; }
-
-template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false>
-__global__ void __launch_bounds__(kWave * upsert_waves(OP))
+/* WAVES wavefronts per workgroup, each with its own 64 keys and its own staging area.  One
+ * everywhere except insert_and_evict on a table that is about full, whose wavefronts claim their
+ * part of the evicted-keys output together: updates of one word are served one at a time, about
+ * 15 ns each, and one per wavefront and trip (some 24 thousand for 2^20 keys into full buckets)
+ * took 0.07 ms of the call's 0.46.  (While buckets have free slots there is nothing to claim,
+ * and two wavefronts that wait for each other in every trip are 4 % slower than one.) */
+template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1>
+__global__ void __launch_bounds__(kWave * WAVES)
     __attribute__((amdgpu_waves_per_eu(BOUNDS && OP != kOpAccumOrAssign ? 4 : 1)))
 upsert_kernel(View v, UpsertArgs a) {
   static_assert(!(BOUNDS && LOCKED_RULE), "the bounded search does not look at key words");
-  constexpr int WAVES = upsert_waves(OP);
+  static_assert(WAVES == 1 || OP == kOpInsertAndEvict, "only insert_and_evict has anything to share");
   __shared__ KeyMeta s_meta_all[WAVES][kWave];
   __shared__ int64_t s_slot_all[WAVES][kWave];
   __shared__ __attribute__((aligned(16))) uint16_t s_em_all[WAVES][kWave][kTile];
