@@ -151,6 +151,53 @@ def test_config3_insert_and_evict_zipf(oracle):
     t.close()
 
 
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kCustomized])
+def test_insert_and_evict_ragged_batches_on_a_full_table(oracle, strategy):
+    """On a full table the kernel runs two wavefronts of 64 keys per workgroup that claim their
+    entries of the evicted-keys output together: batches that fill neither, one, or one and a
+    bit of a workgroup, and larger ragged ones."""
+    cap, dim = 1 << 14, 8
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim, evict_strategy=strategy)
+    lru = strategy == EvictStrategy.kLru
+    if lru:
+        t.set_clock(1, 1 << 40)
+        o.set_clock(1, 1 << 40)
+    seed, pos, batch = 0x484B5611, 0, 1
+
+    def scores_for(n):
+        return None if lru else w.monotone_scores(batch, n, seed=11)
+
+    while pos < 2 * cap:  # twice the capacity: every bucket is full
+        keys = w.unique_keys(seed, pos, 4096)
+        vals = w.values_from_keys(keys, dim)
+        sc = scores_for(4096)
+        t.insert_or_assign(4096, dev(keys), dev(vals), None if sc is None else dev(sc))
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+        pos += 4096
+        batch += 1
+    assert t.size() == o.size()
+    for n in (1, 63, 64, 65, 127, 128, 129, 1000, 4097):
+        # half resident (from the last batches), half new
+        keys = np.concatenate([w.unique_keys(seed, pos - n, n // 2), w.unique_keys(seed, pos, n - n // 2)])
+        pos += n
+        vals = w.values_from_keys(keys, dim) + np.float32(batch)
+        sc = scores_for(n)
+        ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+        ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        es = torch.zeros(n, dtype=torch.int64, device=DEV)
+        cnt = t.insert_and_evict(n, dev(keys), dev(vals), None if sc is None else dev(sc), ek, ev, es)
+        oek, oev, oes = o.insert_and_evict(keys, bytes_of(vals), sc)
+        assert cnt == len(oek), n
+        gk, _, _ = sort_by_key(*export_table(t, dim * 4))
+        a = canonical_evicted(host_u64(ek[:cnt]), host_bytes(ev[:cnt], cnt, dim * 4), host_u64(es[:cnt]), gk)
+        b = canonical_evicted(oek, oev, oes, gk)
+        assert (a[0] == b[0]).all() and (a[1] == b[1]).all() and (a[2] == b[2]).all(), n
+        assert len(np.unique(host_u64(ek[:cnt]))) == cnt, n  # no entry claimed twice, none left out
+        batch += 1
+    assert_same_table(t, o, dim * 4)
+    t.close()
+
+
 # ---- config 5 at reduced capacity: EpochLRU, accum_or_assign, export_batch_if, erase -----------------------
 
 def test_config5_accum_export_erase(oracle):
