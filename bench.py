@@ -84,9 +84,12 @@ class HipEvent:
         return ms.value
 
     def __del__(self):
-        if self._e:
-            HipEvent._hip.hipEventDestroy(self._e)
-            self._e = None
+        try:
+            if self._e:
+                HipEvent._hip.hipEventDestroy(self._e)
+                self._e = None
+        except Exception:  # interpreter shutdown: the library may be gone already
+            pass
 
 
 def measured_traffic(kernel):
