@@ -193,23 +193,36 @@ zero_words_kernel(uint32_t* p, uint64_t n) {
   if (q * 4 < n) reinterpret_cast<uint4*>(p)[q] = make_uint4(0, 0, 0, 0);
 }
 
-/* The score bounds of an LRU table from scratch: for every line of 16 slots the lowest score of
- * its keys, but nothing above a value that no score written from now on is below (as
- * UpsertArgs::bound_cap), and 0 for a line without keys.  A free slot does not count: what it gets later
- * is a score of that time.  Eight lanes per line, one wavefront per 8 lines; the caller has
- * the table to itself. */
+/* What the score bounds are rebuilt against and where the limits of the next upsert live. */
+struct BoundsRebuild {
+  Clock clock;
+  int32_t strategy;
+  uint64_t epoch;
+  unsigned long long* clock_word;       /* hardware clock: gets a reading, which the upsert that
+                                           follows takes as its own limit (UpsertArgs::bound_cap_in) */
+  const unsigned long long* floor_word; /* scores from the caller: the lowest score of the batch
+                                           that is about to run (score_floor_kernel) */
+  unsigned long long* ceil_word;        /* with floor_word: gets the limit the bounds were made with */
+};
+
+/* The score bounds from scratch: for every line of 16 slots the lowest score of its keys, but
+ * nothing above a value that no score written from now on is below (as UpsertArgs::bound_cap),
+ * and 0 for a line without keys.  A free slot does not count: what it gets later is a score of
+ * that time.  Eight lanes per line, one wavefront per 8 lines; the caller has the table to
+ * itself. */
 __global__ void __launch_bounds__(256)
-rebuild_bounds_kernel(View v, Clock clock, unsigned long long* cap_word) {
+rebuild_bounds_kernel(View v, BoundsRebuild r) {
   const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  /* hardware clock: the upsert that follows takes its own limit for bounds from this word
-   * (UpsertArgs::bound_cap_in), which has no reading yet the first time */
-  if (t == 0 && cap_word) *cap_word = now_ns(clock, 0);
+  if (t == 0 && r.clock_word) *r.clock_word = now_ns(r.clock, 0);
+  /* deterministic clock: the base of the call that is about to run; hardware clock: now, which
+   * is before anything that call writes; scores from the caller: the lowest of that call */
+  uint64_t cap = r.clock.mode == 1 ? r.clock.base : now_ns(r.clock, 0);
+  if (r.strategy == HKV_EPOCH_LRU) cap = (r.epoch << 32) | ((cap >> 20) & kLow32);
+  if (r.floor_word) cap = *r.floor_word;
+  if (t == 0 && r.ceil_word) *r.ceil_word = cap;
   const uint64_t line = t >> 3;
   const int j = (int)(t & 7);
   if (line >= v.capacity / 16) return; /* whole tiles leave together: lines are a multiple of 8 */
-  /* deterministic clock: the base of the call that is about to run; hardware clock: now, which
-   * is before anything that call writes */
-  const uint64_t cap = clock.mode == 1 ? clock.base : now_ns(clock, 0);
   const uint4 k = *reinterpret_cast<const uint4*>(v.keys + line * 16 + j * 2);
   const uint4 s = *reinterpret_cast<const uint4*>(v.scores + line * 16 + j * 2);
   const uint64_t k0 = k.x | ((uint64_t)k.y << 32), k1 = k.z | ((uint64_t)k.w << 32);
@@ -221,6 +234,36 @@ rebuild_bounds_kernel(View v, Clock clock, unsigned long long* cap_word) {
   if (k1 != v.empty_key && s1 < m) m = s1;
   m = tile_min(m);
   if (j == 0) v.bounds[line] = m == kMaxScore ? 0 : (m < cap ? m : cap);
+}
+
+/* The lowest score a batch can leave in the table, for the strategies that take scores from the
+ * caller: Customized and LFU store the caller's score for a new key (an LFU key that is found
+ * ends above it), EpochLFU the epoch over its low half (kernel_utils.cuh:332-371, 464-517,
+ * 567-593).  `out` must hold kMaxScore when the kernel starts: `next`, the word the following
+ * call will use, is reset here, and the two words are used in turn.  Few, large workgroups:
+ * updates of one word are served one at a time. */
+__global__ void __launch_bounds__(1024)
+score_floor_kernel(const uint64_t* scores, uint64_t n, int strategy, uint64_t epoch,
+                   unsigned long long* out, unsigned long long* next) {
+  __shared__ unsigned long long s_part[16];
+  uint64_t m = kMaxScore;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    uint64_t x = scores[i];
+    if (strategy == HKV_EPOCH_LFU && epoch != kIgnoredEpoch) x = (epoch << 32) | (x & kLow32);
+    m = x < m ? x : m;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint64_t o = __shfl_xor((unsigned long long)m, off);
+    m = o < m ? o : m;
+  }
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); w++) m = s_part[w] < m ? s_part[w] : m;
+    __hip_atomic_fetch_min(out, (unsigned long long)m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (blockIdx.x == 0) *next = kMaxScore;
+  }
 }
 
 /* ---- built-in predicates (hkv_predicate) -------------------------------------- */

@@ -168,8 +168,12 @@ struct hkv_table {
   hkv_allocator alloc;
   void* d_meta;          /* digests + keys + scores + sizes + score bounds in one arena */
   std::atomic<uint64_t> keys_offered{0}; /* keys handed to upserts since creation or clear: above the size */
-  bool score_bounds;     /* LRU upserts search victims through the score bounds (HKV_SCORE_BOUNDS=0: off) */
+  bool score_bounds;     /* upserts into full buckets search victims through the score bounds
+                            (HKV_SCORE_BOUNDS=0: off; switched off for good once a score-writing call
+                            has been recorded into a HIP graph, see writes_scores_outside_bounds) */
   std::atomic<bool> bounds_stale{true}; /* a call may have written scores below the bounds */
+  uint64_t bounds_epoch = 0; /* EpochLRU: epoch and era (clock >> 52: the low half of such a score */
+  uint64_t bounds_era = 0;   /* wraps once per era) of the last call that used the bounds */
   uint64_t meta_bytes;
   void* d_values;        /* value rows in HBM */
   void* h_values;        /* host address of the pinned value rows (hybrid) */
@@ -191,6 +195,10 @@ struct hkv_table {
   bool locked_recount;     /* unlock_keys has run since the count was last read */
   unsigned long long* d_bound_caps; /* two device words: clock readings of the last calls that used the score bounds, used in turn */
   unsigned bound_cap_turn = 0;
+  unsigned long long* d_score_floor; /* two device words, used in turn: the lowest score of a batch (score_floor_kernel) */
+  unsigned score_floor_turn = 0;
+  unsigned long long* d_bound_ceil;  /* device word: no bound of the table is above it (strategies with scores from the caller) */
+  unsigned long long* d_load_sample; /* device word: the sum fast_load_factor reads back */
   unsigned long long* d_locked; /* device word: slots left LOCKED by those calls, less the unlocked */
   bool dual;               /* TableMode::kMemory: two candidate buckets per key */
   bool io_by_cpu;          /* value rows of the writers are moved by host threads */
@@ -475,6 +483,8 @@ int noalloc_scratch(int device, uint32_t** out) {
 }
 
 constexpr unsigned kCounterWords = 128;
+/* behind the counters: d_locked, d_bound_caps[2], d_score_floor[2], d_bound_ceil, d_load_sample */
+constexpr unsigned kExtraWords = 7;
 
 /* A device word for a call that returns a count.  The word belongs to the call from the
  * lease to its end (the call zeroes it on its stream, a kernel adds to it, the host reads it
@@ -540,7 +550,7 @@ int sync_clock(hkv_table* t) {
       t->clock.offset = t0 + (t1 - t0) / 2 - (uint64_t)ticks * t->clock.ns_per_tick;
     }
   }
-  HKV_HIP(hipMemset(d, 0, (kCounterWords + 3) * sizeof(unsigned long long)));
+  HKV_HIP(hipMemset(d, 0, (kCounterWords + kExtraWords) * sizeof(unsigned long long)));
   return HKV_SUCCESS;
 }
 
@@ -663,16 +673,20 @@ int reserve_impl(hkv_table* t, uint64_t new_capacity, hipStream_t s) {
  * 1024) buckets stand for the table; the incoming batch counts as all new */
 int fast_load_factor(hkv_table* t, uint64_t delta, hipStream_t s, float* out) {
   const uint32_t n = (uint32_t)std::min<uint64_t>(t->view.buckets_num, 1024);
-  CounterLease lease(t, s);
-  unsigned long long* d = lease.word();
+  /* A word of its own, not one of the leased counters: callers that hold a lease come through
+   * here (the count-returning insert_and_evict), and with all leases out they would wait for
+   * each other.  The kernel stores its whole result in one write, so callers that overlap read
+   * one or the other's sample of the same buckets, which serves the estimate as well. */
+  unsigned long long* d = t->d_load_sample;
   {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
     hipLaunchKernelGGL(partial_size_kernel, dim3(1), dim3(256), 0, s, t->view, n, d);
     HKV_HIP(hipGetLastError());
   }
-  uint64_t sum = 0;
-  HKV_TRY(lease.read(&sum));
+  unsigned long long sum = 0;
+  HKV_HIP(hipMemcpyAsync(&sum, d, sizeof sum, hipMemcpyDeviceToHost, s));
+  HKV_HIP(hipStreamSynchronize(s));
   *out = (float)((delta * 1.0) / (t->view.capacity * 1.0) + (sum * 1.0) / (kBucketSize * n * 1.0));
   return HKV_SUCCESS;
 }
@@ -703,8 +717,6 @@ int settle_locked_count(hkv_table* t, hipStream_t s) {
   return HKV_SUCCESS;
 }
 
-/* A call recorded into a HIP graph runs again with every replay: the pass that builds the score
- * bounds does not belong into one (the plain kernel is recorded instead while the bounds are stale). */
 bool capturing(hipStream_t s) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &st) != hipSuccess) {
@@ -712,6 +724,106 @@ bool capturing(hipStream_t s) {
     return false;
   }
   return st == hipStreamCaptureStatusActive;
+}
+
+/* A call that writes scores is about to run without looking after the score bounds (the plain
+ * upsert kernels, the two-phase path, lock_keys / find_and_update, assign on a table whose
+ * bounds are stale anyway).  The caller holds its role of the group lock, so this is ordered
+ * with the upsert that next rebuilds the bounds.
+ * - A call that is being recorded into a HIP graph runs again with every replay, at times the
+ *   library knows nothing of, with the scores, epoch and clock base of the day it was recorded:
+ *   from then on the table does without the bounds.
+ * - LRU and EpochLRU scores come from the clock and only grow, whichever kernel writes them
+ *   (`own_rule`: the call follows the table's strategy, i.e. no ignore_evict_strategy): the
+ *   bounds stay right.  Every other score may be below a bound: they are made again before
+ *   their next use. */
+void writes_scores_outside_bounds(hkv_table* t, hipStream_t s, bool own_rule) {
+  if (!t->score_bounds) return;
+  const int st = t->opts.evict_strategy;
+  if (capturing(s)) {
+    /* (a replay of an LRU call on the hardware clock writes the time of the replay, which is as
+     * good as any: such a table keeps its bounds; an epoch or a deterministic clock is recorded
+     * with its value of today) */
+    if (!(own_rule && st == HKV_LRU && t->clock.mode == 0)) t->score_bounds = false;
+    return;
+  }
+  if (own_rule && (st == HKV_LRU || st == HKV_EPOCH_LRU)) return;
+  t->bounds_stale = true;
+}
+
+uint64_t host_realtime_ns() {
+  struct timespec ts;
+  clock_gettime(CLOCK_REALTIME, &ts);
+  return (uint64_t)ts.tv_sec * UINT64_C(1000000000) + (uint64_t)ts.tv_nsec;
+}
+
+/* Whether this upsert searches victims through the score bounds, and with which limits (the
+ * fields of `a`); launches what has to run first (the batch's lowest score, the rebuild).  The
+ * caller holds the inserter role on `s`. */
+template <int OP>
+bool prepare_bounds(hkv_table* t, UpsertArgs& a, int vec, hipStream_t s) {
+  const int st = t->opts.evict_strategy;
+  if (!t->score_bounds || a.strategy != st || !(vec == 16 || OP == kOpFindOrInsertPtr)) return false;
+  /* The bounded search pays once buckets are full; a table that cannot be nine tenths full yet (it
+   * has not been offered that many keys since it was created or cleared) takes the plain kernel. */
+  if (t->keys_offered * 10 < t->view.capacity * 9) return false;
+  if (capturing(s)) return false; /* writes_scores_outside_bounds() then switches the bounds off */
+  const bool from_clock = st == HKV_LRU || st == HKV_EPOCH_LRU;
+  if (st == HKV_EPOCH_LRU) {
+    /* (epoch << 32) | (clock >> 20 & 0xFFFFFFFF) grows while the epoch does not go back and the low
+     * half does not wrap (every 2^52 ns); a call that may see the wrap happen, or a clock that
+     * cannot be read here, does without the bounds */
+    const uint64_t now = t->clock.mode == 1 ? t->clock.base : host_realtime_ns();
+    const uint64_t low = (now >> 20) & kLow32;
+    const uint64_t margin = t->clock.mode == 1 ? a.n + 1 : (UINT64_C(1) << 14); /* 2^14 * 2^20 ns = 17 s */
+    if (low + margin > kLow32 || (t->clock.mode == 0 && low < margin)) {
+      t->bounds_stale = true;
+      return false;
+    }
+    if (t->epoch < t->bounds_epoch || (t->epoch == t->bounds_epoch && (now >> 52) != t->bounds_era))
+      t->bounds_stale = true;
+    t->bounds_epoch = t->epoch;
+    t->bounds_era = now >> 52;
+  }
+  BoundsRebuild r{};
+  r.clock = t->clock;
+  r.strategy = st;
+  r.epoch = t->epoch;
+  if (from_clock) {
+    /* No bound may be above a score that this call writes.  Deterministic clock: the call's
+     * scores start at its base.  Hardware clock: they are later than the start of the last
+     * call of this kind, which that call left in a device word (this one leaves its own in
+     * the other word). */
+    a.bound_cap = t->clock.base;
+    if (t->clock.mode == 0) {
+      a.bound_cap_in = t->d_bound_caps + (t->bound_cap_turn & 1);
+      a.bound_cap_out = t->d_bound_caps + ((t->bound_cap_turn + 1) & 1);
+      t->bound_cap_turn++;
+      r.clock_word = const_cast<unsigned long long*>(a.bound_cap_in);
+    }
+  } else {
+    /* Scores from the caller: the limit is the lowest score this batch can leave behind, found
+     * by a pass over its scores; keys that write a score below the limits of earlier calls
+     * (d_bound_ceil) lower their line's bound themselves (hkv_upsert.hpp). */
+    unsigned long long* floor_word = t->d_score_floor + (t->score_floor_turn & 1);
+    unsigned long long* next_word = t->d_score_floor + ((t->score_floor_turn + 1) & 1);
+    t->score_floor_turn++;
+    const unsigned blocks = (unsigned)std::min<uint64_t>(64, (a.n + 8191) / 8192);
+    hipLaunchKernelGGL(score_floor_kernel, dim3(blocks), dim3(1024), 0, s, a.scores, a.n, st, t->epoch,
+                       floor_word, next_word);
+    a.bound_cap_in = floor_word;
+    a.bound_ceil = t->d_bound_ceil;
+    r.floor_word = floor_word;
+    r.ceil_word = t->d_bound_ceil;
+  }
+  /* bounds that were never set (a new or cleared table reaching this point) or that may be
+   * above a score (scores from outside the clock) are made from the scores as they are */
+  if (t->bounds_stale.exchange(false)) {
+    const uint64_t threads = t->view.capacity / 16 * 8;
+    hipLaunchKernelGGL(rebuild_bounds_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                       t->view, r);
+  }
+  return true;
 }
 
 /* `hybrid_rule`: the operation follows the lock-key kernels of hybrid mode when
@@ -725,8 +837,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
   a.value_kind = t->opts.value_kind;
   const bool refuse_equal = OP == kOpFindOrInsertPtr || (hybrid_rule && !t->pure_hbm);
   a.refuse_equal = refuse_equal;
-  /* scores that do not come from the table's clock may be lower than what the bounds say */
-  if (a.strategy != t->opts.evict_strategy) t->bounds_stale = true;
+  const bool own_rule = a.strategy == t->opts.evict_strategy;
   t->keys_offered += a.n;
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
@@ -742,6 +853,7 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
     /* a table that has been offered fewer keys than nine tenths of its slots evicts next to nothing */
     const bool pair = OP == kOpInsertAndEvict && t->keys_offered * 10 >= t->view.capacity * 9;
     if (two_phase) {
+      writes_scores_outside_bounds(t, s, own_rule);
       if constexpr (OP != kOpFindOrInsertPtr)
         HKV_TRY(run_two_phase<OP>(t, a, vec, refuse_equal, s));
     } else if (t->keys_may_be_locked) {
@@ -749,32 +861,12 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
        * be hidden from the victim scan, which then reads the key words beside the scores; with
        * no such slot the plain scan finds the same victims (a slot locked by another key of
        * the batch is retried instead of skipped) */
+      writes_scores_outside_bounds(t, s, own_rule);
       launch_upsert_for<OP, true>(pair, vec, t->view, a, s);
-    } else if (t->score_bounds && a.strategy == HKV_LRU && (vec == 16 || OP == kOpFindOrInsertPtr) &&
-               t->keys_offered * 10 >= t->view.capacity * 9 && !(t->bounds_stale && capturing(s))) {
-      /* LRU scores only grow, which is what keeps the score bounds right by themselves.  The
-       * bounded search pays once buckets are full; a table that cannot be nine tenths full yet
-       * (it has not been offered that many keys since it was created or cleared) takes the plain
-       * kernel, whose few evictions leave the bounds as they are, which is as right as before. */
-      /* No bound may be above a score that this call writes.  Deterministic clock: the call's
-       * scores start at its base.  Hardware clock: they are later than the start of the last
-       * call of this kind, which that call left in a device word (this one leaves its own in
-       * the other word). */
-      a.bound_cap = t->clock.base;
-      if (t->clock.mode == 0) {
-        a.bound_cap_in = t->d_bound_caps + (t->bound_cap_turn & 1);
-        a.bound_cap_out = t->d_bound_caps + ((t->bound_cap_turn + 1) & 1);
-        t->bound_cap_turn++;
-      }
-      /* bounds that were never set (a new or cleared table reaching this point) or that may be
-       * above a score (scores from outside the clock) are made from the scores as they are */
-      if (t->bounds_stale.exchange(false)) {
-        const uint64_t threads = t->view.capacity / 16 * 8;
-        hipLaunchKernelGGL(rebuild_bounds_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           t->view, t->clock, const_cast<unsigned long long*>(a.bound_cap_in));
-      }
+    } else if (prepare_bounds<OP>(t, a, vec, s)) {
       launch_upsert_for<OP, false, true>(pair, vec, t->view, a, s);
     } else {
+      writes_scores_outside_bounds(t, s, own_rule);
       launch_upsert_for<OP, false>(pair, vec, t->view, a, s);
     }
     HKV_HIP(hipGetLastError());
@@ -1119,7 +1211,7 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   {
     const char* b = getenv("HKV_SCORE_BOUNDS");
     /* only LRU keeps them right by itself (hkv_upsert.hpp); other tables carry none */
-    t->score_bounds = !(b && !strcmp(b, "0")) && t->opts.evict_strategy == HKV_LRU && !t->dual;
+    t->score_bounds = !(b && !strcmp(b, "0")) && !t->dual;
   }
   if (const char* e = getenv("HKV_UPSERT_PATH")) {
     if (!strcmp(e, "auto")) t->upsert_path = 0;
@@ -1207,16 +1299,22 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->pure_hbm = v.hbm_slots == v.capacity;
   void* cnt = nullptr;
   {
-    int rc = table_alloc(t, 0, &cnt, (kCounterWords + 3) * sizeof(unsigned long long));
+    int rc = table_alloc(t, 0, &cnt, (kCounterWords + kExtraWords) * sizeof(unsigned long long));
     if (rc) return bail(rc);
   }
   t->d_counters = (unsigned long long*)cnt;
   for (unsigned w = 0; w < kCounterWords; w++) t->counter_free.push_back(w);
   t->d_locked = t->d_counters + kCounterWords;
   t->d_bound_caps = t->d_counters + kCounterWords + 1;
+  t->d_score_floor = t->d_counters + kCounterWords + 3;
+  t->d_bound_ceil = t->d_counters + kCounterWords + 5;
+  t->d_load_sample = t->d_counters + kCounterWords + 6;
   {
     int rc = sync_clock(t);
     if (rc) return bail(rc);
+    /* score_floor_kernel takes the minimum into a word that holds the highest score */
+    if (hipMemset(t->d_score_floor, 0xFF, 2 * sizeof(unsigned long long)) != hipSuccess)
+      return bail(fail(HKV_ERROR_HIP, "hipMemset of the score floor words failed"));
   }
   t->reach_max_capacity = t->dual || o->init_capacity * 2 > o->max_capacity; /* merlin_hashtable.cuh:1064-1069 */
   *out = t;
@@ -1346,11 +1444,11 @@ int hkv_insert_or_assign_noalloc(hkv_table* t, uint64_t n, const uint64_t* keys,
   a.clock = t->clock;
   a.value_kind = t->opts.value_kind;
   a.refuse_equal = !t->pure_hbm; /* the lock-key rule of hybrid mode, as hkv_insert_or_assign */
-  if (a.strategy != t->opts.evict_strategy) t->bounds_stale = true;
   const int vec = pick_vec(t->view.value_bytes, {values});
   {
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
+    writes_scores_outside_bounds(t, s, a.strategy == t->opts.evict_strategy);
     /* slots left LOCKED by lock_keys are invisible to the second phase; whether any are left
      * after unlock_keys is settled by the next ordinary upsert (it reads a device counter) */
     if (t->keys_may_be_locked)
@@ -1549,6 +1647,7 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
       e = g.acquire();
       if (e == hipSuccess && touch_scores) {
         a.values = nullptr;
+        writes_scores_outside_bounds(t, s, true);
         launch_assign<false>(16, t->view, a, s);
         e = hipGetLastError();
       }
@@ -1575,6 +1674,13 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
   {
     LockGuard g(t, StreamGroupLock::kUpdater, s);
     HKV_HIP(g.acquire());
+    /* Customized: the caller's score replaces the old one and may be below the line's bound */
+    if (t->score_bounds && touch_scores && scores && a.strategy == HKV_CUSTOMIZED) {
+      if (t->bounds_stale || capturing(s))
+        writes_scores_outside_bounds(t, s, true);
+      else
+        a.bound_ceil = t->d_bound_ceil;
+    }
     if (lockfree)
       launch_assign<true>(vec, t->view, a, s);
     else
@@ -1708,6 +1814,7 @@ int hkv_lock_keys(hkv_table* t, uint64_t n, const uint64_t* keys, uint64_t** loc
     LockGuard g(t, StreamGroupLock::kInserter, s);
     HKV_HIP(g.acquire());
     t->keys_may_be_locked = true;
+    writes_scores_outside_bounds(t, s, true);
     hipLaunchKernelGGL((touch_kernel<true>), dim3(grid_for(n)), dim3(kWave), 0, s, t->view, a);
     HKV_HIP(hipGetLastError());
   }
@@ -1908,6 +2015,8 @@ uint64_t hkv_bucket_count(const hkv_table* t) { return t->view.buckets_num; }
 int hkv_is_pure_hbm(const hkv_table* t) { return t->pure_hbm; }
 
 int hkv_set_global_epoch(hkv_table* t, uint64_t epoch) {
+  /* scores of an earlier epoch are below what the score bounds were made for */
+  if (epoch < t->epoch && t->epoch != kIgnoredEpoch) t->bounds_stale = true;
   t->epoch = epoch;
   return HKV_SUCCESS;
 }

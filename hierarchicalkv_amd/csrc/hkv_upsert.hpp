@@ -73,6 +73,10 @@ struct UpsertArgs {
   uint64_t bound_cap;
   const unsigned long long* bound_cap_in;
   unsigned long long* bound_cap_out;
+  /* strategies whose scores come from the caller (Customized, LFU, EpochLFU): a device word that
+   * no bound of the table is above.  A key that writes a score below it lowers the bound of
+   * its line itself.  Null where scores only grow (LRU, EpochLRU). */
+  unsigned long long* bound_ceil;
 };
 
 /* ScoreFunctor<Strategy>::desired_when_missed, kernel_utils.cuh:275-279,
@@ -97,16 +101,16 @@ __device__ __forceinline__ uint64_t desired_when_missed(const UpsertArgs& a,
 /* ScoreFunctor<Strategy>::update_with_digest, kernel_utils.cuh:291-302,
  * 353-371, 422-434, 490-517, 581-593: digest and score of an accepted key.
  * The slot is locked by the caller. */
-__device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
-                                           uint64_t slot, uint32_t digest,
-                                           uint64_t desired, uint64_t in_score,
-                                           uint64_t i, bool new_insert) {
+__device__ __forceinline__ uint64_t write_meta(const View& v, const UpsertArgs& a,
+                                               uint64_t slot, uint32_t digest,
+                                               uint64_t desired, uint64_t in_score,
+                                               uint64_t i, bool new_insert) {
   const int STRATEGY = a.strategy;
   uint64_t s = desired;
   if (STRATEGY == HKV_LRU) {
     s = now_ns(a.clock, i);
   } else if (STRATEGY == HKV_LFU) {
-    if (!a.scores) return;
+    if (!a.scores) return kMaxScore;
     s = new_insert ? in_score : in_score + ld_u64(v.scores + slot);
   } else if (STRATEGY == HKV_EPOCH_LFU) {
     if (!new_insert) {
@@ -121,6 +125,7 @@ __device__ __forceinline__ void write_meta(const View& v, const UpsertArgs& a,
    * owner (the reference rewrites the same value, kernel_utils.cuh:296-300) */
   if (new_insert) st_u8(v.digests + slot, (uint8_t)digest);
   st_u64(v.scores + slot, s);
+  return s; /* what the slot holds now (kMaxScore above: nothing was written) */
 }
 
 /* wrapping adds of the 8- and 16-bit lanes of a word (signed and unsigned alike) */
@@ -613,10 +618,20 @@ upsert_kernel(View v, UpsertArgs a) {
   const uint64_t i = ((uint64_t)blockIdx.x * WAVES + wave) * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
 
-  uint64_t bound_cap = 0;
+  uint64_t bound_cap = 0, bound_ceil = 0;
   if constexpr (BOUNDS) {
     bound_cap = a.bound_cap_in ? *a.bound_cap_in : a.bound_cap;
     if (a.bound_cap_out && blockIdx.x == 0 && threadIdx.x == 0) *a.bound_cap_out = now_ns(a.clock, 0);
+    /* EpochLRU: the limit is a clock reading, the scores are made from it (kernel_utils.cuh:403-411) */
+    if (a.strategy == HKV_EPOCH_LRU) bound_cap = (a.epoch << 32) | ((bound_cap >> 20) & kLow32);
+    if (a.bound_ceil) {
+      /* the word is raised to this call's limit by one thread while the others read it: either
+       * value is one that no bound is above, the old bounds by the old value and the bounds this
+       * call sets by its limit */
+      const uint64_t c = *a.bound_ceil;
+      bound_ceil = c > bound_cap ? c : bound_cap;
+      if (blockIdx.x == 0 && threadIdx.x == 0 && bound_cap > c) *a.bound_ceil = bound_cap;
+    }
   }
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   const uint64_t in_score = (a.scores && i < a.n) ? a.scores[i] : 0;
@@ -836,7 +851,15 @@ upsert_kernel(View v, UpsertArgs a) {
        * the line's other scores */
       if (BOUNDS && (got == kStEvict || got == kStReclaimed))
         st_u64(v.bounds + (slot >> 4), new_bound < bound_cap ? new_bound : bound_cap);
-      write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
+      const uint64_t stored = write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
+      /* Scores from the caller may be below what the line's bound says: a key that goes into a
+       * free slot, and under Customized a key that was found (its score becomes the caller's; LFU
+       * and EpochLFU only add to it).  Such a key lowers the bound itself.  A key that takes a
+       * victim's slot cannot be below the victim's score, which the bound was not above, except
+       * under LFU, whose line has just been given a bound that no score of this call is below. */
+      if (BOUNDS && a.bound_ceil && stored < bound_ceil &&
+          (got == kStEmpty || (got == kStDuplicate && a.strategy == HKV_CUSTOMIZED)))
+        __hip_atomic_fetch_min(v.bounds + (slot >> 4), stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
     }
     if (OP == kOpInsertAndEvict && total) {
@@ -904,21 +927,25 @@ struct AssignArgs {
   Clock clock;
   int32_t touch_scores;
   int32_t strategy;
+  /* Customized tables with score bounds in use: the device word no bound is above (as
+   * UpsertArgs::bound_ceil); a key whose new score is below it lowers its line's bound */
+  const unsigned long long* bound_ceil;
 };
 
-__device__ __forceinline__ void assign_score(const View& v, const AssignArgs& a,
-                                             uint64_t slot, uint64_t i) {
+/* the score the slot holds afterwards; kMaxScore when it was left as it is */
+__device__ __forceinline__ uint64_t assign_score(const View& v, const AssignArgs& a,
+                                                 uint64_t slot, uint64_t i) {
   const int STRATEGY = a.strategy;
   uint64_t s;
   if (STRATEGY == HKV_LRU) {
     s = now_ns(a.clock, i);
   } else if (STRATEGY == HKV_LFU) {
-    if (!a.scores) return;
+    if (!a.scores) return kMaxScore;
     s = ld_u64(v.scores + slot) + a.scores[i];
   } else if (STRATEGY == HKV_EPOCH_LRU) {
     s = (a.epoch << 32) | ((now_ns(a.clock, i) >> 20) & kLow32);
   } else if (STRATEGY == HKV_EPOCH_LFU) {
-    if (!a.scores) return;
+    if (!a.scores) return kMaxScore;
     const uint64_t in = a.scores[i] & kLow32;
     s = ld_u64(v.scores + slot) & kLow32;
     if (kLow32 - s > in)
@@ -926,10 +953,11 @@ __device__ __forceinline__ void assign_score(const View& v, const AssignArgs& a,
     else
       s = (a.epoch << 32) | kLow32;
   } else {
-    if (!a.scores) return;
+    if (!a.scores) return kMaxScore;
     s = a.scores[i];
   }
   st_u64(v.scores + slot, s);
+  return s;
 }
 
 /* LOCKFREE: the call is the only writer on the table while it runs and its keys are unique,
@@ -945,6 +973,7 @@ assign_kernel(View v, AssignArgs a) {
   const int lane = threadIdx.x;
   const uint64_t i = (uint64_t)blockIdx.x * kWave + lane;
   const uint32_t units = v.value_bytes / VEC;
+  const uint64_t bound_ceil = a.bound_ceil ? *a.bound_ceil : 0;
   const uint64_t key = stage_keys(v, a.keys, a.n, i, s_meta, s_slot, lane);
   s_unsure[lane] = 0;
   __syncthreads();
@@ -976,7 +1005,11 @@ assign_kernel(View v, AssignArgs a) {
     }
     const bool locked = got == kStDuplicate;
     uint8_t* row = value_row(v, (uint64_t)(hit < 0 ? 0 : hit));
-    if (locked && a.touch_scores) assign_score(v, a, (uint64_t)hit, i);
+    if (locked && a.touch_scores) {
+      const uint64_t stored = assign_score(v, a, (uint64_t)hit, i);
+      if (a.bound_ceil && stored < bound_ceil)
+        __hip_atomic_fetch_min(v.bounds + ((uint64_t)hit >> 4), stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     if (a.values) {
       const int move = locked ? kMoveInToTable : kMoveNone;
       uint8_t* usr = const_cast<uint8_t*>(a.values) + i * v.value_bytes;

@@ -608,6 +608,54 @@ def test_reserve_keeps_the_map_and_doubles_until_the_limit(oracle):
     t.close()
 
 
+def test_set_max_capacity_scenario_of_the_reference(oracle):
+    # set_max_capacity (merlin_hashtable.cuh:3561-3579) by the reference's own scenario
+    # (tests/dynamic_max_capacity_test.cc.cu:39-134): fill a table of 2^12 slots that may grow to
+    # 2^14 with consecutive integer keys through insert_and_evict until it is 98 % full, raise the
+    # limit, reserve up to it (the capacity then equals the new limit and the load factor is at most
+    # a half), go on until the limit would pass 2^17; every key ever inserted is then either in the
+    # table or among the evicted ones, each with the row made from it, and the closed forms of the
+    # text: a limit that is not a power of two raises, one below the capacity changes nothing.
+    dim, n = 2, 2500
+    cap_limit, uplimit = 1 << 14, 1 << 17
+    o = default_options(init_capacity=1 << 12, max_capacity=cap_limit, dim=dim, max_load_factor=0.5,
+                        evict_strategy=EvictStrategy.kLru)
+    t = oracle.OracleTable(o)
+    t.set_clock(1, 1 << 40)
+    seen = {}
+    offset = 0
+    while True:
+        keys = np.arange(offset, offset + n, dtype=np.uint64)
+        ek, ev, _ = t.insert_and_evict(keys, vals_of(keys, dim), None)
+        offset += n
+        assert offset <= 2 * uplimit, "too many keys without filling the table"
+        for k, v in zip(ek.tolist(), ev):
+            seen[k] = v.tobytes()
+        if t.size() / t.capacity() >= 0.98:
+            assert t.capacity() == cap_limit  # grown by itself up to the limit, not past it
+            with pytest.raises(oracle.OracleError):
+                t.set_max_capacity(cap_limit * 2 + 2)  # not a power of two
+            t.set_max_capacity(cap_limit // 4)  # below the capacity: ignored
+            t.reserve(cap_limit * 2)
+            assert t.capacity() == cap_limit
+            cap_limit *= 2
+            if cap_limit > uplimit:
+                break
+            t.set_max_capacity(cap_limit)
+            t.reserve(cap_limit)
+            assert t.capacity() == cap_limit
+            assert t.size() / t.capacity() <= 0.5
+    k, v, _ = t.export_all()
+    for key, row in zip(k.tolist(), v):
+        seen[key] = row.tobytes()
+    assert t.capacity() * 2 == cap_limit
+    assert len(seen) >= t.capacity() * 0.98
+    assert sorted(seen) == list(range(offset))  # nothing lost, nothing made up
+    want = vals_of(np.array(sorted(seen), dtype=np.uint64), dim)
+    assert all(seen[key] == want[i].tobytes() for i, key in enumerate(sorted(seen)))
+    t.close()
+
+
 # ---- lock_keys / unlock_keys / find_and_update ---------------------------------------
 
 def test_lock_unlock_truth_table(oracle):

@@ -1,6 +1,8 @@
-"""The score bounds of LRU tables (hkv_table_view::bounds): for every line of 16 slots a value that
-is not above any score in the line, which the LRU upserts use to find a bucket's lowest score from
-one or two of its eight score lines.  Checked here:
+"""The score bounds of a table (hkv_table_view::bounds): for every line of 16 slots a value that
+is not above any score in the line, which the upserts use to find a bucket's lowest score from
+one or two of its eight score lines.  LRU and EpochLRU scores only grow, so their bounds stay right
+by themselves; under Customized, LFU and EpochLFU a key that writes a score below its line's bound
+lowers the bound itself.  Checked here:
   * the invariant itself, read back from device memory after mixed call sequences, on the
     deterministic and on the hardware clock (a bound above a score would send an eviction to the
     wrong slot sooner or later);
@@ -40,9 +42,9 @@ def bounds_hold(t):
     return len(bad) == 0, bad[:5], int((bounds > 0).sum())
 
 
-def make(cap, dim, **kw):
+def make(cap, dim, strategy=EvictStrategy.kLru, **kw):
     o = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 30, dim=dim,
-                        evict_strategy=EvictStrategy.kLru, **kw)
+                        evict_strategy=strategy, **kw)
     t = HashTable()
     t.init(o)
     return t, o
@@ -143,4 +145,291 @@ def test_scores_from_outside_the_clock(oracle):
         ot.insert_or_assign(k, bytes_of(v), None)
         assert bounds_hold(t)[0]
         assert_same_table(t, ot, dim * 4)
+    t.close()
+
+
+@pytest.mark.parametrize("dim", [64, 128])
+def test_bounded_kernels_with_wide_rows(oracle, dim):
+    """The bounded search in the instantiations that move rows of 256 and 512 bytes (two and four
+    16-byte units per lane, which is what a table of dim 64 / 128 runs): insert_or_assign,
+    find_or_insert, insert_and_evict (two wavefronts per workgroup) and accum_or_assign on a table
+    filled past load factor 1.0, LRU on the deterministic clock, every call against the oracle."""
+    from gpu_util import canonical_evicted, export_table, host_bytes, host_u64, sort_by_key
+    cap, bs = 1 << 14, 3000
+    t, o = make(cap, dim)
+    ot = oracle.OracleTable(o)
+    t.set_clock(1, 1 << 44)
+    ot.set_clock(1, 1 << 44)
+    seed, pos = 630 + dim, 0
+    vb = dim * 4
+    while pos < cap + 4 * bs:  # past load factor 1.0: the last batches evict
+        k = w.unique_keys(seed, pos, bs)
+        v = w.uniform_values(seed, pos, bs, dim)
+        t.insert_or_assign(bs, dev(k), dev(v))
+        ot.insert_or_assign(k, bytes_of(v), None)
+        pos += bs
+    assert t.size() == ot.size()
+    assert_same_table(t, ot, vb)
+    ok, _, n_tight = bounds_hold(t)
+    assert ok and n_tight > 0  # the bounded kernel has been at work
+    for rep in range(3):
+        # insert_or_assign: half from the latest batch (highest scores: no key of this batch can
+        # evict one of them before its turn), half new
+        k = np.concatenate([w.unique_keys(seed, pos - bs // 2, bs // 2), w.unique_keys(seed, pos, bs // 2)])
+        pos += bs // 2
+        v = w.uniform_values(seed + 1, pos, len(k), dim)
+        t.insert_or_assign(len(k), dev(k), dev(v))
+        ot.insert_or_assign(k, bytes_of(v), None)
+        assert_same_table(t, ot, vb)
+        # find_or_insert: the same mix; hits hand their rows back, misses insert
+        k = np.concatenate([w.unique_keys(seed, pos - bs // 2, bs // 2), w.unique_keys(seed, pos, bs // 2)])
+        pos += bs // 2
+        v = w.uniform_values(seed + 2, pos, len(k), dim)
+        dv = dev(v)
+        t.find_or_insert(len(k), dev(k), dv)
+        ov = bytes_of(v).copy()
+        ot.find_or_insert(k, ov, None)
+        torch.cuda.synchronize()
+        assert (host_bytes(dv, len(k), vb) == ov).all()
+        assert_same_table(t, ot, vb)
+        # insert_and_evict: evicted keys, rows and scores
+        k = np.concatenate([w.unique_keys(seed, pos - bs // 2, bs // 2), w.unique_keys(seed, pos, bs // 2 + 37)])
+        pos += bs // 2 + 37
+        n = len(k)
+        v = w.uniform_values(seed + 3, pos, n, dim)
+        ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+        ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        es = torch.zeros(n, dtype=torch.int64, device=DEV)
+        cnt = t.insert_and_evict(n, dev(k), dev(v), None, ek, ev, es)
+        oek, oev, oes = ot.insert_and_evict(k, bytes_of(v), None)
+        assert cnt == len(oek) and cnt > 0
+        gk, _, _ = sort_by_key(*export_table(t, vb))
+        a = canonical_evicted(host_u64(ek[:cnt]), host_bytes(ev[:cnt], cnt, vb), host_u64(es[:cnt]), gk)
+        b = canonical_evicted(oek, oev, oes, gk)
+        assert (a[0] == b[0]).all() and (a[1] == b[1]).all() and (a[2] == b[2]).all()
+        assert_same_table(t, ot, vb)
+        # accum_or_assign: recent keys accumulate, new keys are assigned, flags from contains
+        k = np.concatenate([w.unique_keys(seed, pos - bs // 2, bs // 2), w.unique_keys(seed, pos, bs // 2)])
+        pos += bs // 2
+        d = (w.uniform_values(seed + 4, pos, len(k), dim) * np.float32(0.01)).astype(np.float32)
+        founds = torch.zeros(len(k), dtype=torch.bool, device=DEV)
+        t.contains(len(k), dev(k), founds)
+        torch.cuda.synchronize()
+        flags = founds.cpu().numpy()
+        assert (flags == ot.contains(k)).all() and flags.any() and not flags.all()
+        t.accum_or_assign(len(k), dev(k), dev(d), founds)
+        ot.accum_or_assign(k, bytes_of(d), flags.astype(np.uint8))
+        assert_same_table(t, ot, vb)
+        ok, bad, _ = bounds_hold(t)
+        assert ok, (rep, bad)
+    t.close()
+
+
+# ---- strategies whose scores come from the caller, and EpochLRU ---------------------------------
+
+def upsert(t, ot, k, v, sc):
+    t.insert_or_assign(len(k), dev(k), dev(v), dev(sc))
+    ot.insert_or_assign(k, bytes_of(v), sc)
+
+
+def one_per_bucket(oracle, keys, buckets):
+    """The first key of `keys` for every bucket that any of them falls into."""
+    seen, keep = set(), []
+    for i, k in enumerate(keys.tolist()):
+        b = oracle.locate(k, buckets)[0]
+        if b not in seen:
+            seen.add(b)
+            keep.append(i)
+    return keys[np.array(keep)]
+
+
+def test_customized_scores_that_go_down(oracle):
+    """Customized: a key that is found gets the caller's score, which may be far below the one it
+    had, through insert_or_assign, find_or_insert and assign_scores; a key that goes into a free slot
+    may bring any score.  The bounds must follow, or the next evictions take the wrong keys."""
+    cap, dim, bs = 1 << 13, 4, 2048
+    t, o = make(cap, dim, EvictStrategy.kCustomized)
+    ot = oracle.OracleTable(o)
+    vb = dim * 4
+    seed, pos, batch = 640, 0, 10
+    while pos < cap + 4 * bs:  # past load factor 1.0 with growing scores
+        k = w.unique_keys(seed, pos, bs)
+        upsert(t, ot, k, w.values_from_keys(k, dim), w.monotone_scores(batch, bs, seed=64))
+        pos += bs
+        batch += 1
+    assert_same_table(t, ot, vb)
+    ok, bad, n_tight = bounds_hold(t)
+    assert ok and n_tight > cap // 16 // 4, (bad, n_tight)
+
+    def residents_by_score():
+        k, _, sc = ot.export_all()
+        return k[np.argsort(sc)]
+
+    # the best-scored residents get the lowest scores of the table (hits only: nothing is evicted)
+    top = residents_by_score()[-1500:]
+    a, b_, c = top[:500], top[500:1000], top[1000:]
+    upsert(t, ot, a, w.values_from_keys(a, dim) + 1, np.arange(1, 501, dtype=np.uint64))
+    assert bounds_hold(t)[0]
+    t.assign_scores(len(b_), dev(b_), dev(np.arange(501, 1001, dtype=np.uint64)))
+    ot.assign_scores(b_, np.arange(501, 1001, dtype=np.uint64))
+    assert bounds_hold(t)[0]
+    v = w.values_from_keys(c, dim)
+    dv = dev(v)
+    t.find_or_insert(len(c), dev(c), dv, dev(np.arange(1001, 1501, dtype=np.uint64)))
+    ov = bytes_of(v).copy()
+    ot.find_or_insert(c, ov, np.arange(1001, 1501, dtype=np.uint64))
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    # free slots taken with scores below everything else (one key per bucket: two such keys in a
+    # full bucket would evict each other in an order that nothing fixes)
+    gone = residents_by_score()[2000:2600]
+    t.erase(len(gone), dev(gone))
+    ot.erase(gone)
+    k = one_per_bucket(oracle, w.unique_keys(seed + 1, 0, 400), cap // 128)
+    upsert(t, ot, k, w.values_from_keys(k, dim), np.arange(2001, 2001 + len(k), dtype=np.uint64))
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    # new keys with high scores: the low ones go first, through all three inserting calls
+    for rep in range(4):
+        k = w.unique_keys(seed + 2, rep * 900, 900)
+        v = w.values_from_keys(k, dim)
+        sc = w.monotone_scores(batch, len(k), seed=64)
+        batch += 1
+        if rep % 2 == 0:
+            ek = torch.zeros(len(k), dtype=torch.int64, device=DEV)
+            ev = torch.zeros(len(k), dim, dtype=torch.float32, device=DEV)
+            es = torch.zeros(len(k), dtype=torch.int64, device=DEV)
+            cnt = t.insert_and_evict(len(k), dev(k), dev(v), dev(sc), ek, ev, es)
+            oek, _, oes = ot.insert_and_evict(k, bytes_of(v), sc)
+            assert cnt == len(oek)
+            got = sorted(zip(ek[:cnt].cpu().numpy().view(np.uint64).tolist(),
+                             es[:cnt].cpu().numpy().view(np.uint64).tolist()))
+            assert got == sorted(zip(oek.tolist(), oes.tolist()))
+        else:
+            upsert(t, ot, k, v, sc)
+        ok, bad, _ = bounds_hold(t)
+        assert ok, (rep, bad)
+        assert_same_table(t, ot, vb)
+    # a batch whose own scores are below the last batches': its bounds may not go above them
+    k = w.unique_keys(seed + 3, 0, 900)
+    upsert(t, ot, k, w.values_from_keys(k, dim), w.monotone_scores(5, len(k), seed=64))  # all refused or low
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    k = w.unique_keys(seed + 4, 0, 900)
+    upsert(t, ot, k, w.values_from_keys(k, dim), w.monotone_scores(batch, len(k), seed=64))
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLfu, EvictStrategy.kEpochLfu])
+def test_frequency_scores_and_bounds(oracle, strategy):
+    """LFU / EpochLFU: a new key comes in with the caller's count, which under LFU may be below
+    everything in its bucket (LFU never refuses); a key that is found only gains.  EpochLFU scores
+    go down when the epoch is set back."""
+    cap, dim, bs = 1 << 13, 4, 2048
+    t, o = make(cap, dim, strategy)
+    ot = oracle.OracleTable(o)
+    vb = dim * 4
+    epoch_lfu = strategy == EvictStrategy.kEpochLfu
+    if epoch_lfu:
+        t.set_global_epoch(3)
+        ot.set_global_epoch(3)
+
+    def distinct(b, n):
+        return (np.uint64(b + 1) << np.uint64(20)) + np.random.Generator(np.random.PCG64(b)).permutation(n).astype(np.uint64)
+    seed, pos, batch = 650, 0, 0
+    while pos < cap + 4 * bs:
+        k = w.unique_keys(seed, pos, bs)
+        upsert(t, ot, k, w.values_from_keys(k, dim), distinct(batch, bs))
+        pos += bs
+        batch += 1
+    assert_same_table(t, ot, vb)
+    ok, bad, n_tight = bounds_hold(t)
+    assert ok and n_tight > cap // 16 // 4, (bad, n_tight)
+    # hits only: counts go up
+    k = w.unique_keys(seed, pos - bs, bs)
+    present = ot.contains(k)
+    k = k[present]
+    upsert(t, ot, k, w.values_from_keys(k, dim) + 2, distinct(40, len(k)))
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    if epoch_lfu:
+        t.set_global_epoch(2)  # back: whatever is written now is below the rest
+        ot.set_global_epoch(2)
+    # new keys with counts below everything, one per bucket
+    k = one_per_bucket(oracle, w.unique_keys(seed + 1, 0, 300), cap // 128)
+    upsert(t, ot, k, w.values_from_keys(k, dim), np.arange(1, len(k) + 1, dtype=np.uint64))
+    assert_same_table(t, ot, vb)
+    if epoch_lfu:
+        t.set_global_epoch(5)
+        ot.set_global_epoch(5)
+    # and new keys with high counts: under LFU the low ones above are what goes
+    for rep in range(3):
+        k = w.unique_keys(seed + 2, rep * 900, 900)
+        upsert(t, ot, k, w.values_from_keys(k, dim), distinct(50 + rep, len(k)))
+        ok, bad, _ = bounds_hold(t)
+        assert ok, (rep, bad)
+        assert_same_table(t, ot, vb)
+    t.close()
+
+
+def test_epoch_lru_bounds(oracle):
+    """EpochLRU scores are (epoch << 32) | low half of clock >> 20: they grow while the epoch does
+    not go back and the low half does not wrap.  Both are made to happen."""
+    cap, dim, bs = 1 << 13, 4, 2048
+    t, o = make(cap, dim, EvictStrategy.kEpochLru)
+    ot = oracle.OracleTable(o)
+    vb = dim * 4
+    base = 1 << 44
+    t.set_clock(1, base)
+    ot.set_clock(1, base)
+    seed, pos = 660, 0
+
+    def epoch(e):
+        t.set_global_epoch(e)
+        ot.set_global_epoch(e)
+
+    def step(n=bs, both=False):
+        nonlocal pos
+        k = w.unique_keys(seed, pos, n)
+        if both:  # half from the latest batch, half new
+            k = np.concatenate([w.unique_keys(seed, pos - n // 2, n // 2), k[: n - n // 2]])
+        pos += n
+        upsert(t, ot, k, w.values_from_keys(k, dim), None)
+
+    epoch(1)
+    while pos < cap + 3 * bs:
+        step()
+    assert_same_table(t, ot, vb)
+    ok, bad, n_tight = bounds_hold(t)
+    assert ok and n_tight > cap // 16 // 4, (bad, n_tight)
+    epoch(2)
+    for _ in range(3):
+        step(both=True)
+        assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    epoch(1)  # back: new scores below the old ones
+    for _ in range(2):
+        step()
+        assert bounds_hold(t)[0]
+        assert_same_table(t, ot, vb)
+    epoch(3)
+    step()  # (the latest batch holds low scores now: not what a batch should look for and evict at once)
+    step(both=True)
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
+    # the low half of the clock wraps inside a call, and between calls
+    wrap = (0xFFFFFFFF - 1000) << 20
+    t.set_clock(1, wrap)
+    ot.set_clock(1, wrap)
+    for _ in range(2):  # the deterministic clock moves on by 2^40 ns = 2^20 units per call
+        step()
+        assert_same_table(t, ot, vb)
+    epoch(4)  # above everything again, on the new side of the wrap
+    step()
+    assert bounds_hold(t)[0]
+    step(both=True)
+    assert bounds_hold(t)[0]
+    assert_same_table(t, ot, vb)
     t.close()
