@@ -683,12 +683,15 @@ upsert_kernel(View v, UpsertArgs a) {
           got = kStDuplicate;
           pos = (uint32_t)(hit - (int64_t)bslot);
           victim = key;
-        } else if (seen != v.locked_key) {
-          /* the slot belongs to another key now: ours was evicted in this
-           * batch, or the probe was looking at somebody else's lock */
+        } else {
+          /* The slot belongs to another key now (ours was evicted in this batch, or the probe
+           * was looking at somebody else's lock), or it is LOCKED: by a key of this batch that is
+           * taking it over or about to give it back, or for good (lock_keys, a batch-mate of
+           * the pointer overload that keeps its slots).  The second probe finds out which,
+           * and its waiting is bounded. */
           hit = -1;
           reprobe = true;
-        } /* else: the hit slot is locked by somebody else right now; next trip */
+        }
       } else if (em_lo | em_hi) {
         /* up to three free slots, the first at or after the key's start position
          * so that keys of one bucket spread over the free slots */
@@ -997,9 +1000,11 @@ assign_kernel(View v, AssignArgs a) {
         uint64_t seen = key;
         if (LOCKFREE || cas_lock(v.keys + hit, seen, v.locked_key)) {
           got = kStDuplicate;
-        } else if (seen != v.locked_key) {
+        } else {
+          /* the slot changed hands or is LOCKED (another updater for a moment, lock_keys for
+           * good): look again, for a bounded time */
           hit = -1;
-          reprobe = true; /* the slot changed hands: look again */
+          reprobe = true;
         }
       }
     }

@@ -756,6 +756,10 @@ def test_find_or_insert_with_locked_key_pointers(oracle):
     keys = w.unique_keys(95, 0, bs)
     vals = w.values_from_keys(keys, dim)
     sc = w.monotone_scores(1, bs)
+    # the keys that the batch below finds again hold the highest scores: a key of that batch that
+    # evicts cannot take one of them before its own turn (it would come back as a new key, which is
+    # one of the outcomes a concurrent batch may have, but not the one the oracle's order gives)
+    sc[:1000] += np.uint64(1 << 39)
     t.insert_or_assign(bs, dev(keys), dev(vals), dev(sc))
     o.insert_or_assign(keys, vals.view(np.uint8).reshape(bs, -1), sc)
     n = 3000
