@@ -53,7 +53,10 @@ class HipEvent:
     """A HIP event for timing only, created with hipEventDisableSystemFence: recording it does not
     write the caches back and invalidate them, as the events torch creates do, so the kernel after
     it starts as it would with no event there (hip_runtime_api.h says as much of the flag).  The
-    timed region ends with a device synchronisation, after which the time stamps are read."""
+    timed region ends with a device synchronisation, after which the time stamps are read.
+    Two uses: record() puts the event on the stream between two calls; a pair handed to the
+    library (hkv_time_next_kernel) is attached to one kernel launch and gets the start and the end
+    of that kernel's execution, which is what a profiler's trace reports for it."""
     _hip = None
 
     def __init__(self, torch):
@@ -70,6 +73,10 @@ class HipEvent:
         rc = HipEvent._hip.hipEventCreateWithFlags(C.byref(self._e), 0x20000000)  # hipEventDisableSystemFence
         if rc:
             raise RuntimeError("hipEventCreateWithFlags: %d" % rc)
+
+    @property
+    def handle(self):
+        return self._e
 
     def record(self):
         rc = HipEvent._hip.hipEventRecord(self._e, self._C.c_void_p(self._torch.cuda.current_stream().cuda_stream))
@@ -109,6 +116,13 @@ def main():
     ap.add_argument("--dim", type=int, default=64)
     ap.add_argument("--batch-log2", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--strategy", choices=["lru", "customized", "epochlru"], default="lru",
+                    help="eviction strategy of the table (the headline workload is LRU; customized: scores "
+                         "(call number << 40) | index from the caller, epochlru: one epoch)")
+    ap.add_argument("--kernel-events", action="store_true",
+                    help="time each kernel by an event pair it is launched with (hkv_time_next_kernel: start and "
+                         "end of its execution, what a profiler's trace reports) instead of by events recorded "
+                         "on the stream between the calls; launches made that way cost the step about 8 us")
     ap.add_argument("--warm-keys", action="store_true",
                     help="resident keys of a step = keys written by the previous step")
     ap.add_argument("--calibrate", action="store_true",
@@ -188,11 +202,24 @@ def main():
     seed = 0x484B5600
     K, W = args.steps, args.warmup
 
+    strategy = {"lru": EvictStrategy.kLru, "customized": EvictStrategy.kCustomized,
+                "epochlru": EvictStrategy.kEpochLru}[args.strategy]
     opts = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * vb,
-                           dim=dim, evict_strategy=EvictStrategy.kLru)
+                           dim=dim, evict_strategy=strategy)
     table = HashTable()
     table.init(opts)
     assert table.is_pure_hbm()
+    if args.strategy == "epochlru":
+        table.set_global_epoch(1)
+    call_no = [0]
+    index = torch.arange(n, dtype=torch.int64, device=dev)
+
+    def next_scores():
+        """Customized: distinct scores that grow from call to call, made on the device."""
+        if args.strategy != "customized":
+            return None
+        call_no[0] += 1
+        return index + (call_no[0] << 40)
 
     def d64(a):
         return torch.from_numpy(a.view(np.int64)).to(dev)
@@ -209,7 +236,7 @@ def main():
         for _ in range(max(1, (cap // n) // 8)):
             keys = w.unique_keys(seed, pos, n)
             vals.uniform_(-1.0, 1.0)
-            table.insert_or_assign(n, d64(keys), vals)
+            table.insert_or_assign(n, d64(keys), vals, next_scores())
             prefill_starts.append(pos)
             pos += n
         size0 = table.size()
@@ -248,16 +275,31 @@ def main():
     out_vals = torch.empty(n, dim, dtype=torch.float32, device=dev)
     founds = torch.empty(n, dtype=torch.bool, device=dev)
 
-    # two events per step: the one after a step's insert_or_assign is the one before the next
-    # step's find (a loop records the one before its first step itself)
+    # The calls of a step are timed by events recorded on the stream between them (one after each
+    # call; the one after a step's insert_or_assign is the one before the next step's find), so
+    # each figure holds one gap between launches, 2 to 3 us.  With --kernel-events every kernel
+    # is launched with an event pair of its own instead (hkv_time_next_kernel): the runtime stamps
+    # it with the start and the end of the kernel's execution, which is what rocprofv3's trace
+    # reports, but launches made that way cost the step about 8 us of wall time.
+    from hierarchicalkv_amd._capi import lib as hkv_lib
+    ev_find = [(HipEvent(torch), HipEvent(torch)) for _ in range(steps)]
+    ev_ins = [(HipEvent(torch), HipEvent(torch)) for _ in range(steps)]
     ev_edge = [HipEvent(torch) for _ in range(steps + 1)]
     ev_mid = [HipEvent(torch) for _ in range(steps)]
 
+    step_scores = [next_scores() for _ in range(steps)]
+
     def step(s):
+        if (not args.kernel_events):
+            table.find(n, find_keys[s], out_vals, founds)
+            ev_mid[s].record()
+            table.insert_or_assign(n, ins_keys[s], ins_vals, step_scores[s])
+            ev_edge[s + 1].record()
+            return
+        hkv_lib.hkv_time_next_kernel(ev_find[s][0].handle, ev_find[s][1].handle)
         table.find(n, find_keys[s], out_vals, founds)
-        ev_mid[s].record()
-        table.insert_or_assign(n, ins_keys[s], ins_vals)
-        ev_edge[s + 1].record()
+        hkv_lib.hkv_time_next_kernel(ev_ins[s][0].handle, ev_ins[s][1].handle)
+        table.insert_or_assign(n, ins_keys[s], ins_vals, step_scores[s])
 
     if args.calibrate:
         cal = torch.empty(2, 1 << 28, dtype=torch.float32, device=dev)
@@ -278,8 +320,12 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
 
-    find_ms = [ev_edge[s].elapsed_time(ev_mid[s]) for s in range(W, steps)]
-    ups_ms = [ev_mid[s].elapsed_time(ev_edge[s + 1]) for s in range(W, steps)]
+    if (not args.kernel_events):
+        find_ms = [ev_edge[s].elapsed_time(ev_mid[s]) for s in range(W, steps)]
+        ups_ms = [ev_mid[s].elapsed_time(ev_edge[s + 1]) for s in range(W, steps)]
+    else:
+        find_ms = [ev_find[s][0].elapsed_time(ev_find[s][1]) for s in range(W, steps)]
+        ups_ms = [ev_ins[s][0].elapsed_time(ev_ins[s][1]) for s in range(W, steps)]
     find_avg = sum(find_ms) / K
     ups_avg = sum(ups_ms) / K
     size1 = table.size()
@@ -291,10 +337,16 @@ def main():
     ups_gbs = ub / (ups_avg * 1e-3) / 1e9
 
     default_workload = (args.capacity_log2 == 26 and dim == 64 and args.batch_log2 == 20
-                        and not args.warm_keys)
+                        and not args.warm_keys and args.strategy == "lru")
     path = os.environ.get("HKV_UPSERT_PATH", "locked")
     ups_traffic = measured_traffic("upsert_kernel") if default_workload and path == "locked" else None
     find_traffic = measured_traffic("lookup_kernel") if default_workload else None
+    timed_by = ("events on the stream around each call" if (not args.kernel_events) else
+                "the event pair each kernel is launched with (start and end of its execution)")
+
+    def traffic_frac(traffic, ms):
+        return None if traffic is None else round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+
     result = {
         "metric": "billion-KV/s for find & insert_or_assign, dim 64, load factor 1.0, 1 GPU",
         "value": round(value, 4),
@@ -310,7 +362,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"capacity 2^{args.capacity_log2}, dim {dim} fp32, batch 2^{args.batch_log2}, "
-                        "LRU, load factor 1.0; step = find (100% hit) + insert_or_assign (50% new)",
+                        f"{args.strategy.upper() if args.strategy == 'lru' else args.strategy}, load factor 1.0; "
+                        "step = find (100% hit) + insert_or_assign (50% new)",
             "load_factor": round(size0 / cap, 4),
             "find_hit_rate": round(hit_rate, 4),
             "size_before": size0,
@@ -323,15 +376,22 @@ def main():
                  "bkvs_2p30": round(n / (find_avg * 1e-3) / 2**30, 4)},
         "insert_or_assign": {"ms": round(ups_avg, 4), "bkvs": round(n / (ups_avg * 1e-3) / 1e9, 4),
                              "bkvs_2p30": round(n / (ups_avg * 1e-3) / 2**30, 4)},
+        # frac: algorithmic bytes / kernel time / peak; traffic_frac: the bytes the counters saw
+        # moving (FETCH_SIZE + WRITE_SIZE of the same workload, profiles/) / kernel time / peak.
+        # The bounded victim search moves fewer bytes than the algorithmic figure bills (it reads
+        # one or two of a bucket's eight score lines), find moves more (whole 128-byte lines for
+        # 8-byte key verifications).
         "roofline": {"kernel": "upsert_kernel<insert_or_assign>" if path == "locked" else
                      "two-phase upsert: upsert_hits_kernel + chained_miss_kernel", "bound": "hbm",
                      "achieved": round(ups_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": ups_traffic,
-                     "bytes_per_key": upsert_bytes(vb, 0.5)},
+                     "traffic_frac": traffic_frac(ups_traffic, ups_avg),
+                     "bytes_per_key": upsert_bytes(vb, 0.5), "timed_by": timed_by},
         "roofline_find": {"kernel": "lookup_kernel<values>", "bound": "hbm",
                           "achieved": round(find_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": round(find_gbs / HBM_PEAK_GBS, 4), "traffic": find_traffic,
-                          "bytes_per_key": find_bytes(vb)},
+                          "traffic_frac": traffic_frac(find_traffic, find_avg),
+                          "bytes_per_key": find_bytes(vb), "timed_by": timed_by},
     }
     table.close()
     del find_keys, ins_keys, ins_vals, out_vals

@@ -123,6 +123,7 @@ SIGNATURES = {
     "hkv_lock_end": (_i, [_T, _i, _p]),
     "hkv_set_clock": (_i, [_T, _i, _u64]),
     "hkv_scores_changed": (_i, [_T]),
+    "hkv_time_next_kernel": (_i, [C.c_void_p, C.c_void_p]),
 }
 
 

@@ -7,6 +7,7 @@
  * the stream-ordered group lock, and the choice of kernel instance per call.
  */
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <atomic>
@@ -326,6 +327,22 @@ int accum_unit(uint32_t value_bytes, const void* p, int kind) {
   return unit >= (int)elem[kind] ? unit : 0;
 }
 
+/* hkv_time_next_kernel: the pair of events that the calling thread's next main kernel (the one
+ * kernel of a find or of an upsert-family call) is launched with.  The runtime stamps them with
+ * the start and the end of that kernel's execution, so the time between them is the kernel's own,
+ * without the gaps between the launches of a stream that events recorded around a call include. */
+thread_local hipEvent_t g_time_start = nullptr, g_time_stop = nullptr;
+
+template <class... KArgs, class... Args>
+void launch_main(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t s, Args... args) {
+  if (g_time_start) {
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, s, g_time_start, g_time_stop, 0, args...);
+    g_time_start = g_time_stop = nullptr;
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, args...);
+  }
+}
+
 /* BOUNDS: the victim search reads the bucket's score bounds and one or two of its score lines
  * instead of all eight (hkv_upsert.hpp); for 16-byte units, which is what tables with rows of a
  * multiple of 16 bytes use. */
@@ -335,30 +352,30 @@ void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   if constexpr (OP == kOpAccumOrAssign && !BOUNDS) {
     /* the two units that only the element-wise add needs */
     if (vec == 8) {
-      hipLaunchKernelGGL((upsert_kernel<OP, 8, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
+      launch_main(upsert_kernel<OP, 8, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
       return;
     }
     if (vec == 2) {
-      hipLaunchKernelGGL((upsert_kernel<OP, 2, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
+      launch_main(upsert_kernel<OP, 2, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
       return;
     }
   }
   if (OP == kOpFindOrInsertPtr) {
-    hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a);
+    launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a);
     return;
   }
   if (vec == 16) {
     switch (pick_upl(v.value_bytes, 16)) {
-      case 1: hipLaunchKernelGGL((upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
-      case 2: hipLaunchKernelGGL((upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
-      case 4: hipLaunchKernelGGL((upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
-      default: hipLaunchKernelGGL((upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS, WAVES>), grid, block, 0, s, v, a); break;
+      case 1: launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
+      case 2: launch_main(upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
+      case 4: launch_main(upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
+      default: launch_main(upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
     }
   } else if constexpr (!BOUNDS) {
     if (vec == 4)
-      hipLaunchKernelGGL((upsert_kernel<OP, 4, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
+      launch_main(upsert_kernel<OP, 4, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
     else
-      hipLaunchKernelGGL((upsert_kernel<OP, 1, 8, LOCKED_RULE, false, WAVES>), grid, block, 0, s, v, a);
+      launch_main(upsert_kernel<OP, 1, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
   }
 }
 
@@ -1078,11 +1095,11 @@ template <int MODE>
 void launch_lookup(int vec, const View& v, const FindArgs& a, hipStream_t s) {
   const dim3 grid(grid_for(a.n)), block(kWave);
   if (vec == 16)
-    hipLaunchKernelGGL((lookup_kernel<MODE, 16>), grid, block, 0, s, v, a);
+    launch_main(lookup_kernel<MODE, 16>, grid, block, s, v, a);
   else if (vec == 4)
-    hipLaunchKernelGGL((lookup_kernel<MODE, 4>), grid, block, 0, s, v, a);
+    launch_main(lookup_kernel<MODE, 4>, grid, block, s, v, a);
   else
-    hipLaunchKernelGGL((lookup_kernel<MODE, 1>), grid, block, 0, s, v, a);
+    launch_main(lookup_kernel<MODE, 1>, grid, block, s, v, a);
 }
 
 /* the missed-keys find: 16 wavefronts per workgroup (see lookup_kernel) */
@@ -2045,6 +2062,14 @@ int hkv_set_clock(hkv_table* t, int mode, uint64_t base) {
   t->clock.mode = (uint32_t)mode;
   t->clock.base = base;
   t->bounds_stale = true; /* the new clock may be behind the old one */
+  return HKV_SUCCESS;
+}
+
+int hkv_time_next_kernel(void* start_event, void* stop_event) {
+  if ((start_event == nullptr) != (stop_event == nullptr))
+    return fail(HKV_ERROR_ARGUMENT, "hkv_time_next_kernel takes two events or none");
+  g_time_start = (hipEvent_t)start_event;
+  g_time_stop = (hipEvent_t)stop_event;
   return HKV_SUCCESS;
 }
 

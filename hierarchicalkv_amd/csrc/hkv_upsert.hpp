@@ -674,49 +674,16 @@ upsert_kernel(View v, UpsertArgs a) {
     uint32_t pos = 0;
     uint64_t victim = 0;
 
-    /* ---- step 1: hits and free slots, one CAS per key ------------------------------------ */
-    bool want_scan = false;
-    if (active) {
-      if (hit >= 0) {
-        uint64_t seen = key;
-        if (cas_lock(v.keys + hit, seen, v.locked_key)) {
-          got = kStDuplicate;
-          pos = (uint32_t)(hit - (int64_t)bslot);
-          victim = key;
-        } else {
-          /* The slot belongs to another key now (ours was evicted in this batch, or the probe
-           * was looking at somebody else's lock), or it is LOCKED: by a key of this batch that is
-           * taking it over or about to give it back, or for good (lock_keys, a batch-mate of
-           * the pointer overload that keeps its slots).  The second probe finds out which,
-           * and its waiting is bounded. */
-          hit = -1;
-          reprobe = true;
-        }
-      } else if (em_lo | em_hi) {
-        /* up to three free slots, the first at or after the key's start position
-         * so that keys of one bucket spread over the free slots */
-#pragma unroll 1
-        for (int attempt = 0; attempt < 3 && got == kStNone && (em_lo | em_hi); attempt++) {
-          const uint32_t p = first_from(em_lo, em_hi, start);
-          if (p < 64)
-            em_lo &= ~(UINT64_C(1) << p);
-          else
-            em_hi &= ~(UINT64_C(1) << (p - 64));
-          uint64_t seen = v.empty_key;
-          if (cas_lock(v.keys + bslot + p, seen, v.locked_key)) {
-            got = kStEmpty;
-            pos = p;
-            victim = v.empty_key;
-          }
-        }
-      } else {
-        want_scan = true;
-      }
-    }
+    /* what the key needs, known from the probe: its own slot, a free one, or a victim's */
+    const bool has_hit = active && hit >= 0;
+    const bool has_free = active && hit < 0 && (em_lo | em_hi) != 0;
+    const bool want_scan = active && hit < 0 && (em_lo | em_hi) == 0;
 
-    /* ---- step 2: full buckets: min-score scan by the tile, one bucket after the other ------------
-     * (two buckets in flight per tile took 32 more registers and with them a wavefront per
-     * SIMD: 0.308 against 0.323 ms per 2^20 keys) */
+    /* ---- step 1: full buckets: min-score search by the tile, before any lock is taken ------------
+     * (the search holds nothing, so the keys that were found wait for nobody while it runs, and
+     * the locks of all 64 keys are then taken in one round trip; two buckets in flight per tile
+     * in the full scan took 32 more registers and with them a wavefront per SIMD: 0.308 against
+     * 0.323 ms per 2^20 keys) */
     uint64_t best = kMaxScore;
     uint32_t bpos = 0;
     uint64_t new_bound = 0;
@@ -781,32 +748,90 @@ upsert_kernel(View v, UpsertArgs a) {
       }
     }
 
-    /* ---- step 3: refuse, or lock the victim ---------------------------------------------------- */
+    /* ---- step 2: one lock attempt per key, all in flight together ----------------------------------
+     * a compare-and-swap for a key that was found (key -> LOCKED) or that takes a free slot
+     * (EMPTY -> LOCKED: the first free slot at or after the key's start position, so that keys
+     * of one bucket spread over the free slots); an exchange for a victim: whatever key the slot
+     * held is the victim and the slot is locked (instead of a load and a compare-and-swap).
+     * LOCKED coming back means somebody else holds the slot (nothing changed); EMPTY is put
+     * back at once. */
     bool refused_now = false;
+    bool try_victim = false;
     if (want_scan) {
-      const bool refuse = (a.refuse_equal ? (desired <= best) : (desired < best));
-      if (refuse) {
+      if (a.refuse_equal ? (desired <= best) : (desired < best)) {
         refused_now = true;
         got = kStRefused;
       } else {
-        uint64_t* kp = v.keys + bslot + bpos;
-        /* one exchange instead of a load and a CAS: whatever key the slot held is the
-         * victim and the slot is locked.  LOCKED coming back means somebody else holds
-         * the slot (nothing changed); EMPTY is put back at once. */
-        const uint64_t vk = swap_lock(kp, v.locked_key);
-        const bool mine = vk != v.locked_key && vk != v.empty_key;
-        if (vk == v.empty_key) st_unlock(kp, vk);
-        if (mine) {
-          /* somebody may have raised the score since the scan */
-          if (ld_u64(v.scores + bslot + bpos) <= best) {
-            victim = vk;
-            got = (vk == v.reclaim_key) ? kStReclaimed : kStEvict;
-            pos = bpos;
-          } else {
-            st_unlock(kp, vk); /* nothing was written under this lock */
-          }
-        } /* else: the victim is locked or was taken by somebody else; next trip */
+        try_victim = true;
       }
+    }
+    uint32_t p_free = 0;
+    if (has_free) {
+      p_free = first_from(em_lo, em_hi, start);
+      if (p_free < 64)
+        em_lo &= ~(UINT64_C(1) << p_free);
+      else
+        em_hi &= ~(UINT64_C(1) << (p_free - 64));
+    }
+    uint64_t seen = has_hit ? key : v.empty_key;
+    bool cas_ok = false;
+    if (has_hit || has_free)
+      cas_ok = cas_lock(has_hit ? v.keys + hit : v.keys + bslot + p_free, seen, v.locked_key);
+    uint64_t* const kp = v.keys + bslot + bpos;
+    uint64_t vk = v.locked_key;
+    if (try_victim) vk = swap_lock(kp, v.locked_key);
+
+    /* ---- step 3: what came back ------------------------------------------------------------------------ */
+    if (has_hit) {
+      if (cas_ok) {
+        got = kStDuplicate;
+        pos = (uint32_t)(hit - (int64_t)bslot);
+        victim = key;
+      } else {
+        /* The slot belongs to another key now (ours was evicted in this batch, or the probe
+         * was looking at somebody else's lock), or it is LOCKED: by a key of this batch that is
+         * taking it over or about to give it back, or for good (lock_keys, a batch-mate of
+         * the pointer overload that keeps its slots).  The second probe finds out which,
+         * and its waiting is bounded. */
+        hit = -1;
+        reprobe = true;
+      }
+    }
+    if (has_free) {
+      if (cas_ok) {
+        got = kStEmpty;
+        pos = p_free;
+        victim = v.empty_key;
+      }
+      /* somebody else took it: up to two more of the bucket's free slots */
+#pragma unroll 1
+      for (int attempt = 1; attempt < 3 && got == kStNone && (em_lo | em_hi); attempt++) {
+        const uint32_t p = first_from(em_lo, em_hi, start);
+        if (p < 64)
+          em_lo &= ~(UINT64_C(1) << p);
+        else
+          em_hi &= ~(UINT64_C(1) << (p - 64));
+        uint64_t e = v.empty_key;
+        if (cas_lock(v.keys + bslot + p, e, v.locked_key)) {
+          got = kStEmpty;
+          pos = p;
+          victim = v.empty_key;
+        }
+      }
+    }
+    if (try_victim) {
+      const bool mine = vk != v.locked_key && vk != v.empty_key;
+      if (vk == v.empty_key) st_unlock(kp, vk);
+      if (mine) {
+        /* somebody may have raised the score since the search */
+        if (ld_u64(v.scores + bslot + bpos) <= best) {
+          victim = vk;
+          got = (vk == v.reclaim_key) ? kStReclaimed : kStEvict;
+          pos = bpos;
+        } else {
+          st_unlock(kp, vk); /* nothing was written under this lock */
+        }
+      } /* else: the victim is locked or was taken by somebody else; next trip */
     }
 
     /* ---- step 4: critical sections of every lock taken in this trip ------------------------------ */
@@ -911,7 +936,6 @@ upsert_kernel(View v, UpsertArgs a) {
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
     if constexpr (WAVES == 1) more = pend_mask != 0;
-    if (pend_mask) __builtin_amdgcn_s_sleep(1);
   }
 }
 

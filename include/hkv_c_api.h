@@ -124,8 +124,8 @@ typedef struct hkv_table_view {
   uint8_t pow2_buckets; /* buckets_num is a power of two */
   uint8_t dual_bucket;  /* TableMode::kMemory: a key lives in one of two buckets */
   uint8_t pad_[4];
-  uint64_t* bounds;     /* LRU tables, else NULL.  [buckets_num][8]: for each run of 16 slots a
-                           value that is not above any score in it (0 is always right); kept
+  uint64_t* bounds;     /* NULL for dual-bucket tables.  [buckets_num][8]: for each run of 16
+                           slots a value that is not above any score in it (0 is always right); kept
                            tight by the upserts, which with it read one or two of a bucket's
                            eight score lines instead of all of them.  Whoever lowers a score
                            in place sets the bound of its run to 0 or calls
@@ -353,6 +353,14 @@ int hkv_set_clock(hkv_table* t, int mode, uint64_t base);
  * the scores (hkv_table_view::bounds) before it relies on it again.  No counterpart in the
  * reference, which keeps no such knowledge. */
 int hkv_scores_changed(hkv_table* t);
+
+/* Measurement aid, no counterpart in the reference (its benchmark times whole calls on the host,
+ * benchmark/merlin_hashtable_benchmark.cc.cu:166-265): the next find or upsert-family call made
+ * by the calling thread launches its kernel with these two HIP events (hipEvent_t, created by the
+ * caller), which the runtime stamps with the start and the end of that kernel's execution;
+ * hipEventElapsedTime(start, stop) is then the kernel's own duration, as a profiler reports it.
+ * Two null pointers cancel a pending request. */
+int hkv_time_next_kernel(void* start_event, void* stop_event);
 
 #ifdef __cplusplus
 }
