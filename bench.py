@@ -145,6 +145,9 @@ def main():
                          "3: Zipf insert_and_evict + find at 2^27, dim 64; 4: hybrid HBM + pinned host rows at "
                          "2^28 with HBM and host-link GB/s apart; 5: accum_or_assign / export_batch_if / erase "
                          "at 2^25, dim 128); a markdown table and one JSON line")
+    ap.add_argument("--load-factor", type=float, default=0.0,
+                    help="with --config 2: only this load factor (0.5, 0.75 or 1.0) instead of all three in turn, so "
+                         "that a profiler's last dispatches of each kernel are the timed calls at that load factor")
     ap.add_argument("--group-lock", action="store_true",
                     help="instead of the one-line benchmark: what the API-level group lock costs the host per call, "
                          "as built (stream events, never blocks) against a host-blocking acquisition as the "
@@ -723,6 +726,106 @@ OPS_KERNELS = [
 ]
 
 
+# bench.py --config N under rocprofv3: (run tag, command, title, [(kernel needle, call, which dispatches)]).
+# "last3": the timed calls are the kernel's last three dispatches; "mid3": the middle one of each
+# of its last three triples (configuration 4 looks up row addresses before and after its timed
+# find*); "sum8": one call is eight dispatches, added up.
+CONFIG_PROFILES = [
+    ("cfg2_lf050", "python3 bench.py --config 2 --load-factor 0.5", "configuration 2 (capacity 2^26, dim 8, LRU) at load factor 0.50",
+     [("lookup_kernel<0, 16", "find (100 % hit)", "last3"), ("upsert_kernel<0, 16, 1, false", "insert_or_assign (50 % new)", "last3"),
+      ("upsert_kernel<2, 16, 1, false", "find_or_insert (50 % new)", "last3")]),
+    ("cfg2_lf075", "python3 bench.py --config 2 --load-factor 0.75", "configuration 2 at load factor 0.75",
+     [("lookup_kernel<0, 16", "find (100 % hit)", "last3"), ("upsert_kernel<0, 16, 1, false", "insert_or_assign (50 % new)", "last3"),
+      ("upsert_kernel<2, 16, 1, false", "find_or_insert (50 % new)", "last3")]),
+    ("cfg2_lf100", "python3 bench.py --config 2 --load-factor 1.0", "configuration 2 at load factor 1.00",
+     [("lookup_kernel<0, 16", "find (100 % hit)", "last3"), ("upsert_kernel<0, 16, 1, false", "insert_or_assign (50 % new)", "last3"),
+      ("upsert_kernel<2, 16, 1, false", "find_or_insert (50 % new)", "last3")]),
+    ("cfg3", "python3 bench.py --config 3", "configuration 3 (capacity 2^27, dim 64, Customized, Zipf keys, load factor 1.0)",
+     [("upsert_kernel<1, 16, 2, false", "insert_and_evict", "last3"), ("lookup_kernel<0, 16", "find on the same keys", "last3")]),
+    ("cfg4", "python3 bench.py --config 4", "configuration 4 (capacity 2^28, dim 64, 16 GiB of rows in HBM + 48 GiB pinned, LFU)",
+     [("lookup_kernel<0, 16", "find (about 80 % hit)", "last3"), ("lookup_kernel<1, 16", "find*", "mid3"),
+      ("upsert_kernel<0, 16, 2, false", "insert_or_assign (about 20 % new)", "last3")]),
+    ("cfg5", "python3 bench.py --config 5", "configuration 5 (capacity 2^25, dim 128, EpochLRU, load factor 1.0)",
+     [("upsert_kernel<3, 16, 4, false", "accum_or_assign (70 % existing)", "last3"),
+      ("export_if_kernel", "export_batch_if over the whole table (8 windows)", "sum8"),
+      ("erase_kernel<true>", "erase (2^18 keys)", "last3")]),
+]
+CONFIG_GROUPS = ["trace", "fetch", "write", "wr", "tcp"]
+
+
+def summarize_configs(root, pick, counters, durations):
+    """profiles/config<N>_*.md and .json from rocprofv3 runs of bench.py --config N (see CONFIG_PROFILES)."""
+    groups = dict(PROFILE_GROUPS)
+    for tag, cmd, title, kernels in CONFIG_PROFILES:
+        dur = durations(tag)
+        if not dur:
+            continue
+        cnt = {g: counters(tag, g)[0] for g in CONFIG_GROUPS if g != "trace"}
+
+        def take(values, how):
+            if how == "mid3":
+                v = [values[i] for i in (-2, -5, -8) if len(values) >= -i]
+            elif how == "sum8":
+                return sum(values[-8:])
+            else:
+                v = values[-3:]
+            return sum(v) / len(v) if v else float("nan")
+
+        def cval(g, needle, name, how):
+            k = pick(cnt[g], needle)
+            return take(cnt[g][k][name], how) if k and name in cnt[g][k] else float("nan")
+
+        o = ["# rocprofv3: %s\n" % title,
+             "One MI355X.  Commands, from the repository root after `cd /tmp && export TMPDIR=/tmp && cd -`, one run each "
+             "(the output of the first is kept beside this file as %s.json):\n" % ("config" + tag[3:])]
+        for g in CONFIG_GROUPS:
+            o.append("    rocprofv3 %s --output-format csv -d gpurun_out/prof/%s_%s -o out -- %s" % (groups[g], tag, g, cmd))
+        o.append("    python3 bench.py --profile-summary gpurun_out/prof\n")
+        o.append("Per call: the average over the kernel's timed dispatches (the last three of the run; find* of "
+                 "configuration 4: the middle one of each of the last three triples; export_batch_if: eight windows "
+                 "added up).  FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0 (what they read for a plain 1 GiB "
+                 "device copy, profiles/lookup_kernel_upsert_kernel_cap2p26_dim64_batch2p20.md).  Durations are those of "
+                 "the trace run; a counter run serialises and slows the kernels.  Rows that a kernel reads or writes in "
+                 "pinned host memory do not pass the HBM counters.\n")
+        o.append("| call | kernel | us (trace) | FETCH MB | WRITE MB | traffic GB/s | writes to memory (M) | of them partial, "
+                 "below 64 B (M) | atomics to memory (M) | L1 -> L2 read / write requests (M) | returning atomics (M) | "
+                 "L1 TLB misses (M) |\n|---|---|---|---|---|---|---|---|---|---|---|---|")
+        for needle, call, how in kernels:
+            k = pick(dur, needle)
+            if not k:
+                continue
+            us = take(dur[k], how)
+            fmb = cval("fetch", needle, "FETCH_SIZE", how) * 2.0 * 1024 / 1e6
+            wmb = cval("write", needle, "WRITE_SIZE", how) * 1024 / 1e6
+            wreq = cval("wr", needle, "TCC_EA0_WRREQ_sum", how)
+            w64 = cval("wr", needle, "TCC_EA0_WRREQ_64B_sum", how)
+            short = k.split("(")[0].replace("void ", "").replace("hkv::", "")
+            o.append("| %s | `%s` | %.1f | %.1f | %.1f | %.0f | %.2f | %.2f | %.2f | %.2f / %.2f | %.2f | %.2f |" % (
+                call, short, us, fmb, wmb, (fmb + wmb) / us * 1e3, wreq / 1e6, (wreq - w64) / 1e6,
+                cval("write", needle, "TCC_EA0_ATOMIC_sum", how) / 1e6,
+                cval("tcp", needle, "TCP_TCC_READ_REQ_sum", how) / 1e6, cval("tcp", needle, "TCP_TCC_WRITE_REQ_sum", how) / 1e6,
+                cval("tcp", needle, "TCP_TCC_ATOMIC_WITH_RET_REQ_sum", how) / 1e6,
+                cval("tcp", needle, "TCP_UTCL1_TRANSLATION_MISS_sum", how) / 1e6))
+        # the benchmark's own table and JSON line of the trace run
+        log = os.path.join(root, "%s_trace.log" % tag)
+        line = None
+        if os.path.exists(log):
+            o.append("\n## What `%s` printed in the trace run (HIP-event times per call, algorithmic bytes)\n" % cmd)
+            for ln in open(log):
+                if ln.startswith("|"):
+                    o.append(ln.rstrip())
+                if ln.startswith("{") and '"config"' in ln:
+                    line = ln.strip()
+        name = "config" + tag[3:]
+        path = os.path.join(ROOT, "profiles", name + ".md")
+        with open(path, "w") as f:
+            f.write("\n".join(o) + "\n")
+        print("wrote", path)
+        if line:
+            with open(os.path.join(ROOT, "profiles", name + ".json"), "w") as f:
+                f.write(line + "\n")
+
+
 def summarize_profiles(root):
     """rocprofv3 CSVs -> profiles/*.md + the traffic file.  Per kernel: the average over its last
     dispatches (the timed calls: the launches of the table fill come first), durations from the
@@ -897,6 +1000,7 @@ def summarize_profiles(root):
         with open(path, "w") as f:
             f.write("\n".join(o) + "\n")
         print("wrote", path)
+    summarize_configs(root, pick, counters, durations)
     dur = durations("ceil")
     lat_by, _ = counters("ceil", "lat")
     if dur and lat_by:
@@ -999,7 +1103,7 @@ def run_config(args, torch):
         out = torch.empty(n, dim, dtype=torch.float32, device=dev)
         vals = torch.empty(n, dim, dtype=torch.float32, device=dev).uniform_(-1.0, 1.0)
         pos, fresh, old = 0, 1 << 36, 0
-        for lf in (0.50, 0.75, 1.00):
+        for lf in ((args.load_factor,) if args.load_factor else (0.50, 0.75, 1.00)):
             while pos < int(lf * cap) or (lf == 1.0 and t.size() < 0.999 * cap and pos < 3 * cap):
                 t.insert_or_assign(n, wd.dev_keys(seed, pos, n), vals)
                 pos += n
@@ -1280,6 +1384,14 @@ CEILING_PATTERNS = [
     ("small_cas64", "64-bit compare-and-swap, one per random line", "G ops/s"),
     ("small_xchg64", "64-bit exchange, one per random line", "G ops/s"),
     ("small_xchg32_side", "32-bit exchange on a 4-byte-per-bucket array (fits the Infinity Cache)", "G ops/s"),
+    # (new patterns go to the end: --profile-summary finds the launches of the ones above by their order)
+    ("upsert_pattern_free", "insert_or_assign's accesses on a table with free slots, chained: 50 % absent keys that "
+                            "take a free slot with a compare-and-swap and add one to the bucket's counter, no score "
+                            "reads (algorithmic bytes)", "GB/s"),
+    ("findptr_pattern", "find* / contains: batch key -> digest line -> key word (1.1 lines per key) -> 8-byte result "
+                        "and flag (algorithmic bytes: 153 per key)", "GB/s"),
+    ("erase_pattern", "erase with the table to itself: batch key -> digest line -> key word -> key store, digest "
+                      "store, one atomic on the bucket's counter (algorithmic bytes: 165 per key)", "GB/s"),
 ]
 
 

@@ -182,7 +182,10 @@ k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
  *                          written, 8-byte key and score stores and a 1-byte digest store.
  * `locks` adds what the slot-lock protocol spends: a compare-and-swap and an unlock store per
  * present key, an exchange and a score re-read per absent key (the key store of an absent
- * key doubles as its unlock). */
+ * key doubles as its unlock).
+ * locks == 3: a table with free slots.  An absent key reads no scores: it takes a free slot with
+ * a compare-and-swap and adds one to the bucket's counter (a 32-bit atomic on the 4-byte-per-bucket
+ * array); a quarter of the absent keys fetch a key line for a false digest match. */
 template <bool CHAIN>
 __global__ void __launch_bounds__(64)
 k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int locks) {
@@ -207,10 +210,11 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
   const uint32_t p = (uint32_t)(h >> 40) & 127u;
   uint64_t slot = bk * 128 + p;
   const bool absent = lane & 1;
-  acc += b.keys[slot];
+  const bool free_mode = locks == 3;
+  if (!(free_mode && absent) || (uint32_t)((h >> 52) % 1000) < 250u) acc += b.keys[slot];
   if ((uint32_t)((h >> 48) % 1000) < extra_pm) acc += b.keys[bk * 128 + ((p + 64) & 127u)];
   if (locks) {
-    if (!absent) {
+    if (!absent || free_mode) {
       uint64_t expect = acc;
       __hip_atomic_compare_exchange_strong(b.keys + slot, &expect, acc, __ATOMIC_RELAXED,
                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -220,7 +224,9 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
   if (CHAIN) salt += zero_after((uint32_t)acc);
   /* score scans of the absent keys: keys 8t+1, 8t+3, 8t+5, 8t+7 of each tile, two in flight;
    * with score bounds (locks == 2): the bucket's 8 bounds (64 bytes), then one score line */
-  if (locks == 2) {
+  if (free_mode) {
+    /* no victim search */
+  } else if (locks == 2) {
     uint64_t bd[4];
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -256,7 +262,7 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
       for (int it = 0; it < 8; it++) acc += sc[w][it].x ^ sc[w][it].z;
   }
   if (CHAIN) slot += zero_after((uint32_t)acc);
-  if (locks && absent) {
+  if (locks && absent && !free_mode) {
     acc += __hip_atomic_exchange(b.keys + slot, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (CHAIN) slot += zero_after((uint32_t)acc);
     acc += __hip_atomic_load(b.scores + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -273,6 +279,7 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
     st1_wt(b.digests + slot, (uint8_t)acc);
     st8_wt(b.keys + slot, acc);
     if (locks == 2) st8_wt(reinterpret_cast<uint64_t*>(b.digests) + (slot >> 4), acc);
+    if (free_mode) atomicAdd(b.small + bk, 1u);
   }
   /* rows: dense input -> table rows, 64 rows x units over the 64 lanes */
   const uint32_t upr = sh.row_bytes / 16;
@@ -300,6 +307,44 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
   if (locks && !absent) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     st8_wt(b.keys + slot, acc);
+  }
+}
+
+/* ---- the access pattern of the calls that move no rows -------------------------------------------------
+ * Probe as find's (batch key, digest line, one key word, a second one for `extra_pm` keys in 1000);
+ * kind 0 (find* / contains): one 8-byte result and one flag per key;
+ * kind 1 (erase with the table to itself): an 8-byte key store and a 1-byte digest store into the
+ *        table, and one 32-bit atomic on the bucket's counter per key. */
+__global__ void __launch_bounds__(64)
+k_norow_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int kind) {
+  const int lane = threadIdx.x, tile = lane >> 3, j = lane & 7;
+  const uint64_t base = (uint64_t)blockIdx.x * 64;
+  uint64_t acc = b.in_keys[base + lane];
+  salt += zero_after((uint32_t)acc);
+  uint4 dg[8];
+#pragma unroll
+  for (int r = 0; r < 8; r++) {
+    const uint64_t bk = mix(base + tile * 8 + r + salt) & (sh.buckets - 1);
+    dg[r] = *reinterpret_cast<const uint4*>(b.digests + bk * 128 + j * 16);
+  }
+#pragma unroll
+  for (int r = 0; r < 8; r++) acc += dg[r].x ^ dg[r].w;
+  salt += zero_after((uint32_t)acc);
+  const uint64_t h = mix(base + lane + salt);
+  const uint64_t bk = h & (sh.buckets - 1);
+  const uint32_t p = (uint32_t)(h >> 40) & 127u;
+  uint64_t slot = bk * 128 + p;
+  acc += b.keys[slot];
+  if ((uint32_t)((h >> 48) % 1000) < extra_pm) acc += b.keys[bk * 128 + ((p + 64) & 127u)];
+  slot += zero_after((uint32_t)acc);
+  if (acc == 0x123456789ULL) *b.sink = 1;
+  if (kind == 0) {
+    reinterpret_cast<uint64_t*>(b.out_rows)[base + lane] = acc;
+    b.flags[base + lane] = 1;
+  } else {
+    b.keys[slot] = acc;
+    b.digests[slot] = (uint8_t)acc;
+    atomicAdd(b.small + bk, 1u);
   }
 }
 
@@ -503,6 +548,15 @@ int hkv_ceilings_run(const char* name, int reps, double* ms, double* bytes) {
     } else if (!strcmp(name, "upsert_pattern_chained")) {
       hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 1);
       moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));
+    } else if (!strcmp(name, "upsert_pattern_free")) {
+      hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 50u, 3);
+      moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (169 + 2.0 * sh.row_bytes));
+    } else if (!strcmp(name, "findptr_pattern")) {
+      hipLaunchKernelGGL(k_norow_pattern, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 0);
+      moved = (double)n * 153;
+    } else if (!strcmp(name, "erase_pattern")) {
+      hipLaunchKernelGGL(k_norow_pattern, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 1);
+      moved = (double)n * 165;
     } else if (!strcmp(name, "upsert_pattern_bounds")) {
       hipLaunchKernelGGL(k_upsert_pattern<true>, dim3((unsigned)(n / 64)), dim3(64), 0, 0, sh, b, salt, 100u, 2);
       moved = (double)n * (0.5 * (161 + 2.0 * sh.row_bytes) + 0.5 * (1185 + 2.0 * sh.row_bytes));

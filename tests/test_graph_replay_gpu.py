@@ -220,3 +220,85 @@ def _run_writers(oracle, stream):
         torch.cuda.synchronize()
     t.close()
     ot.close()
+
+
+def test_replays_after_scores_from_outside_the_clock():
+    """An LRU table on the hardware clock whose upserts search victims through the score bounds: an
+    insert_or_assign recorded into a graph must go on evicting the lowest score of a bucket after
+    a call that writes scores from outside the clock (ignore_evict_strategy) has made the bounds
+    stale, replay after replay, with eager upserts (which make the bounds again) in between.
+    Without an oracle (the scores are the time of day): the keys that were given the lowest scores
+    are the first to go, every row that is found is its key's, and the bounds hold at the end."""
+    from test_score_bounds_gpu import bounds_hold
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        cap, dim, n = 1 << 14, 16, 2048
+        o = default_options(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=1 << 30, dim=dim,
+                            evict_strategy=EvictStrategy.kLru)
+        t = HashTable()
+        t.init(o)
+        pos = 0
+        for _ in range(12):  # past load factor 1.0: the last calls use the bounds
+            k = w.unique_keys(55, pos, n)
+            t.insert_or_assign(n, dev(k), dev(w.values_from_keys(k, dim)))
+            pos += n
+        torch.cuda.synchronize()
+        assert bounds_hold(t)[0] and bounds_hold(t)[2] > 0
+        ik = torch.zeros(n, dtype=torch.int64, device=DEV)
+        iv = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+
+        def load(start):
+            k = w.unique_keys(55, start, n)
+            ik.copy_(dev(k))
+            iv.copy_(dev(w.values_from_keys(k, dim)))
+            return k
+        load(pos)
+        pos += n
+        t.insert_or_assign(n, ik, iv)  # warm-up of the exact call
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        load(pos)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=stream):
+            t.insert_or_assign(n, ik, iv)
+        founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+        out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+        for rnd in range(3):
+            # residents get scores far below the clock's
+            low = w.unique_keys(55, pos - 2 * n, n)
+            t.contains(n, dev(low), founds)
+            torch.cuda.synchronize()
+            low = low[founds.cpu().numpy()]
+            assert len(low) > n // 2
+            t.insert_or_assign(len(low), dev(low), dev(w.values_from_keys(low, dim)),
+                               dev(np.arange(1, len(low) + 1, dtype=np.uint64)), ignore_evict_strategy=True)
+            # three replays and an eager upsert: 64 new keys for each of the 128 buckets on average,
+            # at least about 40 for every one, against at most about 30 low-scored keys in a bucket:
+            # they all go if every eviction takes the bucket's lowest score, and most of them stay
+            # if victims are taken from elsewhere
+            for r in range(3):
+                load(pos)
+                pos += n
+                g.replay()
+                if r == 1:  # an eager upsert between replays rebuilds the bounds and uses them
+                    k = w.unique_keys(56, pos, n)
+                    t.insert_or_assign(n, dev(k), dev(w.values_from_keys(k, dim)))
+            torch.cuda.synchronize()
+            f2 = torch.zeros(len(low), dtype=torch.bool, device=DEV)
+            t.contains(len(low), dev(low), f2)
+            torch.cuda.synchronize()
+            assert not f2.cpu().numpy().any(), "keys with the lowest scores outlived 64 new keys per bucket"
+            assert t.size() == cap
+            last = w.unique_keys(55, pos - n, n)
+            t.find(n, dev(last), out, founds)
+            torch.cuda.synchronize()
+            f = founds.cpu().numpy()
+            assert f.all()
+            assert np.array_equal(out.cpu().numpy(), w.values_from_keys(last, dim))
+        k = w.unique_keys(57, 0, n)
+        t.insert_or_assign(n, dev(k), dev(w.values_from_keys(k, dim)))
+        torch.cuda.synchronize()
+        ok, bad, _ = bounds_hold(t)
+        assert ok, bad
+        t.close()
+    torch.cuda.synchronize()
