@@ -45,7 +45,7 @@ def upsert_bytes(vb, new_fraction):
 # counter reads for a 1 GiB device-to-device copy in the same run).  Counters cannot be read
 # from inside this process, so `--profile-summary` writes them to a file beside the profile
 # summaries and the default run reports what that file holds; it applies to the default
-# workload and the default (slot-lock) upsert path only.
+# workload only.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic_cap2p26_dim64_batch2p20.json")
 
 
@@ -341,8 +341,7 @@ def main():
 
     default_workload = (args.capacity_log2 == 26 and dim == 64 and args.batch_log2 == 20
                         and not args.warm_keys and args.strategy == "lru")
-    path = os.environ.get("HKV_UPSERT_PATH", "locked")
-    ups_traffic = measured_traffic("upsert_kernel") if default_workload and path == "locked" else None
+    ups_traffic = measured_traffic("upsert_kernel") if default_workload else None
     find_traffic = measured_traffic("lookup_kernel") if default_workload else None
     timed_by = ("events on the stream around each call" if (not args.kernel_events) else
                 "the event pair each kernel is launched with (start and end of its execution)")
@@ -373,7 +372,6 @@ def main():
             "size_after": size1,
             "prefill_s": round(prefill_s, 1),
             "resident_keys": "warm (previous step)" if args.warm_keys else "cold (old pre-fill batches)",
-            "upsert_path": path,
         },
         "find": {"ms": round(find_avg, 4), "bkvs": round(n / (find_avg * 1e-3) / 1e9, 4),
                  "bkvs_2p30": round(n / (find_avg * 1e-3) / 2**30, 4)},
@@ -384,8 +382,7 @@ def main():
         # The bounded victim search moves fewer bytes than the algorithmic figure bills (it reads
         # one or two of a bucket's eight score lines), find moves more (whole 128-byte lines for
         # 8-byte key verifications).
-        "roofline": {"kernel": "upsert_kernel<insert_or_assign>" if path == "locked" else
-                     "two-phase upsert: upsert_hits_kernel + chained_miss_kernel", "bound": "hbm",
+        "roofline": {"kernel": "upsert_kernel<insert_or_assign>", "bound": "hbm",
                      "achieved": round(ups_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ups_gbs / HBM_PEAK_GBS, 4), "traffic": ups_traffic,
                      "traffic_frac": traffic_frac(ups_traffic, ups_avg),

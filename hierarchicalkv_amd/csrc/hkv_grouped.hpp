@@ -1,15 +1,13 @@
 /*
- * Two-phase upserts: the large-batch path of insert_or_assign,
- * insert_and_evict, find_or_insert and accum_or_assign.
+ * Two-phase insert_or_assign: the path behind hkv_insert_or_assign_noalloc, the entry point for
+ * callers that cannot allocate.
  *
- * Same per-key semantics as the slot-lock kernel (hkv_upsert.hpp, after
- * upsert.cuh:52-233, upsert_and_evict.cuh:27-1099, find_or_insert.cuh:27-1050,
- * accum_or_assign.cuh:83-174); what changes is who may touch a slot.  An
- * inserter runs alone on the table (the API-level group lock, as
- * group_lock.cuh:43-56), so the only conflicts are between keys of the same
- * batch, and only between keys that are absent: a key that is present owns its
- * slot (keys of a batch are unique), absent keys of one bucket compete for its
- * free slots and victims.  Hence two phases, each one kernel:
+ * Same per-key semantics as the slot-lock kernel (hkv_upsert.hpp, after upsert.cuh:52-233);
+ * what changes is who may touch a slot.  An inserter runs alone on the table (the API-level
+ * group lock, as group_lock.cuh:43-56), so the only conflicts are between keys of the same
+ * batch, and only between keys that are absent: a key that is present owns its slot (keys of a
+ * batch are unique), absent keys of one bucket compete for its free slots and victims.  Hence
+ * two phases, each one kernel:
  *
  *   upsert_hits_kernel   every key is probed as in find.  A key that is present
  *                        gets its new score and row at once, without a lock.
@@ -28,11 +26,9 @@
  *
  * The serial order this amounts to - all present keys, then the absent ones
  * bucket by bucket - is one of the orders the slot-lock kernel could have
- * produced.  What is saved: the slot-lock protocol spends a compare-and-swap
- * and an unlock store per present key and an exchange and a score re-read per
- * absent key, each of them a small access that the memory side serves as a
- * read-modify-write of a 64-byte piece, and a bucket that takes several keys of
- * a batch is scanned once instead of once per key.
+ * produced.  The path has no locks and needs no memory beyond the list heads and links, which is
+ * why the no-alloc entry point runs on it; as the general path it measured slower than the
+ * slot-lock kernel (two launches, a second pass over the keys), so nothing else uses it.
  */
 #ifndef HKV_GROUPED_HPP_
 #define HKV_GROUPED_HPP_
@@ -104,10 +100,8 @@ struct ChainArgs {
  *            strategy needs it) and the row traffic of the operation, the whole
  *            wavefront moving the rows of its keys, VEC bytes per lane;
  *   absent   hung into the list of its bucket for the second phase.
- * accum_or_assign drops the keys whose flag disagrees with what was found
- * (accum_or_assign.cuh:139-156).
  */
-template <int OP, int VEC>
+template <int VEC>
 __global__ void __launch_bounds__(kWave)
 upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
   __shared__ KeyMeta s_meta[kWave];
@@ -123,13 +117,8 @@ upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
 
   const bool valid = (s_meta[lane].info & 0x100u) != 0;
   const int64_t slot = s_slot[lane];
-  bool hit = valid && slot >= 0;
-  bool miss = valid && slot < 0;
-  if (OP == kOpAccumOrAssign && valid) {
-    const bool is_accum = a.accum_flags[i] != 0;
-    if (hit && !is_accum) hit = false;
-    if (miss && is_accum) miss = false;
-  }
+  const bool hit = valid && slot >= 0;
+  const bool miss = valid && slot < 0;
   if (i < a.n) {
     uint32_t before = kChainEnd;
     if (miss)
@@ -144,13 +133,6 @@ upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
     uint64_t snew;
     if (final_score(a, false, desired, in_score, old, snew)) v.scores[slot] = snew;
   }
-  if (OP == kOpAccumOrAssign) {
-    /* rows move for the keys that stay "present" only */
-    __syncthreads();
-    if (!hit) s_slot[lane] = -1;
-    __syncthreads();
-  }
-
   /* rows: 64 rows x units-per-row spread over the 64 lanes; all loads of a
    * batch are issued before the first store */
   using T = typename VecType<VEC>::type;
@@ -158,30 +140,18 @@ upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
   const uint32_t total = units * kWave;
   const bool pow2 = (units & (units - 1)) == 0;
   const uint32_t sh = 31 - __clz(units);
-  constexpr int kBatch = VEC == 16 ? (OP == kOpAccumOrAssign ? 8 : 16) : 4;
-  uint8_t* usr_base = (OP == kOpFindOrInsert ? a.values_io : const_cast<uint8_t*>(a.values_in)) +
-                      base * v.value_bytes;
+  constexpr int kBatch = VEC == 16 ? 16 : 4;
+  const uint8_t* usr_base = a.values_in + base * v.value_bytes;
   for (uint32_t idx0 = lane; idx0 < total; idx0 += kWave * kBatch) {
     T buf[kBatch];
-    T tab[OP == kOpAccumOrAssign ? kBatch : 1];
 #pragma unroll
     for (int b = 0; b < kBatch; b++) {
       const uint32_t idx = idx0 + b * kWave;
       buf[b] = T{};
-      if (OP == kOpAccumOrAssign) tab[b] = T{};
       if (idx < total) {
         const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
         const uint32_t c = idx - kk * units;
-        const int64_t sl = s_slot[kk];
-        if (sl >= 0) {
-          if (OP == kOpFindOrInsert) {
-            buf[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
-          } else {
-            buf[b] = ld_unit<VEC, false>(usr_base + (uint64_t)kk * v.value_bytes, c);
-            if (OP == kOpAccumOrAssign)
-              tab[b] = reinterpret_cast<const T*>(value_row(v, (uint64_t)sl))[c];
-          }
-        }
+        if (s_slot[kk] >= 0) buf[b] = ld_unit<VEC, false>(usr_base + (uint64_t)kk * v.value_bytes, c);
       }
     }
 #pragma unroll
@@ -191,15 +161,7 @@ upsert_hits_kernel(View v, UpsertArgs a, ChainArgs h) {
         const uint32_t kk = pow2 ? (idx >> sh) : (idx / units);
         const uint32_t c = idx - kk * units;
         const int64_t sl = s_slot[kk];
-        if (sl >= 0) {
-          if (OP == kOpFindOrInsert) {
-            st_unit<VEC, false>(usr_base + (uint64_t)kk * v.value_bytes, c, buf[b]);
-          } else if (OP == kOpAccumOrAssign) {
-            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, add_unit(tab[b], buf[b], a.value_kind));
-          } else {
-            st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
-          }
-        }
+        if (sl >= 0) st_unit<VEC, true>(value_row(v, (uint64_t)sl), c, buf[b]);
       }
     }
   }
@@ -304,7 +266,7 @@ __device__ __forceinline__ Top2 tile_top2(const View& v, uint64_t bslot, int j, 
  * computed by all 8 lanes alike from the same LDS entries, so the lanes agree
  * without talking; only the minimum search and the free-slot mask cross lanes.
  */
-template <int OP, int VEC, int UPL>
+template <int VEC, int UPL>
 __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
                                              const ChainArgs& g, uint32_t bkt, uint32_t sb,
                                              uint32_t se, const uint64_t* s_key,
@@ -315,7 +277,7 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
   const int tile = lane >> 3;
   const int tile_base = lane & ~(kTile - 1);
   const uint64_t bslot = (uint64_t)bkt * kBucketSize;
-  const uint8_t* rows_in = OP == kOpFindOrInsert ? a.values_io : a.values_in;
+  const uint8_t* rows_in = a.values_in;
 
   bool dg_dirty = false;
   int size_delta = 0;
@@ -362,7 +324,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
     int got[kGrpKeys];
     uint32_t pos[kGrpKeys];
     uint64_t snew[kGrpKeys];
-    uint64_t best_seen[kGrpKeys];
     bool wrs[kGrpKeys], cancelled[kGrpKeys], need_vk[kGrpKeys];
     int vic_from[kGrpKeys];
     bool scanned = false;
@@ -374,7 +335,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       got[q] = kStNone;
       pos[q] = 0;
       snew[q] = 0;
-      best_seen[q] = 0;
       wrs[q] = false;
       cancelled[q] = false;
       need_vk[q] = false;
@@ -470,9 +430,8 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       const bool tomb_digest =
           tile_ballot(j == (int)(bpos >> 4) && dg_byte(dg, bpos & 15u) == v.reclaim_digest, tile) != 0;
       got[q] = kStEvict;
-      need_vk[q] = vic_from[q] < 0 && (OP == kOpInsertAndEvict || tomb_digest);
+      need_vk[q] = vic_from[q] < 0 && tomb_digest;
       pos[q] = bpos;
-      best_seen[q] = best;
       if (j == (int)(bpos >> 4)) dg_set(dg, bpos & 15u, info & 0xFFu);
       dg_dirty = true;
     }
@@ -489,82 +448,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
       if (got[q] == kStEvict && need_vk[q] && victim[q] == v.reclaim_key) {
         got[q] = kStReclaimed;
         size_delta++;
-      }
-#pragma unroll
-      for (int p = 0; p < q; p++)
-        if (vic_from[q] == p) victim[q] = s_key[q0 + p];
-    }
-
-    /* ---- what leaves the table (upsert_and_evict.cuh:188-194, 218-224, 236-245) ------------------------ */
-    if (OP == kOpInsertAndEvict) {
-      int emits = 0;
-#pragma unroll
-      for (int q = 0; q < kGrpKeys; q++) emits += (got[q] == kStRefused || got[q] == kStEvict);
-      /* one counter update per wavefront and pass: the tiles that have something
-       * to emit right now add up their counts (an atomic per bucket on this one
-       * word would serialise the whole launch) */
-      const unsigned long long leaders = __ballot(j == 0 && emits > 0);
-      unsigned long long idx = 0;
-      if (leaders) {
-        int before = 0, total = 0;
-        for (unsigned long long m = leaders; m; m &= m - 1) {
-          const int l = (int)__ffsll(m) - 1;
-          const int e = __shfl(emits, l);
-          total += e;
-          if (l < tile_base) before += e;
-        }
-        const int first_leader = (int)__ffsll(leaders) - 1;
-        unsigned long long base = 0;
-        if (lane == first_leader) base = atomicAdd(a.evicted_counter, (unsigned long long)total);
-        base = __shfl(base, first_leader);
-        idx = base + (unsigned long long)before;
-      }
-      if (emits) {
-#pragma unroll
-        for (int q = 0; q < kGrpKeys; q++) {
-          const bool refused_now = got[q] == kStRefused;
-          if (!(refused_now || got[q] == kStEvict)) continue;
-          const uint64_t iq = s_idx[q0 + q];
-          if (j == 0) {
-            a.evicted_keys[idx] = refused_now ? s_key[q0 + q] : victim[q];
-            if (a.evicted_scores) {
-              const uint64_t in_score = a.scores ? a.scores[iq] : 0;
-              a.evicted_scores[idx] = refused_now ? desired_when_missed(a, in_score, iq) : best_seen[q];
-            }
-          }
-          /* a refused key leaves with its own row, a victim that is a key of this
-           * pass with the row it came with, any other victim with its table row */
-          const uint8_t* src;
-          bool table = false;
-          if (refused_now) {
-            src = a.values_in + iq * v.value_bytes;
-          } else if (vic_from[q] >= 0) {
-            uint64_t ifrom = 0;
-#pragma unroll
-            for (int p = 0; p < q; p++)
-              if (vic_from[q] == p) ifrom = s_idx[q0 + p];
-            src = a.values_in + ifrom * v.value_bytes;
-          } else {
-            src = value_row(v, bslot + pos[q]);
-            table = true;
-          }
-          uint8_t* dst = a.evicted_values + idx * v.value_bytes;
-          for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
-            T x[UPL];
-#pragma unroll
-            for (int w = 0; w < UPL; w++) {
-              const uint32_t u = u0 + j + w * kTile;
-              x[w] = T{};
-              if (u < units) x[w] = table ? ld_unit<VEC, true>(src, u) : ld_unit<VEC, false>(src, u);
-            }
-#pragma unroll
-            for (int w = 0; w < UPL; w++) {
-              const uint32_t u = u0 + j + w * kTile;
-              if (u < units) st_unit<VEC, false>(dst, u, x[w]);
-            }
-          }
-          idx++;
-        }
       }
     }
 
@@ -621,7 +504,7 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
  *          asked for before the current one is worked on.
  * A list longer than kChainStage is finished in further rounds of walk and place.
  */
-template <int OP, int VEC, int UPL>
+template <int VEC, int UPL>
 __global__ void __launch_bounds__(kWave)
 __attribute__((amdgpu_waves_per_eu(3)))
 chained_miss_kernel(View v, UpsertArgs a, ChainArgs g) {
@@ -690,7 +573,7 @@ chained_miss_kernel(View v, UpsertArgs a, ChainArgs g) {
       if (w1 < nwork) dg1 = digests_of(w1);
       const uint32_t lb = s_list[w0];
       const uint32_t sb = lb * kChainStage;
-      group_bucket<OP, VEC, UPL>(v, a, g, (uint32_t)(b0 + lb), sb, sb + s_count[lb], s_key, s_idx,
+      group_bucket<VEC, UPL>(v, a, g, (uint32_t)(b0 + lb), sb, sb + s_count[lb], s_key, s_idx,
                                  s_info, units, lane, dg0);
       w0 = w1;
       dg0 = dg1;

@@ -186,10 +186,6 @@ struct hkv_table {
   uint64_t epoch;
   Clock clock;
   mutable StreamGroupLock lock;
-  void* d_scratch;          /* two-phase upserts: list heads per bucket + links per key */
-  uint64_t scratch_buckets; /* bucket count the heads were laid out for */
-  uint64_t scratch_keys;    /* links allocated */
-  int upsert_path; /* 0 choose per call, 1 slot locks always, 2 grouped whenever possible */
   bool reach_max_capacity; /* merlin_hashtable.cuh:1064: no further growth */
   bool keys_may_be_locked; /* LOCKED key words may sit in the table (lock_keys, the pointer
                               overload with locked_key_ptrs), until the count below reads 0 */
@@ -392,85 +388,40 @@ void launch_upsert_for(bool pair, int vec, const View& v, const UpsertArgs& a, h
   launch_upsert<OP, LOCKED_RULE, BOUNDS, 1>(vec, v, a, s);
 }
 
-/* Whether a batch goes through the two-phase path (hkv_grouped.hpp). */
-bool two_phase_feasible(const hkv_table* t, uint64_t n) {
-  /* the second phase has no locks: it needs the inserter's exclusivity */
-  if (t->upsert_path == 1 || !t->opts.api_lock || n >= (UINT64_C(1) << 31)) return false;
-  if (t->keys_may_be_locked) return false; /* the second phase does not look at key words */
-  if (t->upsert_path == 2) return true;
-  /* the second phase visits every bucket's head word: worth it for batches that reach a fair
-   * share of the buckets */
-  return n >= 32768 && n * 8 >= t->view.buckets_num;
-}
-
-template <template <int, int, int> class Launcher, int OP, class... Args>
+/* The two kernels of the two-phase insert_or_assign (hkv_grouped.hpp) for a row size. */
+template <template <int, int> class Launcher, class... Args>
 void dispatch_vec_upl(int vec, uint32_t value_bytes, Args&&... args) {
   if (vec == 16) {
     switch (pick_upl(value_bytes, 16)) {
-      case 1: Launcher<OP, 16, 1>::go(args...); break;
-      case 2: Launcher<OP, 16, 2>::go(args...); break;
-      case 4: Launcher<OP, 16, 4>::go(args...); break;
-      default: Launcher<OP, 16, 8>::go(args...); break;
+      case 1: Launcher<16, 1>::go(args...); break;
+      case 2: Launcher<16, 2>::go(args...); break;
+      case 4: Launcher<16, 4>::go(args...); break;
+      default: Launcher<16, 8>::go(args...); break;
     }
   } else if (vec == 4) {
-    Launcher<OP, 4, 8>::go(args...);
+    Launcher<4, 8>::go(args...);
   } else {
-    Launcher<OP, 1, 8>::go(args...);
+    Launcher<1, 8>::go(args...);
   }
 }
 
-template <int OP, int VEC, int UPL>
+template <int VEC, int UPL>
 struct LaunchHits {
   static void go(const View& v, const UpsertArgs& a, const ChainArgs& c, hipStream_t s) {
-    hipLaunchKernelGGL((upsert_hits_kernel<OP, VEC>), dim3(grid_for(a.n)), dim3(kWave), 0, s, v, a, c);
+    hipLaunchKernelGGL((upsert_hits_kernel<VEC>), dim3(grid_for(a.n)), dim3(kWave), 0, s, v, a, c);
   }
 };
-template <int OP, int VEC, int UPL>
+template <int VEC, int UPL>
 struct LaunchMisses {
   static void go(const View& v, const UpsertArgs& a, const ChainArgs& c, hipStream_t s) {
-    hipLaunchKernelGGL((chained_miss_kernel<OP, VEC, UPL>), dim3(grid_for(v.buckets_num)), dim3(kWave), 0,
+    hipLaunchKernelGGL((chained_miss_kernel<VEC, UPL>), dim3(grid_for(v.buckets_num)), dim3(kWave), 0,
                        s, v, a, c);
   }
 };
 
-/* Scratch of the two-phase path: the per-bucket list heads (all zero between calls) and the
- * per-key links.  Grown when a larger batch or a larger table comes along; the caller holds the
- * inserter role on `s`, so once `s` has drained nothing uses the old block any more. */
-int two_phase_scratch(hkv_table* t, uint64_t n, hipStream_t s, ChainArgs& c) {
-  auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
-  const uint64_t head_bytes = up(t->view.buckets_num * 4);
-  if (t->scratch_buckets != t->view.buckets_num || n > t->scratch_keys) {
-    HKV_HIP(hipStreamSynchronize(s));
-    table_free(t, 0, t->d_scratch);
-    t->d_scratch = nullptr;
-    t->scratch_buckets = t->scratch_keys = 0;
-    const uint64_t keys = std::max<uint64_t>(n + n / 4, 1 << 16);
-    HKV_TRY(table_alloc(t, 0, &t->d_scratch, head_bytes + up(keys * 4)));
-    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((head_bytes / 16 + 255) / 256)), dim3(256), 0, s,
-                       (uint32_t*)t->d_scratch, head_bytes / 4);
-    HKV_HIP(hipGetLastError());
-    t->scratch_buckets = t->view.buckets_num;
-    t->scratch_keys = keys;
-  }
-  c.head = (uint32_t*)t->d_scratch;
-  c.next = (uint32_t*)((uint8_t*)t->d_scratch + head_bytes);
-  return HKV_SUCCESS;
-}
-
-/* Caller holds the inserter role on `s`. */
-template <int OP>
-int run_two_phase(hkv_table* t, const UpsertArgs& a, int vec, bool locked_rule, hipStream_t s) {
-  ChainArgs c{};
-  HKV_TRY(two_phase_scratch(t, a.n, s, c));
-  c.locked_rule = locked_rule;
-  dispatch_vec_upl<LaunchHits, OP>(vec, t->view.value_bytes, t->view, a, c, s);
-  dispatch_vec_upl<LaunchMisses, OP>(vec, t->view.value_bytes, t->view, a, c, s);
-  return HKV_SUCCESS;
-}
-
-/* ---- the two-phase path on a scratch area that is part of the library image -----------------
- * hkv_insert_or_assign_noalloc: list heads and links live in a file-scope device array instead
- * of memory the call may have to allocate.  In host code the array's name is only a handle for
+/* ---- the two-phase insert_or_assign on a scratch area that is part of the library image -------
+ * hkv_insert_or_assign_noalloc: list heads and links live in a file-scope device array, so the
+ * call allocates nothing.  In host code the array's name is only a handle for
  * the symbol: its device address is looked up once per device (each device holds its own copy
  * of the array) and that pointer is what the kernels and the clearing launch get. */
 constexpr uint64_t kNoAllocMaxBuckets = UINT64_C(1) << 20; /* capacity up to 2^27 */
@@ -861,19 +812,9 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
     HKV_HIP(g.acquire());
     HKV_TRY(settle_locked_count(t, s));
     if (OP == kOpFindOrInsertPtr && a.locked_key_ptrs) t->keys_may_be_locked = true;
-    bool two_phase = OP != kOpFindOrInsertPtr && two_phase_feasible(t, a.n);
-    /* insert_and_evict: the second phase updates the one evicted-counter word once per
-     * wavefront and pass, and updates of one word are served one at a time; only the forced
-     * mode of the tests takes it there */
-    if (OP == kOpInsertAndEvict && t->upsert_path != 2) two_phase = false;
-    if (vec == 8 || vec == 2) two_phase = false; /* units only the slot-lock kernel has */
     /* a table that has been offered fewer keys than nine tenths of its slots evicts next to nothing */
     const bool pair = OP == kOpInsertAndEvict && t->keys_offered * 10 >= t->view.capacity * 9;
-    if (two_phase) {
-      writes_scores_outside_bounds(t, s, own_rule);
-      if constexpr (OP != kOpFindOrInsertPtr)
-        HKV_TRY(run_two_phase<OP>(t, a, vec, refuse_equal, s));
-    } else if (t->keys_may_be_locked) {
+    if (t->keys_may_be_locked) {
       /* slots that lock_keys (or the pointer overload with locked_key_ptrs) left LOCKED must
        * be hidden from the victim scan, which then reads the key words beside the scores; with
        * no such slot the plain scan finds the same victims (a slot locked by another key of
@@ -1213,27 +1154,16 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->d_values = nullptr;
   t->d_counters = nullptr;
   t->h_values = nullptr;
-  t->d_scratch = nullptr;
-  t->scratch_buckets = t->scratch_keys = 0;
   t->keys_may_be_locked = false;
   t->locked_recount = false;
   t->dual = o->table_mode == 1;
   t->io_by_cpu = o->io_by_cpu != 0;
   t->io_stage = nullptr;
   t->io_stage_bytes = 0;
-  /* HKV_UPSERT_PATH: "locked" = slot-lock kernel always (the default: it is the faster
-   * one per find + insert_or_assign step), "auto" = two-phase for large batches,
-   * "grouped" = two-phase whenever it is possible (tests) */
-  t->upsert_path = 1;
   {
     const char* b = getenv("HKV_SCORE_BOUNDS");
-    /* only LRU keeps them right by itself (hkv_upsert.hpp); other tables carry none */
+    /* dual-bucket tables have their own kernel, which scans both buckets */
     t->score_bounds = !(b && !strcmp(b, "0")) && !t->dual;
-  }
-  if (const char* e = getenv("HKV_UPSERT_PATH")) {
-    if (!strcmp(e, "auto")) t->upsert_path = 0;
-    if (!strcmp(e, "locked")) t->upsert_path = 1;
-    if (!strcmp(e, "grouped")) t->upsert_path = 2;
   }
   memset(&t->view, 0, sizeof t->view);
   t->epoch = kIgnoredEpoch;
@@ -1379,7 +1309,6 @@ int hkv_table_destroy(hkv_table* t) {
   (void)hipDeviceSynchronize();
   table_free(t, 0, t->d_meta);
   table_free(t, 0, t->d_counters);
-  table_free(t, 0, t->d_scratch);
   table_free(t, 0, t->d_values);
   table_free(t, 1, t->h_values);
   if (t->io_stage) (void)hipHostFree(t->io_stage);
@@ -1481,8 +1410,8 @@ int hkv_insert_or_assign_noalloc(hkv_table* t, uint64_t n, const uint64_t* keys,
     const uint64_t head_words = (t->view.buckets_num + 3) & ~UINT64_C(3);
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((head_words / 4 + 255) / 256)), dim3(256), 0, s,
                        c.head, head_words);
-    dispatch_vec_upl<LaunchHits, kOpInsertOrAssign>(vec, t->view.value_bytes, t->view, a, c, s);
-    dispatch_vec_upl<LaunchMisses, kOpInsertOrAssign>(vec, t->view.value_bytes, t->view, a, c, s);
+    dispatch_vec_upl<LaunchHits>(vec, t->view.value_bytes, t->view, a, c, s);
+    dispatch_vec_upl<LaunchMisses>(vec, t->view.value_bytes, t->view, a, c, s);
     HKV_HIP(hipGetLastError());
   }
   if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;

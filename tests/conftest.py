@@ -17,11 +17,3 @@ def pytest_configure(config):
 def oracle():
     import oracle_binding
     return oracle_binding
-
-
-@pytest.fixture(params=["locked", "grouped"])
-def upsert_path(request, monkeypatch):
-    """Run a GPU test once per upsert implementation: the slot-lock kernel and
-    the two-phase path (the library reads HKV_UPSERT_PATH when a table is created)."""
-    monkeypatch.setenv("HKV_UPSERT_PATH", request.param)
-    return request.param

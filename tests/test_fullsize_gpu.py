@@ -71,9 +71,7 @@ def export_keys(t, vb_unused, pred=Predicate.kAlways, pattern=0, threshold=0, wi
 
 # ---- configuration 2: 2^26 slots, dim 8, LRU; load factors 0.50 / 0.75 / 1.00 -----------------------------
 
-@pytest.mark.parametrize("path", ["locked", "auto"])
-def test_config2_throughput_shape_full_size(path, monkeypatch):
-    monkeypatch.setenv("HKV_UPSERT_PATH", path)
+def test_config2_throughput_shape_full_size():
     cap, dim, n, seed = 1 << 26, 8, 1 << 20, 2
     t = make_table(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * dim * 4, dim=dim,
                    evict_strategy=EvictStrategy.kLru)
@@ -152,9 +150,7 @@ def test_config2_throughput_shape_full_size(path, monkeypatch):
 
 # ---- configuration 3: 2^27 slots, dim 64 (32 GB of rows), Customized, Zipf insert_and_evict ------------------
 
-@pytest.mark.parametrize("path", ["locked", "auto"])
-def test_config3_insert_and_evict_full_size(path, monkeypatch):
-    monkeypatch.setenv("HKV_UPSERT_PATH", path)
+def test_config3_insert_and_evict_full_size():
     cap, dim, n, seed = 1 << 27, 64, 1 << 20, 3
     t = make_table(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * dim * 4, dim=dim,
                    evict_strategy=EvictStrategy.kCustomized)
@@ -280,9 +276,7 @@ def test_config4_hybrid_full_size():
 
 # ---- configuration 5: 2^25 slots, dim 128, EpochLRU; accum_or_assign, export_batch_if, erase ------------------
 
-@pytest.mark.parametrize("path", ["locked", "auto"])
-def test_config5_update_export_full_size(path, monkeypatch):
-    monkeypatch.setenv("HKV_UPSERT_PATH", path)
+def test_config5_update_export_full_size():
     cap, dim, n, seed = 1 << 25, 128, 1 << 20, 5
     t = make_table(init_capacity=cap, max_capacity=cap, max_hbm_for_vectors=cap * dim * 4, dim=dim,
                    evict_strategy=EvictStrategy.kEpochLru)

@@ -95,7 +95,6 @@ class LibraryDriver:
 
 
 @pytest.mark.gpu
-@pytest.mark.usefixtures("upsert_path")
 def test_library_reproduces_the_fixture():
     inp, want = load_fixture()
     d = LibraryDriver()

@@ -12,7 +12,7 @@ from gpu_util import (DEV, assert_same_table, dev, export_table, host_bytes, hos
 from hierarchicalkv_amd import (EvictStrategy, HashTable, MerlinException, Predicate, ValueKind,
                                 default_options)
 
-pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("upsert_path")]
+pytestmark = pytest.mark.gpu
 M64 = (1 << 64) - 1
 
 

@@ -17,7 +17,7 @@ from gpu_util import (DEV, assert_same_table, canonical_evicted, dev, export_tab
 from hierarchicalkv_amd import (EvictStrategy, HashTable, MerlinException, Predicate, ValueKind,
                                 default_options)
 
-pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("upsert_path")]
+pytestmark = pytest.mark.gpu
 
 
 def make_pair(oracle, hybrid=False, **kw):

@@ -12,7 +12,7 @@ from gpu_util import (DEV, assert_same_table, canonical_evicted, dev, export_tab
                       host_u64, sort_by_key)
 from hierarchicalkv_amd import EvictStrategy, HashTable, Predicate, default_options
 
-pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("upsert_path")]
+pytestmark = pytest.mark.gpu
 
 
 def bytes_of(a):

@@ -66,6 +66,62 @@ def test_noalloc_equals_insert_or_assign_on_two_calls_in_a_row(oracle, strategy)
         t.close()
 
 
+@pytest.mark.parametrize("dim,strategy", [(3, EvictStrategy.kCustomized), (8, EvictStrategy.kLfu),
+                                          (64, EvictStrategy.kEpochLru), (128, EvictStrategy.kEpochLfu),
+                                          (300, EvictStrategy.kLru)])
+def test_noalloc_row_sizes_strategies_and_long_lists(oracle, dim, strategy):
+    """The two-phase path by itself against the oracle: rows of 12 bytes (4-byte units), 32, 256, 512
+    and 1200 bytes (more than one pass of a tile), every strategy, a table of 32 buckets so that a
+    bucket takes dozens of keys of one call (lists longer than one staging round), free slots left
+    by erase, hits and new keys mixed."""
+    cap = 1 << 12
+    vb = dim * 4
+    opts = default_options(init_capacity=cap, max_capacity=cap, dim=dim, max_hbm_for_vectors=1 << 30,
+                           evict_strategy=strategy)
+    t = HashTable()
+    t.init(opts)
+    o = oracle.OracleTable(opts)
+    clocked = strategy in (EvictStrategy.kLru, EvictStrategy.kEpochLru)
+    if clocked:
+        t.set_clock(1, 1 << 44)
+        o.set_clock(1, 1 << 44)
+    if strategy in (EvictStrategy.kEpochLru, EvictStrategy.kEpochLfu):
+        t.set_global_epoch(2)
+        o.set_global_epoch(2)
+    seed, pos, batch = 700 + dim, 0, 1
+
+    def call(keys, bump=0.0):
+        nonlocal batch
+        n = len(keys)
+        vals = w.values_from_keys(keys, dim) + np.float32(bump)
+        # distinct, growing from call to call, and below 2^32 (EpochLFU keeps the low half only)
+        sc = None if clocked else ((np.uint64(batch) << np.uint64(20)) +
+                                   np.random.Generator(np.random.PCG64(batch)).permutation(n).astype(np.uint64))
+        batch += 1
+        t.insert_or_assign_noalloc(n, dev(keys), dev(vals), dev(sc))
+        o.insert_or_assign(keys, vals.view(np.uint8).reshape(n, vb), sc)
+        torch.cuda.synchronize()
+        assert_same_table(t, o, vb)
+
+    for n in (1500, 3000, 3000):  # past load factor 1.0 from an empty table: free slots, then victims
+        call(w.unique_keys(seed, pos, n))
+        pos += n
+    gone = w.unique_keys(seed, pos - 1000, 700)
+    t.erase(len(gone), dev(gone))
+    o.erase(gone)
+    assert_same_table(t, o, vb)
+    for rep in range(3):
+        # hits are keys of the latest call (the highest scores: no key of the batch can evict one
+        # of them before its turn; under LFU they only gain), the rest is new
+        old = w.unique_keys(seed, pos - 600, 600)
+        old = old[o.contains(old)]
+        new = w.unique_keys(seed, pos, 2001)
+        pos += 2001
+        call(np.concatenate([old, new]), bump=rep + 1.0)
+    t.close()
+    o.close()
+
+
 def test_noalloc_refuses_what_it_cannot_do():
     dim = 4
     grow = HashTable()
