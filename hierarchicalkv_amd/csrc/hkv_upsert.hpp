@@ -435,7 +435,9 @@ template <int VEC, int UPL, bool CAN_READ_TABLE, bool CAN_ACCUM>
 __device__ __forceinline__ void bulk_rows(int move, uint8_t* tab, uint8_t* usr,
                                           uint32_t units, int value_kind, int lane) {
   using T = typename VecType<VEC>::type;
-  constexpr int kGroup = kRowUnits / UPL < 1 ? 1 : (kRowUnits / UPL < kTile ? kRowUnits / UPL : kTile);
+  /* accumulating holds two rows per key (the table's and the caller's): half as many keys at a time */
+  constexpr int kUnits = CAN_ACCUM ? kRowUnits / 2 : kRowUnits;
+  constexpr int kGroup = kUnits / UPL < 1 ? 1 : (kUnits / UPL < kTile ? kUnits / UPL : kTile);
   const int j = lane & (kTile - 1);
   const int lane_base = lane & ~(kTile - 1);
   for (uint32_t u0 = 0; u0 < units; u0 += kTile * UPL) {
@@ -594,7 +596,7 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * and two wavefronts that wait for each other in every trip are 4 % slower than one.) */
 template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1>
 __global__ void __launch_bounds__(kWave * WAVES)
-    __attribute__((amdgpu_waves_per_eu(BOUNDS && OP != kOpAccumOrAssign ? 4 : 1)))
+    __attribute__((amdgpu_waves_per_eu(BOUNDS ? 4 : 1)))
 upsert_kernel(View v, UpsertArgs a) {
   static_assert(!(BOUNDS && LOCKED_RULE), "the bounded search does not look at key words");
   static_assert(WAVES == 1 || OP == kOpInsertAndEvict, "only insert_and_evict has anything to share");
