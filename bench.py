@@ -1383,12 +1383,11 @@ CEILING_PATTERNS = [
     ("small_xchg32_side", "32-bit exchange on a 4-byte-per-bucket array (fits the Infinity Cache)", "G ops/s"),
     # (new patterns go to the end: --profile-summary finds the launches of the ones above by their order)
     ("upsert_pattern_free", "insert_or_assign's accesses on a table with free slots, chained: 50 % absent keys that "
-                            "take a free slot with a compare-and-swap and add one to the bucket's counter, no score "
-                            "reads (algorithmic bytes)", "GB/s"),
+                            "take a free slot with a compare-and-swap, no score reads (algorithmic bytes)", "GB/s"),
     ("findptr_pattern", "find* / contains: batch key -> digest line -> key word (1.1 lines per key) -> 8-byte result "
                         "and flag (algorithmic bytes: 153 per key)", "GB/s"),
     ("erase_pattern", "erase with the table to itself: batch key -> digest line -> key word -> key store, digest "
-                      "store, one atomic on the bucket's counter (algorithmic bytes: 165 per key)", "GB/s"),
+                      "store (algorithmic bytes: 165 per key)", "GB/s"),
 ]
 
 

@@ -184,8 +184,7 @@ k_find_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm) {
  * present key, an exchange and a score re-read per absent key (the key store of an absent
  * key doubles as its unlock).
  * locks == 3: a table with free slots.  An absent key reads no scores: it takes a free slot with
- * a compare-and-swap and adds one to the bucket's counter (a 32-bit atomic on the 4-byte-per-bucket
- * array); a quarter of the absent keys fetch a key line for a false digest match. */
+ * a compare-and-swap; a quarter of the absent keys fetch a key line for a false digest match. */
 template <bool CHAIN>
 __global__ void __launch_bounds__(64)
 k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int locks) {
@@ -279,7 +278,6 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
     st1_wt(b.digests + slot, (uint8_t)acc);
     st8_wt(b.keys + slot, acc);
     if (locks == 2) st8_wt(reinterpret_cast<uint64_t*>(b.digests) + (slot >> 4), acc);
-    if (free_mode) atomicAdd(b.small + bk, 1u);
   }
   /* rows: dense input -> table rows, 64 rows x units over the 64 lanes */
   const uint32_t upr = sh.row_bytes / 16;
@@ -314,7 +312,7 @@ k_upsert_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int lock
  * Probe as find's (batch key, digest line, one key word, a second one for `extra_pm` keys in 1000);
  * kind 0 (find* / contains): one 8-byte result and one flag per key;
  * kind 1 (erase with the table to itself): an 8-byte key store and a 1-byte digest store into the
- *        table, and one 32-bit atomic on the bucket's counter per key. */
+ *        table. */
 __global__ void __launch_bounds__(64)
 k_norow_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int kind) {
   const int lane = threadIdx.x, tile = lane >> 3, j = lane & 7;
@@ -344,7 +342,6 @@ k_norow_pattern(Shape sh, Buffers b, uint64_t salt, uint32_t extra_pm, int kind)
   } else {
     b.keys[slot] = acc;
     b.digests[slot] = (uint8_t)acc;
-    atomicAdd(b.small + bk, 1u);
   }
 }
 

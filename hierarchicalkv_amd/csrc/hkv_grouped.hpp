@@ -280,7 +280,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
   const uint8_t* rows_in = a.values_in;
 
   bool dg_dirty = false;
-  int size_delta = 0;
 
   /* free slots of the bucket, bit p for slot p */
   uint64_t em_lo = 0, em_hi = 0;
@@ -367,7 +366,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
         pos[q] = p;
         if (j == (int)(p >> 4)) dg_set(dg, p & 15u, info & 0xFFu);
         dg_dirty = true;
-        size_delta++;
         continue;
       }
       if (!scanned) {
@@ -447,7 +445,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
     for (int q = 0; q < kGrpKeys; q++) {
       if (got[q] == kStEvict && need_vk[q] && victim[q] == v.reclaim_key) {
         got[q] = kStReclaimed;
-        size_delta++;
       }
     }
 
@@ -490,7 +487,6 @@ __device__ __forceinline__ void group_bucket(const View& v, const UpsertArgs& a,
   }
 
   if (dg_dirty) st_u128(v.digests + bslot + j * 16, dg);
-  if (size_delta && j == 0) atomicAdd(v.sizes + bkt, size_delta);
 }
 
 /*

@@ -30,7 +30,7 @@ fill_kernel(View v, int zero_scores) {
     }
     if (v.bounds) v.bounds[t] = 0; /* one per 16 slots */
   }
-  if (t < v.buckets_num) v.sizes[t] = 0;
+  if (v.sizes && t < v.buckets_num) v.sizes[t] = 0;
 }
 
 /* one sample of the constant-rate device counter (table creation: see Clock) */
@@ -41,8 +41,9 @@ __global__ void clock_sample_kernel(unsigned long long* out) { *out = wall_clock
  * of the group lock), so the key word is overwritten with a plain store as in the reference
  * (core_kernels.cuh:723-737; like there, a batch that names a key twice in different
  * wavefronts may count it twice).  Otherwise the slot changes hands with a compare-and-swap.
- * Keys of an 8-lane tile that fall into one bucket share one update of its size, and a key
- * that the tile holds twice is erased once. */
+ * A key that an 8-lane tile holds twice is erased once.  No counter is kept per bucket (the
+ * number of keys of a table is the number of digests that are not the EMPTY marker, counted
+ * when somebody asks), so an erase is two stores. */
 template <bool EXCLUSIVE>
 __global__ void __launch_bounds__(kWave)
 erase_kernel(View v, const uint64_t* keys, uint64_t n) {
@@ -83,35 +84,27 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
       if (!EXCLUSIVE) st_u64(v.keys + slot, v.empty_key);
     }
   }
-  const uint32_t bkt = erased ? (uint32_t)(slot >> 7) : 0xFFFFFFFFu;
-  int same = 0;
-  bool first = true;
-#pragma unroll
-  for (int q = 0; q < kTile; q++) {
-    const uint32_t other = __shfl(bkt, tile_base + q);
-    if (other == bkt) {
-      same++;
-      if (q < j) first = false;
-    }
-  }
-  if (erased && first) atomicSub(v.sizes + bkt, same);
 }
 
-/* Sum of the per-bucket sizes (SumOp over buckets_size, core_kernels.cuh:1395-1423) */
+/* Number of keys of the table (the reference sums per-bucket counters, SumOp over buckets_size,
+ * core_kernels.cuh:1395-1423).  A slot holds a key exactly when its digest is not the EMPTY
+ * marker (a live key never stores that byte, erase and clear put it back), so the count is one
+ * streaming pass over the digest array, 16 bytes per lane and step; no call that inserts or
+ * erases pays for a counter.  The first `buckets` buckets are counted (all of them for size(),
+ * the first 1024 for the load-factor estimate, merlin_hashtable.cuh:3796-3830).
+ * Few blocks: the one word they all add to takes one update at a time. */
 __global__ void __launch_bounds__(256)
-size_kernel(View v, unsigned long long* out) {
-  /* the array starts on a 256-byte boundary: four counters per load, the tail one by one;
-   * few blocks, because the one word they all add to takes one update at a time */
+size_kernel(View v, uint64_t buckets, unsigned long long* out) {
   uint64_t local = 0;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const uint64_t quads = v.buckets_num / 4;
-  const int4* q = reinterpret_cast<const int4*>(v.sizes);
-  for (uint64_t b = tid; b < quads; b += stride) {
-    const int4 x = q[b];
-    local += (uint64_t)x.x + (uint64_t)x.y + (uint64_t)x.z + (uint64_t)x.w;
+  const uint64_t groups = buckets * (kBucketSize / 16);
+  const uint32_t e4 = v.empty_digest * 0x01010101u;
+  const uint4* d = reinterpret_cast<const uint4*>(v.digests);
+  for (uint64_t g = tid; g < groups; g += stride) {
+    const uint4 x = d[g];
+    local += 16 - __popc(match16(x, e4));
   }
-  for (uint64_t b = quads * 4 + tid; b < v.buckets_num; b += stride) local += (uint64_t)v.sizes[b];
   __shared__ unsigned long long s_part[4];
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
@@ -129,8 +122,7 @@ size_kernel(View v, unsigned long long* out) {
  * of the new table, and both start out empty: every entry can keep its slot
  * position, so no destination search and no compaction is needed (positions
  * are not observable through the API).  Tombstones stay in bucket b.  One
- * wavefront per 64 slots; it counts its live keys per destination bucket with
- * two ballots and moves their rows together.
+ * wavefront per 64 slots; it moves the rows of its live keys together.
  */
 __global__ void __launch_bounds__(256)
 rehash_kernel(View src, View dst) {
@@ -155,14 +147,7 @@ rehash_kernel(View src, View dst) {
     dst.digests[d] = src.digests[s];
     dst.scores[d] = src.scores[s];
   }
-  const unsigned long long stay = __ballot(live && nb == b);
-  const unsigned long long move = __ballot(live && nb != b);
-  if (lane == 0) {
-    /* the 64 slots of a wavefront belong to one bucket */
-    if (stay) atomicAdd(dst.sizes + b, (int)__popcll(stay));
-    if (move) atomicAdd(dst.sizes + b + src.buckets_num, (int)__popcll(move));
-  }
-  unsigned long long rest = stay | move;
+  unsigned long long rest = __ballot(live);
   while (rest) {
     const int l = __ffsll(rest) - 1;
     rest &= rest - 1;
@@ -171,13 +156,15 @@ rehash_kernel(View src, View dst) {
   }
 }
 
-/* sum of the sizes of the first n buckets (fast_load_factor,
- * merlin_hashtable.cuh:3796-3830); one workgroup */
+/* keys in the first n buckets (fast_load_factor, merlin_hashtable.cuh:3796-3830); one workgroup,
+ * which stores its whole result in one write */
 __global__ void __launch_bounds__(256)
-partial_size_kernel(View v, uint32_t n, unsigned long long* out) {
+load_sample_kernel(View v, uint32_t n, unsigned long long* out) {
   __shared__ unsigned long long s_part[4];
   unsigned long long local = 0;
-  for (uint32_t b = threadIdx.x; b < n; b += 256) local += (unsigned long long)v.sizes[b];
+  const uint32_t e4 = v.empty_digest * 0x01010101u;
+  const uint4* d = reinterpret_cast<const uint4*>(v.digests);
+  for (uint32_t g = threadIdx.x; g < n * (kBucketSize / 16); g += 256) local += 16 - __popc(match16(d[g], e4));
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;
   __syncthreads();

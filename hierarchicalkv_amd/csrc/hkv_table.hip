@@ -544,19 +544,20 @@ int alloc_arenas(hkv_table* t, uint64_t buckets_num, View& v, TableMem& m) {
   v.buckets_num = buckets_num;
   v.capacity = buckets_num * kBucketSize;
   v.pow2_buckets = ispow2(buckets_num);
-  /* metadata arena: digests | keys | scores | sizes | score bounds, each 256-byte aligned */
+  /* metadata arena: digests | keys | scores | sizes (dual-bucket tables) | score bounds, each 256-byte aligned */
   auto up = [](uint64_t x) { return (x + 255) & ~UINT64_C(255); };
   const uint64_t off_keys = up(v.capacity);
   const uint64_t off_scores = off_keys + up(v.capacity * 8);
   const uint64_t off_sizes = off_scores + up(v.capacity * 8);
-  const uint64_t off_bounds = off_sizes + up(v.buckets_num * 4);
+  const uint64_t off_bounds = off_sizes + (t->dual ? up(v.buckets_num * 4) : 0);
   m.meta_bytes = off_bounds + (t->score_bounds ? up(v.buckets_num * 8 * sizeof(uint64_t)) : 0);
   HKV_TRY(table_alloc(t, 0, &m.d_meta, m.meta_bytes));
   uint8_t* base = (uint8_t*)m.d_meta;
   v.digests = base;
   v.keys = (uint64_t*)(base + off_keys);
   v.scores = (uint64_t*)(base + off_scores);
-  v.sizes = (int32_t*)(base + off_sizes);
+  /* keys per bucket: only the two-choice placement of a dual-bucket table reads them */
+  v.sizes = t->dual ? (int32_t*)(base + off_sizes) : nullptr;
   v.bounds = t->score_bounds ? (uint64_t*)(base + off_bounds) : nullptr;
   /* value rows: whole buckets in HBM while max_hbm_for_vectors lasts
    * (initialize_buckets, core_kernels.cuh:195-236), the rest pinned + mapped */
@@ -649,7 +650,7 @@ int fast_load_factor(hkv_table* t, uint64_t delta, hipStream_t s, float* out) {
   {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
-    hipLaunchKernelGGL(partial_size_kernel, dim3(1), dim3(256), 0, s, t->view, n, d);
+    hipLaunchKernelGGL(load_sample_kernel, dim3(1), dim3(256), 0, s, t->view, n, d);
     HKV_HIP(hipGetLastError());
   }
   unsigned long long sum = 0;
@@ -1931,9 +1932,10 @@ int hkv_size(const hkv_table* t, hkv_stream_t stream, uint64_t* out) {
     LockGuard g(t, StreamGroupLock::kReader, s);
     HKV_HIP(g.acquire());
     hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, d);
+    /* 16 digest bytes per lane and step; a workgroup per 2^16 slots, 512 at most */
     const unsigned blocks =
-        (unsigned)std::min<uint64_t>((t->view.buckets_num + 4095) / 4096, 128);
-    hipLaunchKernelGGL(size_kernel, dim3(blocks), dim3(256), 0, s, t->view, d);
+        (unsigned)std::min<uint64_t>((t->view.capacity + 65535) / 65536, 512);
+    hipLaunchKernelGGL(size_kernel, dim3(blocks), dim3(256), 0, s, t->view, t->view.buckets_num, d);
     HKV_HIP(hipGetLastError());
   }
   return lease.read(out);

@@ -890,7 +890,6 @@ upsert_kernel(View v, UpsertArgs a) {
       if (BOUNDS && a.bound_ceil && stored < bound_ceil &&
           (got == kStEmpty || (got == kStDuplicate && a.strategy == HKV_CUSTOMIZED)))
         __hip_atomic_fetch_min(v.bounds + (slot >> 4), stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (got == kStEmpty || got == kStReclaimed) atomicAdd(v.sizes + me.bkt, 1);
     }
     if (OP == kOpInsertAndEvict && total) {
       if (threadIdx.x == 0) s_claim[set] = claimed;

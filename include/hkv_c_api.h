@@ -109,7 +109,8 @@ typedef struct hkv_table_view {
   uint8_t* digests;  /* [buckets_num][128] one byte per slot                 */
   uint64_t* keys;    /* [buckets_num][128]                                   */
   uint64_t* scores;  /* [buckets_num][128]                                   */
-  int32_t* sizes;    /* [buckets_num] live keys per bucket                   */
+  int32_t* sizes;    /* dual-bucket tables: [buckets_num] keys per bucket; else NULL (a
+                        slot holds a key exactly when its digest is not empty_digest) */
   uint8_t* values;   /* HBM part of the value rows, slot-major               */
   uint8_t* host_values; /* pinned host part (hybrid mode) or NULL            */
   uint64_t hbm_slots;   /* slots [0,hbm_slots) live in `values`, the rest in

@@ -8,7 +8,8 @@
  *   digests[b][128] u8   one 128-byte line per bucket
  *   keys[b][128]    u64
  *   scores[b][128]  u64
- *   sizes[b]        i32
+ *   sizes[b]        i32  keys per bucket, dual-bucket tables only (elsewhere a slot holds a key
+ *                        exactly when its digest is not the EMPTY marker)
  *   values          slot-major rows of value_bytes; slots below hbm_slots in
  *                   HBM, the rest in pinned host memory (hybrid mode)
  */
@@ -260,7 +261,7 @@ erase_if_kernel(hkv_table_view v, Pred pred, uint64_t pattern, uint64_t threshol
       /* a free slot again, not a tombstone: see erase_kernel */
       v.keys[s] = v.empty_key;
       v.digests[s] = v.empty_digest;
-      atomicSub(v.sizes + (s >> 7), 1);
+      if (v.sizes) atomicSub(v.sizes + (s >> 7), 1);
       local++;
     }
   }
@@ -420,7 +421,7 @@ erase_if_v2_kernel(hkv_table_view v, uint64_t n, Pred pred, unsigned long long* 
     if (match) {
       v.digests[slot] = v.empty_digest;
       v.keys[slot] = v.empty_key;
-      atomicSub(v.sizes + (slot >> 7), 1);
+      if (v.sizes) atomicSub(v.sizes + (slot >> 7), 1);
       local++;
     }
   }
