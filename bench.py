@@ -813,6 +813,16 @@ def summarize_configs(root, pick, counters, durations):
                     o.append(ln.rstrip())
                 if ln.startswith("{") and '"config"' in ln:
                     line = ln.strip()
+        if line:
+            try:
+                peak = json.loads(line).get("host_link_peak")
+            except ValueError:
+                peak = None
+            if peak:
+                o.append("\nHost link in the same run, pinned host memory <-> device copies of 1 GiB: %.1f GB/s host to "
+                         "device, %.1f GB/s device to host; `host_link_gbs` above is the bytes of the rows that live "
+                         "in pinned host memory over the call's time, `hbm_gbs` the rest of the call's algorithmic "
+                         "bytes over the same time." % (peak["h2d_gbs"], peak["d2h_gbs"]))
         name = "config" + tag[3:]
         path = os.path.join(ROOT, "profiles", name + ".md")
         with open(path, "w") as f:
@@ -959,8 +969,9 @@ def summarize_profiles(root):
                 col(r, "TCC_EA0_RDREQ_32B_sum", 1e-6, "%.3f"), col(r, "TCC_EA0_WRREQ_sum", 1e-6),
                 col(r, "TCC_EA0_WRREQ_64B_sum", 1e-6), part, col(r, "TCC_EA0_ATOMIC_sum", 1e-6)))
         o.append("\n## Wavefronts, LDS, vector memory, address translation\n")
-        o.append("Registers per lane: twice rocprofv3's VGPR_Count field, which counts register pairs on this part (the "
-                 "compiler's resource report for the same kernels reads 114 and 118 registers, both allocated as 120).\n")
+        o.append("Registers per lane: twice rocprofv3's VGPR_Count field, which counts register pairs on this part "
+                 "(registers are allocated in blocks of 8: the compiler's resource report for `lookup_kernel<0, 16>` reads "
+                 "114, for the bounded `upsert_kernel<0, 16, 2>` 125).\n")
         o.append("| call | wavefronts | vector registers per lane | LDS bytes per workgroup | scratch | occupancy % of the maximum | vector memory reads "
                  "/ writes (M instructions) | L1 -> L2 read / write requests (M) | returning atomics (M) | L1 TLB misses (M) | "
                  "LDS instructions (M) | LDS bank-conflict cycles (M) |\n|---|---|---|---|---|---|---|---|---|---|---|---|")

@@ -101,10 +101,14 @@ size_kernel(View v, uint64_t buckets, unsigned long long* out) {
   const uint64_t groups = buckets * (kBucketSize / 16);
   const uint32_t e4 = v.empty_digest * 0x01010101u;
   const uint4* d = reinterpret_cast<const uint4*>(v.digests);
-  for (uint64_t g = tid; g < groups; g += stride) {
-    const uint4 x = d[g];
-    local += 16 - __popc(match16(x, e4));
+  /* four loads in flight per lane */
+  uint64_t g = tid;
+  for (; g + 3 * stride < groups; g += 4 * stride) {
+    const uint4 x0 = d[g], x1 = d[g + stride], x2 = d[g + 2 * stride], x3 = d[g + 3 * stride];
+    local += 64 - __popc(match16(x0, e4)) - __popc(match16(x1, e4)) - __popc(match16(x2, e4)) -
+             __popc(match16(x3, e4));
   }
+  for (; g < groups; g += stride) local += 16 - __popc(match16(d[g], e4));
   __shared__ unsigned long long s_part[4];
   for (int off = 32; off > 0; off >>= 1) local += __shfl_xor(local, off);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = local;

@@ -936,6 +936,7 @@ int cpu_io_upsert(hkv_table* t, UpsertArgs a, void* values, bool reads, hipStrea
     e = g.acquire();
     if (e == hipSuccess) e = hipMemsetAsync(d_tmp, 0, n * 9, s); /* reserved / refused keys: no address */
     if (e == hipSuccess) {
+      writes_scores_outside_bounds(t, s, a.strategy == t->opts.evict_strategy);
       launch_upsert<kOpFindOrInsertPtr, true>(16, t->view, a, s);
       hipLaunchKernelGGL(cpu_io_owner_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s,
                          t->view, a.keys, (uint8_t**)d_tmp,
