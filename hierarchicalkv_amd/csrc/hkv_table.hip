@@ -1622,8 +1622,10 @@ static int assign_common(hkv_table* t, uint64_t n, const uint64_t* keys,
   {
     LockGuard g(t, StreamGroupLock::kUpdater, s);
     HKV_HIP(g.acquire());
-    /* Customized: the caller's score replaces the old one and may be below the line's bound */
-    if (t->score_bounds && touch_scores && scores && a.strategy == HKV_CUSTOMIZED) {
+    /* Customized: the caller's score replaces the old one and may be below the line's bound;
+     * EpochLFU: so may the old count under today's epoch, if the key carries a later one */
+    if (t->score_bounds && touch_scores && scores &&
+        (a.strategy == HKV_CUSTOMIZED || a.strategy == HKV_EPOCH_LFU)) {
       if (t->bounds_stale || capturing(s))
         writes_scores_outside_bounds(t, s, true);
       else

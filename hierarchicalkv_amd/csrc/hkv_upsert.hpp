@@ -670,7 +670,18 @@ upsert_kernel(View v, UpsertArgs a) {
     if (__ballot(pending && reprobe))
       settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, waited, lane);
 
-    const bool active = pending && !reprobe;
+    bool active = pending && !reprobe;
+    if constexpr (OP == kOpAccumOrAssign) {
+      /* accum_or_assign.cuh:139-156: a key whose flag and presence disagree (accumulate onto
+       * a key that is not there, assign to one that is) changes nothing.  It is done without
+       * a lock: the reference takes the slot and gives it back, and a free slot that is given
+       * back has meanwhile been crossed off by the bucket's other new keys, which then look
+       * for a victim in a bucket that is not full. */
+      if (active && (a.accum_flags[i] != 0) != (hit >= 0)) {
+        pending = false;
+        active = false;
+      }
+    }
     const uint64_t desired = desired_when_missed(a, in_score, i);
     int got = kStNone;
     uint32_t pos = 0;
@@ -755,8 +766,8 @@ upsert_kernel(View v, UpsertArgs a) {
      * (EMPTY -> LOCKED: the first free slot at or after the key's start position, so that keys
      * of one bucket spread over the free slots); an exchange for a victim: whatever key the slot
      * held is the victim and the slot is locked (instead of a load and a compare-and-swap).
-     * LOCKED coming back means somebody else holds the slot (nothing changed); EMPTY is put
-     * back at once. */
+     * LOCKED coming back means somebody else holds the slot (nothing changed); EMPTY means
+     * the slot is free after all and is now this key's. */
     bool refused_now = false;
     bool try_victim = false;
     if (want_scan) {
@@ -823,7 +834,14 @@ upsert_kernel(View v, UpsertArgs a) {
     }
     if (try_victim) {
       const bool mine = vk != v.locked_key && vk != v.empty_key;
-      if (vk == v.empty_key) st_unlock(kp, vk);
+      if (vk == v.empty_key) {
+        /* The slot has become free since the probe (an erase that runs beside this call) and
+         * the exchange has locked it: it is taken like any free slot.  Putting EMPTY back and
+         * searching again would find the same slot, whose old score is still the lowest. */
+        got = kStEmpty;
+        pos = bpos;
+        victim = v.empty_key;
+      }
       if (mine) {
         /* somebody may have raised the score since the search */
         if (ld_u64(v.scores + bslot + bpos) <= best) {
@@ -840,12 +858,7 @@ upsert_kernel(View v, UpsertArgs a) {
     const bool locked = got != kStNone && got != kStRefused;
     const uint64_t slot = bslot + pos;
     uint8_t* row = value_row(v, slot);
-    bool commit = locked;
-    if (OP == kOpAccumOrAssign && locked) {
-      /* accum_or_assign.cuh:139-156: flag and outcome must agree */
-      const bool is_accum = a.accum_flags[i] != 0;
-      commit = is_accum == (got == kStDuplicate);
-    }
+    const bool commit = locked;
 
     /* upsert_and_evict.cuh:188-194, 218-224, 236-245: an evicted key leaves with its old row
      * and the scanned minimum, a refused key with its input.  One counter update per workgroup
@@ -883,12 +896,14 @@ upsert_kernel(View v, UpsertArgs a) {
         st_u64(v.bounds + (slot >> 4), new_bound < bound_cap ? new_bound : bound_cap);
       const uint64_t stored = write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
       /* Scores from the caller may be below what the line's bound says: a key that goes into a
-       * free slot, and under Customized a key that was found (its score becomes the caller's; LFU
-       * and EpochLFU only add to it).  Such a key lowers the bound itself.  A key that takes a
+       * free slot, and a key that was found, under Customized (its score becomes the caller's)
+       * and under EpochLFU (it moves to the epoch of today, which may be an earlier one than its
+       * own; LFU only adds to it).  Such a key lowers the bound itself.  A key that takes a
        * victim's slot cannot be below the victim's score, which the bound was not above, except
        * under LFU, whose line has just been given a bound that no score of this call is below. */
       if (BOUNDS && a.bound_ceil && stored < bound_ceil &&
-          (got == kStEmpty || (got == kStDuplicate && a.strategy == HKV_CUSTOMIZED)))
+          (got == kStEmpty ||
+           (got == kStDuplicate && (a.strategy == HKV_CUSTOMIZED || a.strategy == HKV_EPOCH_LFU))))
         __hip_atomic_fetch_min(v.bounds + (slot >> 4), stored, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (OP == kOpInsertAndEvict && total) {
@@ -955,7 +970,7 @@ struct AssignArgs {
   Clock clock;
   int32_t touch_scores;
   int32_t strategy;
-  /* Customized tables with score bounds in use: the device word no bound is above (as
+  /* Customized and EpochLFU tables with score bounds in use: the device word no bound is above (as
    * UpsertArgs::bound_ceil); a key whose new score is below it lowers its line's bound */
   const unsigned long long* bound_ceil;
 };

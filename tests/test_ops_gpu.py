@@ -1202,3 +1202,47 @@ def test_one_digest_for_a_whole_bucket(oracle):
     o.assign(same, bytes_of(av), as_)
     assert_same_table(t, o, dim * 4)
     t.close()
+
+
+@pytest.mark.parametrize("bounds", ["on", "off"])
+def test_accum_flags_that_disagree_in_nearly_full_buckets(oracle, monkeypatch, bounds):
+    """accum_or_assign with some thirty new keys per bucket and a handful of free slots in each:
+    half of the new keys are flagged "accumulate" and so change nothing, the other half share
+    the free slots and then evict.  A key whose flag disagrees with its presence takes no slot,
+    not even for a moment: a slot that is taken and handed back looks taken to the bucket's other
+    new keys, which then search a victim in a bucket that is not full (and, with the handed-back
+    slot still holding score 0, find that very slot over and over).  With the bounded search
+    and with the full scan, against the oracle."""
+    if bounds == "off":
+        monkeypatch.setenv("HKV_SCORE_BOUNDS", "0")
+    cap, dim = 1 << 12, 4  # 32 buckets
+    t, o, _ = make_pair(oracle, init_capacity=cap, max_capacity=cap, dim=dim)
+    t.set_clock(1, 1 << 44)
+    o.set_clock(1, 1 << 44)
+    vb = dim * 4
+    rng = np.random.default_rng(91)
+    fill(t, o, 91, 3, 1000, dim)  # old keys: the victims
+    pos = 3000
+    for rep in range(4):
+        # the latest keys (highest scores: no eviction of this round reaches them)
+        recent = w.unique_keys(91, pos, 800)
+        rv = w.uniform_values(91, pos, 800, dim)
+        t.insert_or_assign(800, dev(recent), dev(rv))
+        o.insert_or_assign(recent, bytes_of(rv), None)
+        pos += 800
+        if rep:  # free slots again: some of the oldest keys leave
+            gone = w.unique_keys(91, (rep - 1) * 700, 300)
+            t.erase(300, dev(gone))
+            o.erase(gone)
+        assert_same_table(t, o, vb)
+        keys = np.concatenate([recent[:450], w.unique_keys(91, pos, 1050)])
+        pos += 1050
+        keys = keys[rng.permutation(len(keys))]
+        n = len(keys)
+        deltas = w.uniform_values(92 + rep, 0, n, dim)
+        flags = rng.random(n) < 0.5
+        t.accum_or_assign(n, dev(keys), dev(deltas), dev(flags.astype(np.uint8)))
+        o.accum_or_assign(keys, bytes_of(deltas), flags.astype(np.uint8))
+        assert t.size() == o.size()
+        assert_same_table(t, o, vb)
+    t.close()

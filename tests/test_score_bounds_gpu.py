@@ -433,3 +433,72 @@ def test_epoch_lru_bounds(oracle):
     assert bounds_hold(t)[0]
     assert_same_table(t, ot, vb)
     t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kCustomized, EvictStrategy.kLfu, EvictStrategy.kEpochLfu])
+def test_bounds_hold_under_arbitrary_scores(strategy):
+    """No oracle here (with scores that go up and down inside a batch the outcome depends on the order
+    of its keys): random scores from a small range (ties included), hits and new keys mixed, every
+    call that writes scores, epochs that go back and forth.  After every upsert the bounds must not
+    be above any score of their line, no key may be in the table twice, and every key that is found
+    carries the row that was last written for it."""
+    cap, dim = 1 << 12, 4
+    t, o = make(cap, dim, strategy)
+    rng = np.random.default_rng(1234 + int(strategy))
+    universe = w.unique_keys(670, 0, 3 * cap)
+    epoch_lfu = strategy == EvictStrategy.kEpochLfu
+    if epoch_lfu:
+        t.set_global_epoch(5)
+    latest = {}
+    used = 0
+    for step in range(80):
+        n = int(rng.choice([17, 300, 1500]))
+        keys = rng.choice(universe, size=n, replace=False)
+        vals = rng.random((n, dim), dtype=np.float32)
+        sc = rng.integers(1, 1 << int(rng.choice([4, 20, 40])), size=n, dtype=np.uint64)
+        if epoch_lfu and step % 7 == 3:
+            t.set_global_epoch(int(rng.integers(1, 9)))
+        op = rng.choice(["insert_or_assign", "find_or_insert", "insert_and_evict", "accum_or_assign",
+                         "assign", "assign_scores", "erase"], p=[0.35, 0.1, 0.15, 0.1, 0.1, 0.1, 0.1])
+        dk, dv, ds = dev(keys), dev(vals), dev(sc)
+        upsert_call = True
+        if op == "insert_or_assign":
+            t.insert_or_assign(n, dk, dv, ds)
+        elif op == "find_or_insert":
+            t.find_or_insert(n, dk, dv, ds)
+        elif op == "insert_and_evict":
+            ek = torch.zeros(n, dtype=torch.int64, device=DEV)
+            ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+            es = torch.zeros(n, dtype=torch.int64, device=DEV)
+            t.insert_and_evict(n, dk, dv, ds, ek, ev, es)
+        elif op == "accum_or_assign":
+            flags = torch.from_numpy(rng.random(n) < 0.5).to(DEV)
+            t.accum_or_assign(n, dk, dv, flags, ds)
+        elif op == "assign":
+            t.assign(n, dk, dv, ds)
+            upsert_call = False
+        elif op == "assign_scores":
+            t.assign_scores(n, dk, ds)
+            upsert_call = False
+        else:
+            t.erase(n, dk)
+            upsert_call = False
+        used += n if upsert_call else 0
+        if op in ("insert_or_assign", "insert_and_evict", "assign"):
+            for k, v in zip(keys.tolist(), vals):
+                latest[k] = v
+        elif op in ("find_or_insert", "accum_or_assign", "erase"):
+            for k in keys.tolist():
+                latest.pop(k, None)  # (the row depends on whether the key was there: not tracked)
+        if not upsert_call or used < cap:
+            continue  # the bounds are made, and checked here, once upserts use them
+        ok, bad, _ = bounds_hold(t)
+        assert ok, (step, op, bad)
+        from gpu_util import export_table
+        gk, gv, _ = export_table(t, dim * 4)
+        assert len(np.unique(gk)) == len(gk) == t.size(), (step, op)
+        rows = gv.view(np.float32).reshape(len(gk), dim)
+        for k, row in zip(gk.tolist(), rows):
+            if k in latest:
+                assert np.array_equal(row, latest[k]), (step, op, k)
+    t.close()
