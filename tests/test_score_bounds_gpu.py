@@ -435,33 +435,40 @@ def test_epoch_lru_bounds(oracle):
     t.close()
 
 
-@pytest.mark.parametrize("strategy", [EvictStrategy.kCustomized, EvictStrategy.kLfu, EvictStrategy.kEpochLfu])
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kEpochLru, EvictStrategy.kCustomized,
+                                      EvictStrategy.kLfu, EvictStrategy.kEpochLfu])
 def test_bounds_hold_under_arbitrary_scores(strategy):
     """No oracle here (with scores that go up and down inside a batch the outcome depends on the order
-    of its keys): random scores from a small range (ties included), hits and new keys mixed, every
-    call that writes scores, epochs that go back and forth.  After every upsert the bounds must not
-    be above any score of their line, no key may be in the table twice, and every key that is found
-    carries the row that was last written for it."""
+    of its keys): 32 buckets and up to 1500 keys per call, i.e. some 47 keys of a call in every
+    bucket; random scores from a small range (ties included), hits and new keys mixed, every call
+    that writes scores, epochs that go back and forth; LRU and EpochLRU on the hardware clock.
+    After every upsert: no bound is above a score of its line, no key is in the table twice, the
+    table holds nothing but keys it held before and keys of the call, insert_and_evict accounts for
+    every key that left, and every key that is found carries the row that was last written for it."""
+    from gpu_util import export_table, host_u64
     cap, dim = 1 << 12, 4
     t, o = make(cap, dim, strategy)
     rng = np.random.default_rng(1234 + int(strategy))
     universe = w.unique_keys(670, 0, 3 * cap)
-    epoch_lfu = strategy == EvictStrategy.kEpochLfu
-    if epoch_lfu:
+    from_clock = strategy in (EvictStrategy.kLru, EvictStrategy.kEpochLru)
+    epochs = strategy in (EvictStrategy.kEpochLfu, EvictStrategy.kEpochLru)
+    if epochs:
         t.set_global_epoch(5)
     latest = {}
     used = 0
+    resident = set()
     for step in range(80):
         n = int(rng.choice([17, 300, 1500]))
         keys = rng.choice(universe, size=n, replace=False)
         vals = rng.random((n, dim), dtype=np.float32)
         sc = rng.integers(1, 1 << int(rng.choice([4, 20, 40])), size=n, dtype=np.uint64)
-        if epoch_lfu and step % 7 == 3:
+        if epochs and step % 7 == 3:
             t.set_global_epoch(int(rng.integers(1, 9)))
         op = rng.choice(["insert_or_assign", "find_or_insert", "insert_and_evict", "accum_or_assign",
                          "assign", "assign_scores", "erase"], p=[0.35, 0.1, 0.15, 0.1, 0.1, 0.1, 0.1])
-        dk, dv, ds = dev(keys), dev(vals), dev(sc)
+        dk, dv, ds = dev(keys), dev(vals), (None if from_clock else dev(sc))
         upsert_call = True
+        evicted = None
         if op == "insert_or_assign":
             t.insert_or_assign(n, dk, dv, ds)
         elif op == "find_or_insert":
@@ -470,7 +477,8 @@ def test_bounds_hold_under_arbitrary_scores(strategy):
             ek = torch.zeros(n, dtype=torch.int64, device=DEV)
             ev = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
             es = torch.zeros(n, dtype=torch.int64, device=DEV)
-            t.insert_and_evict(n, dk, dv, ds, ek, ev, es)
+            cnt = t.insert_and_evict(n, dk, dv, ds, ek, ev, es)
+            evicted = host_u64(ek[:cnt]).tolist()
         elif op == "accum_or_assign":
             flags = torch.from_numpy(rng.random(n) < 0.5).to(DEV)
             t.accum_or_assign(n, dk, dv, flags, ds)
@@ -490,15 +498,34 @@ def test_bounds_hold_under_arbitrary_scores(strategy):
         elif op in ("find_or_insert", "accum_or_assign", "erase"):
             for k in keys.tolist():
                 latest.pop(k, None)  # (the row depends on whether the key was there: not tracked)
-        if not upsert_call or used < cap:
-            continue  # the bounds are made, and checked here, once upserts use them
-        ok, bad, _ = bounds_hold(t)
-        assert ok, (step, op, bad)
-        from gpu_util import export_table
         gk, gv, _ = export_table(t, dim * 4)
-        assert len(np.unique(gk)) == len(gk) == t.size(), (step, op)
+        now = set(gk.tolist())
+        batch = set(keys.tolist())
+        assert len(now) == len(gk) == t.size() <= cap, (step, op)
+        if op == "erase":
+            assert now == resident - batch, (step, op)
+        elif not upsert_call:
+            assert now == resident, (step, op)
+        else:
+            assert now <= resident | batch, (step, op)
+            if op == "accum_or_assign":
+                pass  # which of its keys come in depends on their flags
+            elif strategy == EvictStrategy.kLru:
+                assert batch <= now, (step, op)  # the scores of the call are the highest: none is refused or evicted
+        if evicted is not None:
+            # Keys of other calls: the ones that left are exactly the ones handed back, once each.
+            # Keys of this call (one may be evicted by another and come in again, or be refused):
+            # one that is not there afterwards has been handed back.
+            left = [k for k in evicted if k not in batch]
+            assert len(set(left)) == len(left) and set(left) <= resident, (step, op)
+            assert now - batch == (resident - batch) - set(left), (step, op)
+            assert batch - now <= set(evicted), (step, op)
+        resident = now
         rows = gv.view(np.float32).reshape(len(gk), dim)
         for k, row in zip(gk.tolist(), rows):
             if k in latest:
                 assert np.array_equal(row, latest[k]), (step, op, k)
+        if upsert_call and used >= cap:  # the bounds are made, and checked here, once upserts use them
+            ok, bad, _ = bounds_hold(t)
+            assert ok, (step, op, bad)
     t.close()
