@@ -78,11 +78,16 @@ erase_kernel(View v, const uint64_t* keys, uint64_t n) {
       uint64_t seen = key;
       erased = cas_lock(v.keys + slot, seen, v.locked_key);
     }
-    if (erased) {
-      v.digests[slot] = v.empty_digest;
-      /* without the group lock an inserter may be looking: the key word opens last */
-      if (!EXCLUSIVE) st_u64(v.keys + slot, v.empty_key);
-    }
+    if (EXCLUSIVE && erased) v.digests[slot] = v.empty_digest;
+  }
+  if (!EXCLUSIVE) {
+    /* Without the group lock an inserter of another launch may be looking: the digest goes out
+     * as a store that every compute die sees, it is complete before the key word opens, and
+     * the key word opens last.  (A digest store that came later than the key word would land
+     * on the digest of the key that took the slot in between.) */
+    if (erased) st_u8(v.digests + slot, (uint8_t)v.empty_digest);
+    wait_stores();
+    if (erased) st_u64(v.keys + slot, v.empty_key);
   }
 }
 

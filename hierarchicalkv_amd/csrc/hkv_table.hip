@@ -1164,8 +1164,10 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   t->io_stage_bytes = 0;
   {
     const char* b = getenv("HKV_SCORE_BOUNDS");
-    /* dual-bucket tables have their own kernel, which scans both buckets */
-    t->score_bounds = !(b && !strcmp(b, "0")) && !t->dual;
+    /* dual-bucket tables have their own kernel, which scans both buckets; without the group
+     * lock two upserts may run at once on two streams, and the limits of the bounds (the clock
+     * reading or lowest score of "the call that is running") are kept per table, not per call */
+    t->score_bounds = !(b && !strcmp(b, "0")) && !t->dual && o->api_lock != 0;
   }
   memset(&t->view, 0, sizeof t->view);
   t->epoch = kIgnoredEpoch;

@@ -220,3 +220,73 @@ def test_two_bucket_mode():
     run_calls(t, strategy, dim, 770, 40, w.unique_keys(771, 0, 3 * cap), [17, 300, 1500],
               ["insert_or_assign", "find"], [0.8, 0.2])
     t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kCustomized])
+def test_streams_without_the_group_lock(strategy):
+    """api_lock = false: calls on different streams run at the same time, kept apart by the
+    slot locks alone.  The caller keeps the key sets of calls that may overlap apart (two calls
+    that bring the same new key at the same moment each give it a slot, in the reference as
+    here): four streams, each with keys of its own, all on one table of 32 buckets, so that
+    the calls take each other's victims, free slots (erase runs beside the upserts) and locks.
+    After every round: no key twice, size() = keys exported, and every key carries, whole, the
+    row its stream wrote for it last (or, after a find_or_insert, the one before)."""
+    cap, dim = 1 << 12, 8
+    t = table(strategy, dim, cap, api_lock=0)
+    rng = np.random.default_rng(780 + int(strategy))
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    universes = [w.unique_keys(781 + s, 0, 6 * cap) for s in range(4)]
+    assert len(np.unique(np.concatenate(universes))) == 24 * cap
+    from_clock = strategy == EvictStrategy.kLru
+    rows_of = {}
+    version = 0
+    for rnd in range(10):
+        # all inputs of the round first, then its twenty calls back to back, so that they overlap
+        calls = []
+        for call in range(5):
+            for s, st in enumerate(streams):
+                n = int(rng.choice([1500, 6000, 20000]))
+                op = str(rng.choice(["insert_or_assign", "find_or_insert", "assign", "erase", "find"],
+                                    p=[0.45, 0.15, 0.1, 0.15, 0.15]))
+                keys = rng.choice(universes[s], size=n, replace=False)
+                version += 1
+                vals = np.full((n, dim), version, np.float32)
+                sc = rng.integers(1, 1 << 20, size=n, dtype=np.uint64)
+                out = torch.zeros(n, dim, dtype=torch.float32, device=DEV)
+                founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+                calls.append((op, st, n, keys, version, dev(keys), dev(vals), None if from_clock else dev(sc),
+                              out, founds))
+        torch.cuda.synchronize()
+        for op, st, n, keys, ver, dk, dv, ds, out, founds in calls:
+            if op == "insert_or_assign":
+                t.insert_or_assign(n, dk, dv, ds, stream=st)
+            elif op == "find_or_insert":
+                t.find_or_insert(n, dk, dv, ds, stream=st)
+            elif op == "assign":
+                t.assign(n, dk, dv, ds, stream=st)
+            elif op == "erase":
+                t.erase(n, dk, stream=st)
+            else:
+                t.find(n, dk, out, founds, stream=st)
+        for op, st, n, keys, ver, *_ in calls:  # (the calls of one stream run in this order)
+            if op == "insert_or_assign":
+                for k in keys.tolist():
+                    rows_of[k] = [ver]
+            elif op == "find_or_insert":
+                for k in keys.tolist():
+                    rows_of[k] = rows_of.get(k, []) + [ver]
+            elif op == "assign":
+                for k in keys.tolist():
+                    if k in rows_of:  # (a key that is absent stays so; one that is there has been written)
+                        rows_of[k] = [ver]
+            elif op == "erase":
+                for k in keys.tolist():
+                    rows_of.pop(k, None)
+        torch.cuda.synchronize()
+        gk, gv, _ = export_table(t, dim * 4)
+        assert len(set(gk.tolist())) == len(gk) == t.size() <= cap, rnd
+        rows = gv.view(np.float32).reshape(len(gk), dim)
+        assert (rows == rows[:, :1]).all(), rnd  # one call's row, not a mixture
+        for k, row in zip(gk.tolist(), rows):
+            assert k in rows_of and int(row[0]) in rows_of[k], (rnd, k, row[0], rows_of.get(k))
+    t.close()
