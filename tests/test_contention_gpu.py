@@ -222,17 +222,20 @@ def test_two_bucket_mode():
     t.close()
 
 
+@pytest.mark.parametrize("api_lock", [0, 1])
 @pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kCustomized])
-def test_streams_without_the_group_lock(strategy):
+def test_four_streams_at_once(strategy, api_lock):
     """api_lock = false: calls on different streams run at the same time, kept apart by the
     slot locks alone.  The caller keeps the key sets of calls that may overlap apart (two calls
     that bring the same new key at the same moment each give it a slot, in the reference as
     here): four streams, each with keys of its own, all on one table of 32 buckets, so that
     the calls take each other's victims, free slots (erase runs beside the upserts) and locks.
     After every round: no key twice, size() = keys exported, and every key carries, whole, the
-    row its stream wrote for it last (or, after a find_or_insert, the one before)."""
+    row its stream wrote for it last (or, after a find_or_insert, the one before).
+    api_lock = true: the same calls, ordered by their roles between the streams (events; an
+    upsert runs alone and searches through the score bounds)."""
     cap, dim = 1 << 12, 8
-    t = table(strategy, dim, cap, api_lock=0)
+    t = table(strategy, dim, cap, api_lock=api_lock)
     rng = np.random.default_rng(780 + int(strategy))
     streams = [torch.cuda.Stream() for _ in range(4)]
     universes = [w.unique_keys(781 + s, 0, 6 * cap) for s in range(4)]
