@@ -30,7 +30,8 @@ UPSERTS = ["insert_or_assign", "find_or_insert", "insert_and_evict", "accum_or_a
 OTHERS = ["assign", "assign_scores", "erase", "find"]
 
 
-def run_calls(t, strategy, dim, seed, steps, universe, sizes, ops, probs, repeat_keys=False, grows=False):
+def run_calls(t, strategy, dim, seed, steps, universe, sizes, ops, probs, repeat_keys=False, grows=False,
+              hidden=0):
     rng = np.random.default_rng(seed)
     from_clock = strategy in (EvictStrategy.kLru, EvictStrategy.kEpochLru)
     vb = dim * 4
@@ -83,7 +84,8 @@ def run_calls(t, strategy, dim, seed, steps, universe, sizes, ops, probs, repeat
         gk, gv, _ = export_table(t, vb)
         now = set(gk.tolist())
         batch = set(keys.tolist())
-        assert len(now) == len(gk) == t.size() <= t.capacity(), where
+        # (`hidden`: slots held by lock_keys, which no export shows but size() counts)
+        assert len(now) == len(gk) == t.size() - hidden <= t.capacity() - hidden, where
         if op == "erase":
             assert now == resident - batch, where
         elif op not in UPSERTS:
@@ -292,4 +294,38 @@ def test_four_streams_at_once(strategy, api_lock):
         assert (rows == rows[:, :1]).all(), rnd  # one call's row, not a mixture
         for k, row in zip(gk.tolist(), rows):
             assert k in rows_of and int(row[0]) in rows_of[k], (rnd, k, row[0], rows_of.get(k))
+    t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kCustomized])
+def test_slots_held_by_lock_keys_survive(strategy):
+    """A quarter of every bucket is held by lock_keys while calls of 1500 other keys fill the
+    table and evict: the victim search reads the key words beside the scores and passes the held
+    slots over, so after unlock_keys every held key is there with its row, whatever its score."""
+    cap, dim = 1 << 12, 4
+    t = table(strategy, dim, cap)
+    rng = np.random.default_rng(790 + int(strategy))
+    from_clock = strategy == EvictStrategy.kLru
+    held = w.unique_keys(791, 0, 1000)
+    hv = rng.random((1000, dim), dtype=np.float32)
+    ones = np.ones(1000, np.uint64)  # the lowest scores of the table: first in line for eviction
+    t.insert_or_assign(1000, dev(held), dev(hv), None if from_clock else dev(ones))
+    ptrs = torch.zeros(1000, dtype=torch.int64, device=DEV)
+    ok = torch.zeros(1000, dtype=torch.bool, device=DEV)
+    t.lock_keys(1000, dev(held), ptrs, ok, scores=None if from_clock else dev(ones))
+    assert bool(ok.all())
+    others = w.unique_keys(792, 0, 4 * cap)
+    run_calls(t, strategy, dim, 793 + int(strategy), 25, others, [300, 1500],
+              ["insert_or_assign", "find_or_insert", "insert_and_evict", "accum_or_assign", "erase"],
+              [0.4, 0.15, 0.2, 0.1, 0.15], hidden=len(held))
+    ok2 = torch.zeros(1000, dtype=torch.bool, device=DEV)
+    t.unlock_keys(1000, ptrs, dev(held), ok2)
+    assert bool(ok2.all())
+    out = torch.zeros(1000, dim, dtype=torch.float32, device=DEV)
+    founds = torch.zeros(1000, dtype=torch.bool, device=DEV)
+    t.find(1000, dev(held), out, founds)
+    torch.cuda.synchronize()
+    assert bool(founds.all()) and np.array_equal(out.cpu().numpy(), hv)
+    gk, _, _ = export_table(t, dim * 4)
+    assert len(set(gk.tolist())) == len(gk) == t.size() <= cap
     t.close()
