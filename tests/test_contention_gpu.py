@@ -329,3 +329,40 @@ def test_slots_held_by_lock_keys_survive(strategy):
     gk, _, _ = export_table(t, dim * 4)
     assert len(set(gk.tolist())) == len(gk) == t.size() <= cap
     t.close()
+
+
+@pytest.mark.parametrize("strategy", [EvictStrategy.kLru, EvictStrategy.kCustomized])
+def test_pointer_overload_that_keeps_its_slots(strategy):
+    """find_or_insert by pointer with locked_key_ptrs: every key the call settles keeps its slot
+    LOCKED until unlock_keys, so the 47 keys that meet in a bucket see more and more slots that
+    are neither theirs nor anybody's victim.  After unlock_keys: no key twice, the pointers of
+    the keys that got in are pairwise different and those keys are found, and under LRU (whose
+    new scores are the highest) every key got in."""
+    cap, dim = 1 << 12, 4
+    t = table(strategy, dim, cap)
+    rng = np.random.default_rng(795 + int(strategy))
+    from_clock = strategy == EvictStrategy.kLru
+    universe = w.unique_keys(796, 0, 3 * cap)
+    run_calls(t, strategy, dim, 797, 8, universe, [1500], ["insert_or_assign"], [1.0])  # full by now
+    for rnd in range(6):
+        n = 1500
+        keys = rng.choice(universe, size=n, replace=False)
+        sc = rng.integers(1, 1 << 20, size=n, dtype=np.uint64)
+        ptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+        founds = torch.zeros(n, dtype=torch.bool, device=DEV)
+        kptrs = torch.zeros(n, dtype=torch.int64, device=DEV)
+        t.find_or_insert_ptr(n, dev(keys), ptrs, founds, None if from_clock else dev(sc), locked_key_ptrs=kptrs)
+        ok = torch.zeros(n, dtype=torch.bool, device=DEV)
+        t.unlock_keys(n, kptrs, dev(keys), ok)
+        torch.cuda.synchronize()
+        p = ptrs.cpu().numpy()
+        got_in = p != 0
+        assert np.array_equal(ok.cpu().numpy(), got_in), rnd
+        assert len(np.unique(p[got_in])) == got_in.sum(), rnd
+        if from_clock:
+            assert got_in.all(), rnd
+        gk, _, _ = export_table(t, dim * 4)
+        now = set(gk.tolist())
+        assert len(now) == len(gk) == t.size() <= cap, rnd
+        assert set(keys[got_in].tolist()) <= now and not (set(keys[~got_in].tolist()) & now), rnd
+    t.close()
