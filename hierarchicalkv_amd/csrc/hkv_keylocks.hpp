@@ -106,7 +106,7 @@ unlock_keys_kernel(View v, uint64_t n, uint64_t* const* key_ptrs, const uint64_t
     ok = true;
   }
   const unsigned long long freed = __ballot(ok);
-  if (freed && (threadIdx.x & (kWave - 1)) == (int)__ffsll(freed) - 1)
+  if (locked_count && freed && (threadIdx.x & (kWave - 1)) == (int)__ffsll(freed) - 1)
     atomicAdd(locked_count, 0ull - (unsigned long long)__popcll(freed)) /* wraps: a subtraction */;
   if (i < n && success) success[i] = ok;
 }

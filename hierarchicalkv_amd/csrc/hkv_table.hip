@@ -815,7 +815,33 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
     if (OP == kOpFindOrInsertPtr && a.locked_key_ptrs) t->keys_may_be_locked = true;
     /* a table that has been offered fewer keys than nine tenths of its slots evicts next to nothing */
     const bool pair = OP == kOpInsertAndEvict && t->keys_offered * 10 >= t->view.capacity * 9;
-    if (t->keys_may_be_locked) {
+    /* Hybrid mode: the reference settles the keys of a batch with one kernel that leaves every
+     * slot it took LOCKED and moves the rows with a second one that unlocks them
+     * (upsert.cuh:1350-1595, find_or_insert.cuh:1417-1676), so no key of a batch ever takes the
+     * slot of another key of the same batch: the later key sees that slot as LOCKED, which the
+     * victim scan of these kernels passes over.  Here the rows move under the same lock; the
+     * slots stay LOCKED until the kernel is done and a second launch opens them.  (A call that
+     * is being recorded into a graph cannot ask for the list of slots: it releases each slot as
+     * soon as its key is in, which is the same as handing the keys over one call at a time.) */
+    const bool hold = hybrid_rule && !t->pure_hbm && !capturing(s) &&
+                      (OP == kOpInsertOrAssign || OP == kOpFindOrInsert);
+    if (hold) {
+      uint64_t** held = nullptr;
+      HKV_HIP(hipMallocAsync((void**)&held, a.n * sizeof(uint64_t*), s));
+      hipError_t e = hipMemsetAsync(held, 0, a.n * sizeof(uint64_t*), s);
+      if (e == hipSuccess) {
+        a.locked_key_ptrs = held;
+        a.locked_count = nullptr; /* nothing stays LOCKED beyond this call */
+        writes_scores_outside_bounds(t, s, own_rule);
+        launch_upsert_for<OP, true>(pair, vec, t->view, a, s);
+        hipLaunchKernelGGL(unlock_keys_kernel, dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, s, t->view,
+                           a.n, (uint64_t* const*)held, a.keys, (uint8_t*)nullptr,
+                           (unsigned long long*)nullptr);
+        e = hipGetLastError();
+      }
+      (void)hipFreeAsync(held, s);
+      HKV_HIP(e);
+    } else if (t->keys_may_be_locked) {
       /* slots that lock_keys (or the pointer overload with locked_key_ptrs) left LOCKED must
        * be hidden from the victim scan, which then reads the key words beside the scores; with
        * no such slot the plain scan finds the same victims (a slot locked by another key of

@@ -889,6 +889,9 @@ upsert_kernel(View v, UpsertArgs a) {
       a.founds[i] = got == kStDuplicate;
       if (a.locked_key_ptrs) a.locked_key_ptrs[i] = locked ? v.keys + slot : nullptr;
     }
+    /* hybrid mode: the slots of a batch stay LOCKED until all its keys are settled; the list
+     * starts out as all null */
+    if (OP != kOpFindOrInsertPtr && LOCKED_RULE && a.locked_key_ptrs && locked) a.locked_key_ptrs[i] = v.keys + slot;
     if (commit) {
       /* a victim's slot gets a score of this call: what bounds its line now is the lowest of
        * the line's other scores */
@@ -942,12 +945,17 @@ upsert_kernel(View v, UpsertArgs a) {
 
     /* ---- step 5: everything written under the locks is out; release them --------------------------- */
     wait_stores();
-    /* the pointer overload may be asked to leave its slots locked for unlock_keys */
-    const bool keep_locked = OP == kOpFindOrInsertPtr && a.locked_key_ptrs != nullptr;
+    /* the pointer overload may be asked to leave its slots locked for unlock_keys; the upserts
+     * of hybrid mode leave theirs locked until the launch is over */
+    const bool keep_locked = (OP == kOpFindOrInsertPtr || LOCKED_RULE) && a.locked_key_ptrs != nullptr;
     if (locked && !keep_locked) st_unlock(v.keys + slot, commit ? key : victim);
     if (keep_locked) {
       const unsigned long long kept = __ballot(locked);
-      if (kept && lane == (int)__ffsll(kept) - 1) atomicAdd(a.locked_count, (unsigned long long)__popcll(kept));
+      /* (no count where the launch that follows opens the slots again: one word takes one update
+       * at a time, and a wavefront's worth of them per trip is a quarter of a millisecond per
+       * 2^20 keys) */
+      if (a.locked_count && kept && lane == (int)__ffsll(kept) - 1)
+        atomicAdd(a.locked_count, (unsigned long long)__popcll(kept));
     }
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);

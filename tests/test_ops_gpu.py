@@ -338,17 +338,21 @@ def test_hybrid_mode(oracle):
     t.close()
 
 
-def test_hybrid_batch_is_some_serial_order(oracle):
-    """Where hybrid mode differs from the reference.  The reference's hybrid upsert holds every
-    slot lock of a batch from its lock kernel to its write kernel (upsert.cuh:1350-1595), so an
-    absent key never takes the slot of another key of its own batch: each takes the lowest-scored
-    resident that is still visible.  The fused kernel here releases a slot as soon as its key is
-    in, so a later key of the batch may evict an earlier one, exactly as if the keys had been
-    handed over one call at a time.  On a one-bucket table with a batch whose scores interleave
-    with the lowest resident scores: the GPU's result must be what the oracle gives for some
-    order of one-key calls (all 120 orders are tried), and it is not what the reference's batch
-    model gives (there the key with score 105 stays, because its slot is invisible to the scans
-    of the later keys of the batch; one key at a time it always loses the slot again)."""
+def test_hybrid_batch_holds_its_locks(oracle):
+    """The reference's hybrid upsert holds every slot lock of a batch from its lock kernel to its
+    write kernel (upsert.cuh:1350-1595), so an absent key never takes the slot of another key of
+    its own batch: each takes the lowest-scored resident that is still visible, or is refused
+    when its score is not above that.  On a one-bucket table with a batch whose scores interleave
+    with the lowest resident scores the outcome depends on which key of the batch comes first, in
+    the reference as here, but not in the way it would if the keys were handed over one call at
+    a time (then the key with score 105 always loses its slot again to a later key; under the
+    batch's locks it keeps it whenever it got one).  The GPU's result must be what the oracle's
+    batch model gives for some order of the batch (all 120 are tried).  Then a batch that tells
+    the two apart: 64 keys whose scores all lie between the lowest and the second lowest
+    resident.  One key at a time the highest of them always ends up as the only survivor (each
+    key evicts the lower one before it); under the batch's locks the survivor is whichever key
+    locked the lowest resident first, and the 63 others, which see nothing below 2000, are
+    refused."""
     import itertools
     dim = 4
     opts = default_options(init_capacity=128, max_capacity=128, dim=dim, max_hbm_for_vectors=0,
@@ -364,7 +368,7 @@ def test_hybrid_batch_is_some_serial_order(oracle):
         ek, _, es = table.export_all()
         return frozenset(zip(ek.tolist(), es.tolist()))
 
-    serial = set()
+    serial, batched = set(), set()
     for order in itertools.permutations(range(5)):
         o = oracle.OracleTable(opts, hybrid=True)
         o.insert_or_assign(keys, bytes_of(vals), sc)
@@ -372,24 +376,56 @@ def test_hybrid_batch_is_some_serial_order(oracle):
             o.insert_or_assign(batch[i:i + 1], bytes_of(bvals[i:i + 1]), bsc[i:i + 1])
         serial.add(resident_map(o))
         o.close()
-    ref = oracle.OracleTable(opts, hybrid=True)
-    ref.insert_or_assign(keys, bytes_of(vals), sc)
-    ref.insert_or_assign(batch, bytes_of(bvals), bsc)
-    batch_model = resident_map(ref)
-    ref.close()
-    assert batch_model not in serial
+        o = oracle.OracleTable(opts, hybrid=True)
+        o.insert_or_assign(keys, bytes_of(vals), sc)
+        p = list(order)
+        o.insert_or_assign(batch[p], bytes_of(bvals[p]), bsc[p])
+        batched.add(resident_map(o))
+        o.close()
+    assert len(batched) > len(serial) == 1
 
-    t = HashTable()
-    t.init(opts)
-    assert not t.is_pure_hbm()
-    t.insert_or_assign(128, dev(keys), dev(vals), dev(sc))
-    t.insert_or_assign(5, dev(batch), dev(bvals), dev(bsc))
-    gk, gv, gs = export_table(t, dim * 4)
-    assert frozenset(zip(gk.tolist(), gs.tolist())) in serial
-    allv = {int(k): v for k, v in zip(np.concatenate([keys, batch]), np.concatenate([bytes_of(vals), bytes_of(bvals)]))}
-    assert all((gv[i] == allv[int(k)]).all() for i, k in enumerate(gk))  # every resident carries its own row
-    assert t.size() == 128
-    t.close()
+    for rep in range(5):
+        t = HashTable()
+        t.init(opts)
+        assert not t.is_pure_hbm()
+        t.insert_or_assign(128, dev(keys), dev(vals), dev(sc))
+        t.insert_or_assign(5, dev(batch), dev(bvals), dev(bsc))
+        gk, gv, gs = export_table(t, dim * 4)
+        assert frozenset(zip(gk.tolist(), gs.tolist())) in batched
+        allv = {int(k): v for k, v in zip(np.concatenate([keys, batch]), np.concatenate([bytes_of(vals), bytes_of(bvals)]))}
+        assert all((gv[i] == allv[int(k)]).all() for i, k in enumerate(gk))  # every resident carries its own row
+        assert t.size() == 128
+        # find_or_insert follows the same kernels (find_or_insert.cuh:1417-1676)
+        io = dev(bvals.copy())
+        t.find_or_insert(5, dev(batch), io, dev(bsc))
+        torch.cuda.synchronize()
+        assert t.size() == 128
+        t.close()
+
+    sc = np.arange(1000, 1000 * 129, 1000, dtype=np.uint64)
+    crowd = w.unique_keys(313, 0, 64)
+    cvals = w.values_from_keys(crowd, dim)
+    survivors = []
+    for top_at in (0, 63, 31, 62):  # where the highest score of the batch sits
+        csc = np.arange(1001, 1065, dtype=np.uint64)
+        csc[[top_at, 63]] = csc[[63, top_at]]
+        for call in ("insert_or_assign", "find_or_insert"):
+            t = HashTable()
+            t.init(opts)
+            t.insert_or_assign(128, dev(keys), dev(vals), dev(sc))
+            if call == "insert_or_assign":
+                t.insert_or_assign(64, dev(crowd), dev(cvals), dev(csc))
+            else:
+                t.find_or_insert(64, dev(crowd), dev(cvals.copy()), dev(csc))
+            gk, gv, gs = export_table(t, dim * 4)
+            mine = np.isin(gk, crowd)
+            assert mine.sum() == 1 and t.size() == 128 and keys[0] not in gk
+            who = int(np.flatnonzero(crowd == gk[mine][0])[0])
+            assert gs[mine][0] == csc[who] and (gv[mine][0] == bytes_of(cvals)[who]).all()
+            survivors.append(csc[who] == 1064)
+            t.close()
+    assert not all(survivors)  # one key at a time it would be the highest score every time
+
 
 
 def test_io_by_cpu(oracle):
