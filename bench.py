@@ -741,7 +741,8 @@ CONFIG_PROFILES = [
      [("upsert_kernel<1, 16, 2, false", "insert_and_evict", "last3"), ("lookup_kernel<0, 16", "find on the same keys", "last3")]),
     ("cfg4", "python3 bench.py --config 4", "configuration 4 (capacity 2^28, dim 64, 16 GiB of rows in HBM + 48 GiB pinned, LFU)",
      [("lookup_kernel<0, 16", "find (about 80 % hit)", "last3"), ("lookup_kernel<1, 16", "find*", "mid3"),
-      ("upsert_kernel<0, 16, 2, false", "insert_or_assign (about 20 % new)", "last3")]),
+      ("upsert_kernel<0, 16, 2, false", "insert_or_assign (about 20 % new): the kernel that settles the keys, moves the rows and leaves the slots locked", "last3"),
+      ("open_held_kernel", "insert_or_assign: the launch that opens the slots", "last3")]),
     ("cfg5", "python3 bench.py --config 5", "configuration 5 (capacity 2^25, dim 128, EpochLRU, load factor 1.0)",
      [("upsert_kernel<3, 16, 4, false", "accum_or_assign (70 % existing)", "last3"),
       ("export_if_kernel", "export_batch_if over the whole table (8 windows)", "sum8"),

@@ -111,5 +111,20 @@ unlock_keys_kernel(View v, uint64_t n, uint64_t* const* key_ptrs, const uint64_t
   if (i < n && success) success[i] = ok;
 }
 
+/* The second launch of an upsert in hybrid mode: every slot the first one left LOCKED gets its
+ * score (it showed kMaxScore meanwhile, so that no key of the batch took it for a victim) and then
+ * its key.  The caller has the table to itself. */
+__global__ void __launch_bounds__(256)
+open_held_kernel(View v, uint64_t n, uint64_t* const* key_ptrs, const uint64_t* scores, const uint64_t* keys) {
+  const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  uint64_t* p = i < n ? key_ptrs[i] : nullptr;
+  if (p != nullptr) {
+    const uint64_t s = scores[i];
+    if (s != kMaxScore) st_u64(v.scores + (p - v.keys), s);
+  }
+  wait_stores();
+  if (p != nullptr) st_u64(p, keys[i]);
+}
+
 }  // namespace hkv
 #endif

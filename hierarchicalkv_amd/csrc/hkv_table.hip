@@ -825,23 +825,20 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
      * soon as its key is in, which is the same as handing the keys over one call at a time.) */
     const bool hold = hybrid_rule && !t->pure_hbm && !capturing(s) &&
                       (OP == kOpInsertOrAssign || OP == kOpFindOrInsert);
+    uint64_t** held = nullptr;
     if (hold) {
-      uint64_t** held = nullptr;
-      HKV_HIP(hipMallocAsync((void**)&held, a.n * sizeof(uint64_t*), s));
-      hipError_t e = hipMemsetAsync(held, 0, a.n * sizeof(uint64_t*), s);
-      if (e == hipSuccess) {
-        a.locked_key_ptrs = held;
-        a.locked_count = nullptr; /* nothing stays LOCKED beyond this call */
-        writes_scores_outside_bounds(t, s, own_rule);
-        launch_upsert_for<OP, true>(pair, vec, t->view, a, s);
-        hipLaunchKernelGGL(unlock_keys_kernel, dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, s, t->view,
-                           a.n, (uint64_t* const*)held, a.keys, (uint8_t*)nullptr,
-                           (unsigned long long*)nullptr);
-        e = hipGetLastError();
+      /* n slot addresses, then n scores */
+      HKV_HIP(hipMallocAsync((void**)&held, a.n * 16, s));
+      const hipError_t e = hipMemsetAsync(held, 0, a.n * 8, s);
+      if (e != hipSuccess) {
+        (void)hipFreeAsync(held, s);
+        HKV_HIP(e);
       }
-      (void)hipFreeAsync(held, s);
-      HKV_HIP(e);
-    } else if (t->keys_may_be_locked) {
+      a.locked_key_ptrs = held;
+      a.held_scores = reinterpret_cast<uint64_t*>(held) + a.n;
+      a.locked_count = nullptr; /* nothing stays LOCKED beyond this call */
+    }
+    if (t->keys_may_be_locked) {
       /* slots that lock_keys (or the pointer overload with locked_key_ptrs) left LOCKED must
        * be hidden from the victim scan, which then reads the key words beside the scores; with
        * no such slot the plain scan finds the same victims (a slot locked by another key of
@@ -854,7 +851,16 @@ int run_upsert(hkv_table* t, UpsertArgs a, int vec, bool hybrid_rule, hipStream_
       writes_scores_outside_bounds(t, s, own_rule);
       launch_upsert_for<OP, false>(pair, vec, t->view, a, s);
     }
-    HKV_HIP(hipGetLastError());
+    hipError_t e = hipGetLastError();
+    if (hold) {
+      if (e == hipSuccess) {
+        hipLaunchKernelGGL(open_held_kernel, dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, s, t->view, a.n,
+                           (uint64_t* const*)held, a.held_scores, a.keys);
+        e = hipGetLastError();
+      }
+      (void)hipFreeAsync(held, s);
+    }
+    HKV_HIP(e);
   }
   if (t->clock.mode == 1) t->clock.base += UINT64_C(1) << 40;
   return HKV_SUCCESS;

@@ -61,6 +61,9 @@ struct UpsertArgs {
                                  addresses go here (find_ptr_or_insert.cuh:232-242) */
   uint8_t* founds;
   unsigned long long* locked_count;   /* with locked_key_ptrs: the table's count of slots left LOCKED */
+  uint64_t* held_scores;              /* the upserts of hybrid mode (the other overloads with locked_key_ptrs):
+                                         the score of every slot that is left LOCKED; the slot itself
+                                         shows kMaxScore until the launch that opens it */
   uint64_t n;
   uint64_t epoch;
   Clock clock;
@@ -104,7 +107,7 @@ __device__ __forceinline__ uint64_t desired_when_missed(const UpsertArgs& a,
 __device__ __forceinline__ uint64_t write_meta(const View& v, const UpsertArgs& a,
                                                uint64_t slot, uint32_t digest,
                                                uint64_t desired, uint64_t in_score,
-                                               uint64_t i, bool new_insert) {
+                                               uint64_t i, bool new_insert, bool hold = false) {
   const int STRATEGY = a.strategy;
   uint64_t s = desired;
   if (STRATEGY == HKV_LRU) {
@@ -124,8 +127,10 @@ __device__ __forceinline__ uint64_t write_meta(const View& v, const UpsertArgs& 
   /* a hit keeps its digest: the byte is only written when the slot changes
    * owner (the reference rewrites the same value, kernel_utils.cuh:296-300) */
   if (new_insert) st_u8(v.digests + slot, (uint8_t)digest);
-  st_u64(v.scores + slot, s);
-  return s; /* what the slot holds now (kMaxScore above: nothing was written) */
+  /* `hold`: the slot stays LOCKED to the end of the launch and must not look like a victim to
+   * the searches that read scores only; the caller keeps `s` for the launch that opens it */
+  st_u64(v.scores + slot, hold ? kMaxScore : s);
+  return s; /* what the slot holds in the end (kMaxScore above: nothing was written) */
 }
 
 /* wrapping adds of the 8- and 16-bit lanes of a word (signed and unsigned alike) */
@@ -666,6 +671,15 @@ upsert_kernel(View v, UpsertArgs a) {
    * that every one arrives at the workgroup's barriers */
   bool more = pend_mask != 0;
   if constexpr (WAVES > 1) more = __syncthreads_or(more);
+  /* hybrid mode, insert_or_assign and find_or_insert: the slots of a batch stay LOCKED to the end
+   * of the launch (the calls without a hybrid form never see the list) */
+  constexpr bool kCanHold = OP == kOpInsertOrAssign || OP == kOpFindOrInsert;
+  const bool hold = kCanHold && a.locked_key_ptrs != nullptr;
+  /* Where every slot that is taken stays LOCKED to the end of the launch, a LOCKED word is never
+   * this key's slot about to be given back: it is another key of the batch, or this key on its
+   * way out.  The second probe does not wait for it.  (With the waits, a key whose digest
+   * matched a held slot kept its wavefront alive for 64 rounds: 0.15 ms per 2^20 keys.) */
+  if ((OP == kOpFindOrInsertPtr || kCanHold) && a.locked_key_ptrs != nullptr) waited = kMaxLockedWaits;
   for (int trip = 0; more; trip++) {
     if (__ballot(pending && reprobe))
       settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, waited, lane);
@@ -889,15 +903,18 @@ upsert_kernel(View v, UpsertArgs a) {
       a.founds[i] = got == kStDuplicate;
       if (a.locked_key_ptrs) a.locked_key_ptrs[i] = locked ? v.keys + slot : nullptr;
     }
-    /* hybrid mode: the slots of a batch stay LOCKED until all its keys are settled; the list
-     * starts out as all null */
-    if (OP != kOpFindOrInsertPtr && LOCKED_RULE && a.locked_key_ptrs && locked) a.locked_key_ptrs[i] = v.keys + slot;
     if (commit) {
       /* a victim's slot gets a score of this call: what bounds its line now is the lowest of
        * the line's other scores */
       if (BOUNDS && (got == kStEvict || got == kStReclaimed))
         st_u64(v.bounds + (slot >> 4), new_bound < bound_cap ? new_bound : bound_cap);
-      const uint64_t stored = write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate);
+      const uint64_t stored = write_meta(v, a, slot, digest, desired, in_score, i, got != kStDuplicate, hold);
+      if (hold) {
+        /* hybrid mode: the slots of a batch stay LOCKED until all its keys are settled; the
+         * list starts out as all null */
+        a.locked_key_ptrs[i] = v.keys + slot;
+        a.held_scores[i] = stored;
+      }
       /* Scores from the caller may be below what the line's bound says: a key that goes into a
        * free slot, and a key that was found, under Customized (its score becomes the caller's)
        * and under EpochLFU (it moves to the epoch of today, which may be an earlier one than its
@@ -947,7 +964,7 @@ upsert_kernel(View v, UpsertArgs a) {
     wait_stores();
     /* the pointer overload may be asked to leave its slots locked for unlock_keys; the upserts
      * of hybrid mode leave theirs locked until the launch is over */
-    const bool keep_locked = (OP == kOpFindOrInsertPtr || LOCKED_RULE) && a.locked_key_ptrs != nullptr;
+    const bool keep_locked = (OP == kOpFindOrInsertPtr || kCanHold) && a.locked_key_ptrs != nullptr;
     if (locked && !keep_locked) st_unlock(v.keys + slot, commit ? key : victim);
     if (keep_locked) {
       const unsigned long long kept = __ballot(locked);
