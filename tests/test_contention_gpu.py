@@ -154,12 +154,17 @@ def test_row_sizes(strategy, dim):
 @pytest.mark.parametrize("strategy", [EvictStrategy.kLfu, EvictStrategy.kCustomized, EvictStrategy.kLru])
 def test_rows_in_host_memory(strategy):
     """Hybrid mode: a quarter of the rows in HBM; the upserts follow the lock-key kernels' rule
-    (a key whose score equals the bucket's lowest is refused)."""
+    (a key whose score equals the bucket's lowest is refused, and no key takes the slot of
+    another key of its call)."""
     cap, dim = 1 << 12, 8
     t = table(strategy, dim, cap, max_hbm_for_vectors=cap * dim * 4 // 4)
     assert not t.is_pure_hbm()
     ops = [o for o in ALL if o != "insert_and_evict"]  # (pure HBM only, as in the reference)
-    run_calls(t, strategy, dim, 710 + int(strategy), 40, w.unique_keys(711, 0, 3 * cap), [17, 300, 1500],
+    # 4000 keys: more than 128 of a call in some buckets, whose slots are then all held by the call
+    # (insert_or_assign and find_or_insert keep their slots locked to the end of the launch) and
+    # refuse the rest; under LRU every key of a call gets in as long as that does not happen
+    sizes = [17, 300, 1500] if strategy == EvictStrategy.kLru else [17, 300, 1500, 4000]
+    run_calls(t, strategy, dim, 710 + int(strategy), 40, w.unique_keys(711, 0, 3 * cap), sizes,
               ops, [0.45, 0.1, 0.1, 0.08, 0.07, 0.1, 0.1])
     t.close()
 
