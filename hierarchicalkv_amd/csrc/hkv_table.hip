@@ -342,36 +342,36 @@ void launch_main(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t s,
 /* BOUNDS: the victim search reads the bucket's score bounds and one or two of its score lines
  * instead of all eight (hkv_upsert.hpp); for 16-byte units, which is what tables with rows of a
  * multiple of 16 bytes use. */
-template <int OP, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1>
+template <int OP, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1, bool HOLD = false>
 void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
   const dim3 grid(grid_for((a.n + WAVES - 1) / WAVES)), block(kWave * WAVES);
   if constexpr (OP == kOpAccumOrAssign && !BOUNDS) {
     /* the two units that only the element-wise add needs */
     if (vec == 8) {
-      launch_main(upsert_kernel<OP, 8, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
+      launch_main(upsert_kernel<OP, 8, 8, LOCKED_RULE, false, WAVES, HOLD>, grid, block, s, v, a);
       return;
     }
     if (vec == 2) {
-      launch_main(upsert_kernel<OP, 2, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
+      launch_main(upsert_kernel<OP, 2, 8, LOCKED_RULE, false, WAVES, HOLD>, grid, block, s, v, a);
       return;
     }
   }
   if (OP == kOpFindOrInsertPtr) {
-    launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a);
+    launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES, HOLD>, grid, block, s, v, a);
     return;
   }
   if (vec == 16) {
     switch (pick_upl(v.value_bytes, 16)) {
-      case 1: launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
-      case 2: launch_main(upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
-      case 4: launch_main(upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
-      default: launch_main(upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS, WAVES>, grid, block, s, v, a); break;
+      case 1: launch_main(upsert_kernel<OP, 16, 1, LOCKED_RULE, BOUNDS, WAVES, HOLD>, grid, block, s, v, a); break;
+      case 2: launch_main(upsert_kernel<OP, 16, 2, LOCKED_RULE, BOUNDS, WAVES, HOLD>, grid, block, s, v, a); break;
+      case 4: launch_main(upsert_kernel<OP, 16, 4, LOCKED_RULE, BOUNDS, WAVES, HOLD>, grid, block, s, v, a); break;
+      default: launch_main(upsert_kernel<OP, 16, 8, LOCKED_RULE, BOUNDS, WAVES, HOLD>, grid, block, s, v, a); break;
     }
   } else if constexpr (!BOUNDS) {
     if (vec == 4)
-      launch_main(upsert_kernel<OP, 4, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
+      launch_main(upsert_kernel<OP, 4, 8, LOCKED_RULE, false, WAVES, HOLD>, grid, block, s, v, a);
     else
-      launch_main(upsert_kernel<OP, 1, 8, LOCKED_RULE, false, WAVES>, grid, block, s, v, a);
+      launch_main(upsert_kernel<OP, 1, 8, LOCKED_RULE, false, WAVES, HOLD>, grid, block, s, v, a);
   }
 }
 
@@ -379,6 +379,13 @@ void launch_upsert(int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
  * evicted-keys output (hkv_upsert.hpp) */
 template <int OP, bool LOCKED_RULE, bool BOUNDS = false>
 void launch_upsert_for(bool pair, int vec, const View& v, const UpsertArgs& a, hipStream_t s) {
+  if constexpr (OP == kOpInsertOrAssign || OP == kOpFindOrInsert) {
+    /* hybrid mode: the list of slots that stay LOCKED to the end of the launch */
+    if (a.held_scores) {
+      launch_upsert<OP, LOCKED_RULE, BOUNDS, 1, true>(vec, v, a, s);
+      return;
+    }
+  }
   if constexpr (OP == kOpInsertAndEvict) {
     if (pair) {
       launch_upsert<OP, LOCKED_RULE, BOUNDS, 2>(vec, v, a, s);

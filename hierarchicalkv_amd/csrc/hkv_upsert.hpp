@@ -599,12 +599,13 @@ __device__ __forceinline__ void settle_reprobes(const View& v, uint64_t key, uin
  * 15 ns each, and one per wavefront and trip (some 24 thousand for 2^20 keys into full buckets)
  * took 0.07 ms of the call's 0.46.  (While buckets have free slots there is nothing to claim,
  * and two wavefronts that wait for each other in every trip are 4 % slower than one.) */
-template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1>
+template <int OP, int VEC, int UPL, bool LOCKED_RULE, bool BOUNDS = false, int WAVES = 1, bool HOLD = false>
 __global__ void __launch_bounds__(kWave * WAVES)
     __attribute__((amdgpu_waves_per_eu(BOUNDS ? 4 : 1)))
 upsert_kernel(View v, UpsertArgs a) {
   static_assert(!(BOUNDS && LOCKED_RULE), "the bounded search does not look at key words");
   static_assert(WAVES == 1 || OP == kOpInsertAndEvict, "only insert_and_evict has anything to share");
+  static_assert(!HOLD || OP == kOpInsertOrAssign || OP == kOpFindOrInsert, "the calls with a hybrid form");
   __shared__ KeyMeta s_meta_all[WAVES][kWave];
   __shared__ int64_t s_slot_all[WAVES][kWave];
   __shared__ __attribute__((aligned(16))) uint16_t s_em_all[WAVES][kWave][kTile];
@@ -671,15 +672,15 @@ upsert_kernel(View v, UpsertArgs a) {
    * that every one arrives at the workgroup's barriers */
   bool more = pend_mask != 0;
   if constexpr (WAVES > 1) more = __syncthreads_or(more);
-  /* hybrid mode, insert_or_assign and find_or_insert: the slots of a batch stay LOCKED to the end
-   * of the launch (the calls without a hybrid form never see the list) */
-  constexpr bool kCanHold = OP == kOpInsertOrAssign || OP == kOpFindOrInsert;
-  const bool hold = kCanHold && a.locked_key_ptrs != nullptr;
+  /* HOLD: hybrid mode, insert_or_assign and find_or_insert: the slots of a batch stay LOCKED to
+   * the end of the launch (an instantiation of its own: as a run-time switch it cost the kernels
+   * of tables without host rows 3 %) */
+  constexpr bool hold = HOLD;
   /* Where every slot that is taken stays LOCKED to the end of the launch, a LOCKED word is never
    * this key's slot about to be given back: it is another key of the batch, or this key on its
    * way out.  The second probe does not wait for it.  (With the waits, a key whose digest
    * matched a held slot kept its wavefront alive for 64 rounds: 0.15 ms per 2^20 keys.) */
-  if ((OP == kOpFindOrInsertPtr || kCanHold) && a.locked_key_ptrs != nullptr) waited = kMaxLockedWaits;
+  if (HOLD || (OP == kOpFindOrInsertPtr && a.locked_key_ptrs != nullptr)) waited = kMaxLockedWaits;
   for (int trip = 0; more; trip++) {
     if (__ballot(pending && reprobe))
       settle_reprobes(v, key, me.bkt, digest, pending, reprobe, hit, em_lo, em_hi, waited, lane);
@@ -964,7 +965,7 @@ upsert_kernel(View v, UpsertArgs a) {
     wait_stores();
     /* the pointer overload may be asked to leave its slots locked for unlock_keys; the upserts
      * of hybrid mode leave theirs locked until the launch is over */
-    const bool keep_locked = (OP == kOpFindOrInsertPtr || kCanHold) && a.locked_key_ptrs != nullptr;
+    const bool keep_locked = HOLD || (OP == kOpFindOrInsertPtr && a.locked_key_ptrs != nullptr);
     if (locked && !keep_locked) st_unlock(v.keys + slot, commit ? key : victim);
     if (keep_locked) {
       const unsigned long long kept = __ballot(locked);
