@@ -508,7 +508,7 @@ chained_miss_kernel(View v, UpsertArgs a, ChainArgs g) {
   __shared__ uint32_t s_idx[kWave * kChainStage];
   __shared__ uint32_t s_info[kWave * kChainStage]; /* digest | start << 8 */
   __shared__ uint8_t s_count[kWave];
-  __shared__ uint8_t s_list[kWave]; /* lanes (buckets) that have keys in this round */
+  __shared__ uint8_t s_list[kWave]; /* lanes (buckets) that have keys in this pass */
 
   const int lane = threadIdx.x;
   const int tile = lane >> 3, j = lane & (kTile - 1);

@@ -1260,7 +1260,7 @@ def test_accum_flags_that_disagree_in_nearly_full_buckets(oracle, monkeypatch, b
     fill(t, o, 91, 3, 1000, dim)  # old keys: the victims
     pos = 3000
     for rep in range(4):
-        # the latest keys (highest scores: no eviction of this round reaches them)
+        # the latest keys (highest scores: no eviction of this repetition reaches them)
         recent = w.unique_keys(91, pos, 800)
         rv = w.uniform_values(91, pos, 800, dim)
         t.insert_or_assign(800, dev(recent), dev(rv))
