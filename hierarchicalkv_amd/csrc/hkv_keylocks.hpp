@@ -82,7 +82,8 @@ touch_kernel(View v, TouchArgs t) {
   if (KEEP_LOCKED) {
     /* one update of the table's count per wavefront */
     const unsigned long long kept = __ballot(ok);
-    if (kept && lane == (int)__ffsll(kept) - 1) atomicAdd(t.locked_count, (unsigned long long)__popcll(kept));
+    if (kept && lane == (int)__ffsll(kept) - 1)
+      atomicAdd(locked_shard(t.locked_count), (unsigned long long)__popcll(kept));
   }
   if (i >= t.n) return;
   if (t.flags) t.flags[i] = ok;
@@ -107,7 +108,7 @@ unlock_keys_kernel(View v, uint64_t n, uint64_t* const* key_ptrs, const uint64_t
   }
   const unsigned long long freed = __ballot(ok);
   if (locked_count && freed && (threadIdx.x & (kWave - 1)) == (int)__ffsll(freed) - 1)
-    atomicAdd(locked_count, 0ull - (unsigned long long)__popcll(freed)) /* wraps: a subtraction */;
+    atomicAdd(locked_shard(locked_count), 0ull - (unsigned long long)__popcll(freed)) /* wraps: a subtraction */;
   if (i < n && success) success[i] = ok;
 }
 

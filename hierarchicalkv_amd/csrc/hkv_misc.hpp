@@ -181,6 +181,8 @@ load_sample_kernel(View v, uint32_t n, unsigned long long* out) {
 }
 
 __global__ void zero_u64_kernel(unsigned long long* p) { *p = 0; }
+/* the table's count of LOCKED slots, all its words (one thread each) */
+__global__ void zero_locked_kernel(unsigned long long* count) { count[threadIdx.x * kLockedStride] = 0; }
 __global__ void zero_i32_kernel(int32_t* p) { *p = 0; }
 /* n 32-bit words from p on become zero (n a multiple of 4, p aligned to 16 bytes) */
 __global__ void __launch_bounds__(256)

@@ -196,7 +196,7 @@ struct hkv_table {
   unsigned score_floor_turn = 0;
   unsigned long long* d_bound_ceil;  /* device word: no bound of the table is above it (strategies with scores from the caller) */
   unsigned long long* d_load_sample; /* device word: the sum fast_load_factor reads back */
-  unsigned long long* d_locked; /* device word: slots left LOCKED by those calls, less the unlocked */
+  unsigned long long* d_locked; /* device words (kLockedShards of them): slots left LOCKED by those calls, less the unlocked */
   bool dual;               /* TableMode::kMemory: two candidate buckets per key */
   bool io_by_cpu;          /* value rows of the writers are moved by host threads */
   std::mutex io_mutex;     /* one CPU-IO call at a time uses the staging area */
@@ -458,8 +458,9 @@ int noalloc_scratch(int device, uint32_t** out) {
 }
 
 constexpr unsigned kCounterWords = 128;
-/* behind the counters: d_locked, d_bound_caps[2], d_score_floor[2], d_bound_ceil, d_load_sample */
-constexpr unsigned kExtraWords = 7;
+/* behind the counters: d_bound_caps[2], d_score_floor[2], d_bound_ceil, d_load_sample, two spare
+ * words, then d_locked (kLockedShards words, a 128-byte line apart) */
+constexpr unsigned kExtraWords = 8 + kLockedShards * kLockedStride;
 
 /* A device word for a call that returns a count.  The word belongs to the call from the
  * lease to its end (the call zeroes it on its stream, a kernel adds to it, the host reads it
@@ -685,9 +686,12 @@ int grow_for(hkv_table* t, uint64_t n, hipStream_t s) {
  * the table is back to the plain kernels. */
 int settle_locked_count(hkv_table* t, hipStream_t s) {
   if (!t->keys_may_be_locked || !t->locked_recount) return HKV_SUCCESS;
-  long long left = 0;
-  HKV_HIP(hipMemcpyAsync(&left, t->d_locked, sizeof left, hipMemcpyDeviceToHost, s));
+  static_assert(sizeof(long long) == sizeof(unsigned long long), "");
+  std::vector<long long> words(kLockedShards * kLockedStride);
+  HKV_HIP(hipMemcpyAsync(words.data(), t->d_locked, words.size() * sizeof(long long), hipMemcpyDeviceToHost, s));
   HKV_HIP(hipStreamSynchronize(s));
+  long long left = 0; /* a shard may be below zero: keys are unlocked by other workgroups than locked them */
+  for (unsigned k = 0; k < kLockedShards; k++) left += words[k * kLockedStride];
   t->locked_recount = false;
   if (left <= 0) t->keys_may_be_locked = false;
   return HKV_SUCCESS;
@@ -1294,11 +1298,11 @@ int create_impl(const hkv_options* o, const hkv_allocator* al, hkv_table** out) 
   }
   t->d_counters = (unsigned long long*)cnt;
   for (unsigned w = 0; w < kCounterWords; w++) t->counter_free.push_back(w);
-  t->d_locked = t->d_counters + kCounterWords;
-  t->d_bound_caps = t->d_counters + kCounterWords + 1;
-  t->d_score_floor = t->d_counters + kCounterWords + 3;
-  t->d_bound_ceil = t->d_counters + kCounterWords + 5;
-  t->d_load_sample = t->d_counters + kCounterWords + 6;
+  t->d_bound_caps = t->d_counters + kCounterWords;
+  t->d_score_floor = t->d_counters + kCounterWords + 2;
+  t->d_bound_ceil = t->d_counters + kCounterWords + 4;
+  t->d_load_sample = t->d_counters + kCounterWords + 5;
+  t->d_locked = t->d_counters + kCounterWords + 8;
   {
     int rc = sync_clock(t);
     if (rc) return bail(rc);
@@ -1891,7 +1895,7 @@ int hkv_clear(hkv_table* t, hkv_stream_t stream) {
   t->locked_recount = false;
   t->keys_offered = 0;
   t->bounds_stale = true;
-  hipLaunchKernelGGL(zero_u64_kernel, dim3(1), dim3(1), 0, s, t->d_locked);
+  hipLaunchKernelGGL(zero_locked_kernel, dim3(1), dim3(kLockedShards), 0, s, t->d_locked);
   const uint64_t groups = t->view.capacity / 16;
   hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s,
                      t->view, 0);

@@ -973,7 +973,7 @@ upsert_kernel(View v, UpsertArgs a) {
        * at a time, and a wavefront's worth of them per trip is a quarter of a millisecond per
        * 2^20 keys) */
       if (a.locked_count && kept && lane == (int)__ffsll(kept) - 1)
-        atomicAdd(a.locked_count, (unsigned long long)__popcll(kept));
+        atomicAdd(locked_shard(a.locked_count), (unsigned long long)__popcll(kept));
     }
     if (got != kStNone) pending = false;
     pend_mask = __ballot(pending);
