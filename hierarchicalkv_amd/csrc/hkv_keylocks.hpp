@@ -39,9 +39,11 @@ __device__ __forceinline__ uint64_t touch_score(const View& v, const TouchArgs& 
   const uint64_t in_score = t.scores ? t.scores[i] : 0;
   const uint64_t desired = desired_when_missed(a, in_score, i);
   const bool needs_old = t.strategy == HKV_LFU || t.strategy == HKV_EPOCH_LFU;
-  const uint64_t old = ld_u64(v.scores + slot);
+  /* the old score is only read where the new one is made from it (a line of memory traffic
+   * per key otherwise) */
+  const uint64_t old = needs_old ? ld_u64(v.scores + slot) : 0;
   uint64_t snew;
-  if (!final_score(a, false, desired, in_score, needs_old ? old : 0, snew)) return old;
+  if (!final_score(a, false, desired, in_score, old, snew)) return ld_u64(v.scores + slot);
   st_u64(v.scores + slot, snew);
   return snew;
 }
