@@ -169,7 +169,11 @@ int hkv_table_destroy(hkv_table* t);
  * batches leave every key in the table once.  A dual-bucket table needs 1
  * (merlin_hashtable.cuh:1167-1169).
  *
- * HashTable::insert_or_assign, merlin_hashtable.cuh:1125-1305 */
+ * HashTable::insert_or_assign, merlin_hashtable.cuh:1125-1305.  On a table with rows in host
+ * memory and with unique_key = 1 (the reference's lock-key and write kernels, upsert.cuh:1350-1595)
+ * every slot a key of the batch takes stays locked until all keys of the batch are settled: no
+ * key takes the slot of another key of its batch, and a key whose score is not above the lowest
+ * score still visible in its bucket is refused.  find_or_insert with values does the same. */
 int hkv_insert_or_assign(hkv_table* t, uint64_t n, const uint64_t* keys,
                          const void* values, const uint64_t* scores,
                          hkv_stream_t stream, int unique_key,
