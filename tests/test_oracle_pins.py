@@ -253,6 +253,48 @@ def test_refusal_rule_strict_vs_hybrid(oracle):
         t.close()
 
 
+def test_hybrid_batch_holds_every_slot_it_took(oracle):
+    # upsert.cuh:1350-1595 (find_or_insert.cuh:1417-1676): the lock kernel of the hybrid upsert
+    # leaves the slot of every key of the batch LOCKED until the write kernel has run, and its
+    # victim scan passes LOCKED slots over.  Worked by hand for one full bucket whose residents
+    # score 100, 110, ... and the batch 105, 200, 115, 125, 99 in this order:
+    #   105 > 100: takes the slot of 100          200: lowest visible is 110, takes it
+    #   115: lowest visible is 120, refused        125 > 120: takes the slot of 120
+    #   99: lowest visible is 130, refused
+    # One key at a time (each call releases its slot) the same keys end differently:
+    #   105 takes 100's slot, 200 takes 105's, 115 takes 110's, 125 takes 115's, 99 is refused.
+    o = default_options(init_capacity=128, max_capacity=128, dim=1, max_hbm_for_vectors=0,
+                        evict_strategy=EvictStrategy.kCustomized)
+    base = w.unique_keys(1, 0, 128)
+    vals = np.zeros((128, 4), np.uint8)
+    sc = np.arange(100, 100 + 10 * 128, 10, dtype=np.uint64)
+    batch = w.unique_keys(2, 0, 5)
+    bsc = np.array([105, 200, 115, 125, 99], np.uint64)
+
+    def scores_of(t):
+        _, _, s = t.export_all()
+        return sorted(s.tolist())
+
+    t = oracle.OracleTable(o, hybrid=True)
+    t.insert_or_assign(base, vals, sc)
+    t.insert_or_assign(batch, vals[:5], bsc)
+    assert scores_of(t) == sorted([x for x in sc.tolist() if x not in (100, 110, 120)] + [105, 200, 125])
+    assert list(t.contains(batch)) == [True, True, False, True, False]
+    t.close()
+    t = oracle.OracleTable(o, hybrid=True)
+    t.insert_or_assign(base, vals, sc)
+    for i in range(5):
+        t.insert_or_assign(batch[i:i + 1], vals[:1], bsc[i:i + 1])
+    assert scores_of(t) == sorted([x for x in sc.tolist() if x not in (100, 110)] + [200, 125])
+    t.close()
+    # find_or_insert follows the same kernels
+    t = oracle.OracleTable(o, hybrid=True)
+    t.insert_or_assign(base, vals, sc)
+    t.find_or_insert(batch, vals[:5].copy(), bsc)
+    assert scores_of(t) == sorted([x for x in sc.tolist() if x not in (100, 110, 120)] + [105, 200, 125])
+    t.close()
+
+
 # ---- insert_and_evict ------------------------------------------------------------------------
 
 def test_insert_and_evict_conservation(oracle):
